@@ -1,0 +1,224 @@
+"""CPU oracle for the A8W8 FP8 GEMM path -- TEST INFRASTRUCTURE ONLY.
+
+numpy/ctypes front end of ``a8w8_oracle.c`` (a plain-C restatement of the reference's
+host arithmetic).  Only the test suite, the smoke check and the benchmark's CPU-baseline
+leg may import this package; the product library never does.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "liba8w8_oracle.so")
+
+_u8p = ctypes.POINTER(ctypes.c_uint8)
+_f32p = ctypes.POINTER(ctypes.c_float)
+_i32p = ctypes.POINTER(ctypes.c_int)
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+
+
+def build(force=False):
+    """Compile the C restatement with gcc (seconds)."""
+    src = os.path.join(_HERE, "a8w8_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liba8w8_oracle.so"], stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(_SO)
+        L.orc_e4m3_fnuz_decode.restype = ctypes.c_float
+        L.orc_e4m3_fnuz_decode.argtypes = [ctypes.c_uint8]
+        L.orc_e4m3_ocp_decode.restype = ctypes.c_float
+        L.orc_e4m3_ocp_decode.argtypes = [ctypes.c_uint8]
+        L.orc_e8m0_decode.restype = ctypes.c_float
+        L.orc_e8m0_decode.argtypes = [ctypes.c_uint8]
+        L.orc_f8_cast_from_f8_bits.restype = ctypes.c_uint32
+        L.orc_f8_cast_from_f8_bits.argtypes = [ctypes.c_uint8, ctypes.c_int]
+        L.orc_e4m3_ocp_encode.restype = ctypes.c_uint8
+        L.orc_e4m3_ocp_encode.argtypes = [ctypes.c_float]
+        L.orc_e4m3_fnuz_encode.restype = ctypes.c_uint8
+        L.orc_e4m3_fnuz_encode.argtypes = [ctypes.c_float]
+        L.orc_cvt_fp8_clamp240.restype = ctypes.c_uint8
+        L.orc_cvt_fp8_clamp240.argtypes = [ctypes.c_float, ctypes.c_int]
+        L.orc_pk_cvt_fp8x4.restype = ctypes.c_uint32
+        L.orc_pk_cvt_fp8x4.argtypes = [_f32p, ctypes.c_int]
+        L.orc_f32_to_bf16.restype = ctypes.c_uint16
+        L.orc_f32_to_bf16.argtypes = [ctypes.c_float]
+        L.orc_decode_vec.argtypes = [_u8p, _f32p, ctypes.c_size_t, ctypes.c_int]
+        L.orc_encode_vec.argtypes = [_f32p, _u8p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int]
+        L.orc_bf16_vec.argtypes = [_f32p, _u16p, ctypes.c_size_t]
+        L.orc_gemm_ref.argtypes = [_u8p, _u8p, _f32p, _f32p, _f32p] + [ctypes.c_int] * 14
+        L.orc_gemm_ref_mx.argtypes = [_u8p, _u8p, _u8p, _u8p, _f32p] + [ctypes.c_int] * 10
+        L.orc_gemm_probe.argtypes = ([_u8p, _u8p, ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 9
+                                     + [_i32p, _i32p, ctypes.c_int, _f32p])
+        L.orc_preshuffle_index.restype = ctypes.c_size_t
+        L.orc_preshuffle_index.argtypes = [ctypes.c_int] * 3
+        L.orc_preshuffle_b.argtypes = [_u8p, _u8p, ctypes.c_int, ctypes.c_int]
+        L.orc_unshuffle_b.argtypes = [_u8p, _u8p, ctypes.c_int, ctypes.c_int]
+        L.orc_flatmm_ref.argtypes = [_u8p, _u8p, _f32p, _f32p, _f32p] + [ctypes.c_int] * 5
+        L.orc_count_abs_mismatch.restype = ctypes.c_long
+        L.orc_count_abs_mismatch.argtypes = [_f32p, _f32p, ctypes.c_size_t, ctypes.c_float]
+        L.orc_num_threads.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def _p(arr, ty):
+    return arr.ctypes.data_as(ty)
+
+
+def _c(arr, dtype):
+    arr = np.ascontiguousarray(arr, dtype=dtype)
+    return arr
+
+
+OCP, FNUZ = 0, 1
+
+# scale-mode numbers of the library ABI
+TENSOR, ROWCOL, BLOCK, MX = 0, 1, 2, 3
+
+
+def decode(codes, dialect=OCP):
+    codes = _c(codes, np.uint8)
+    out = np.empty(codes.shape, np.float32)
+    lib().orc_decode_vec(_p(codes, _u8p), _p(out, _f32p), codes.size, dialect)
+    return out
+
+
+def encode(x, dialect=OCP, clamp240=False):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint8)
+    lib().orc_encode_vec(_p(x, _f32p), _p(out, _u8p), x.size, dialect, int(clamp240))
+    return out
+
+
+def cast_from_f8_bits(code, negative_zero_nan):
+    return lib().orc_f8_cast_from_f8_bits(int(code), int(negative_zero_nan))
+
+
+def pk_cvt_fp8x4(s4, dialect=OCP):
+    s4 = _c(s4, np.float32)
+    assert s4.size == 4
+    return lib().orc_pk_cvt_fp8x4(_p(s4, _f32p), dialect)
+
+
+def e8m0_decode(b):
+    return lib().orc_e8m0_decode(int(b))
+
+
+def to_bf16_bits(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().orc_bf16_vec(_p(x, _f32p), _p(out, _u16p), x.size)
+    return out
+
+
+def bf16_bits_to_f32(h):
+    return (np.ascontiguousarray(h, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def round_bf16(x):
+    """fp32 -> bf16 (RNE) -> fp32."""
+    return bf16_bits_to_f32(to_bf16_bits(x))
+
+
+def _grouping(mode, m, n, k):
+    """gemm_ref (group_m, group_n, group_k, stride_sfa, stride_sfb) for a scale mode."""
+    if mode == TENSOR:
+        return m, n, k, 0, 0
+    if mode == ROWCOL:
+        return 1, 1, k, 0, 1
+    if mode == BLOCK:
+        return 1, 128, 128, m, k // 128
+    raise ValueError(mode)
+
+
+def gemm_ref(a, b, sfa, sfb, mode, rows=None, decode_per_mac=False):
+    """C[rows] (fp32) of the reference CPU GEMM.  a [M,K] u8, b [N,K] u8."""
+    a = _c(a, np.uint8)
+    b = _c(b, np.uint8)
+    m, k = a.shape
+    n = b.shape[0]
+    r0, r1 = rows if rows is not None else (0, m)
+    c = np.zeros((m, n), np.float32)
+    if mode == MX:
+        sfa = _c(sfa, np.uint8)
+        sfb = _c(sfb, np.uint8)
+        lib().orc_gemm_ref_mx(_p(a, _u8p), _p(b, _u8p), _p(sfa, _u8p), _p(sfb, _u8p), _p(c, _f32p),
+                              m, n, k, k, k, n, sfa.shape[-1], sfb.shape[-1], r0, r1)
+    else:
+        sfa = _c(sfa, np.float32)
+        sfb = _c(sfb, np.float32)
+        gm, gn, gk, ssa, ssb = _grouping(mode, m, n, k)
+        lib().orc_gemm_ref(_p(a, _u8p), _p(b, _u8p), _p(sfa, _f32p), _p(sfb, _f32p), _p(c, _f32p),
+                           m, n, k, k, k, n, ssa, ssb, gm, gn, gk, r0, r1, int(decode_per_mac))
+    return c[r0:r1]
+
+
+def gemm_probe(a, b, sfa, sfb, mode, pi, pj):
+    a = _c(a, np.uint8)
+    b = _c(b, np.uint8)
+    m, k = a.shape
+    n = b.shape[0]
+    pi = _c(pi, np.int32)
+    pj = _c(pj, np.int32)
+    out = np.empty(pi.size, np.float32)
+    if mode == MX:
+        sfa = _c(sfa, np.uint8)
+        sfb = _c(sfb, np.uint8)
+        gm = gn = 1
+        gk = 32
+        ssa, ssb = sfa.shape[-1], sfb.shape[-1]
+    else:
+        sfa = _c(sfa, np.float32)
+        sfb = _c(sfb, np.float32)
+        gm, gn, gk, ssa, ssb = _grouping(mode, m, n, k)
+    lib().orc_gemm_probe(_p(a, _u8p), _p(b, _u8p), sfa.ctypes.data, sfb.ctypes.data, k, k, k, ssa, ssb,
+                         gm, gn, gk, mode, _p(pi, _i32p), _p(pj, _i32p), pi.size, _p(out, _f32p))
+    return out
+
+
+def preshuffle_b(b):
+    b = _c(b, np.uint8)
+    n, k = b.shape
+    out = np.empty(n * k, np.uint8)
+    lib().orc_preshuffle_b(_p(b, _u8p), _p(out, _u8p), n, k)
+    return out
+
+
+def unshuffle_b(bs, n, k):
+    bs = _c(bs, np.uint8)
+    out = np.empty((n, k), np.uint8)
+    lib().orc_unshuffle_b(_p(bs, _u8p), _p(out, _u8p), n, k)
+    return out
+
+
+def flatmm_ref(a, bshuf, sfa, sfb, n):
+    a = _c(a, np.uint8)
+    bshuf = _c(bshuf, np.uint8)
+    sfa = _c(sfa, np.float32)
+    sfb = _c(sfb, np.float32)
+    m, k = a.shape
+    c = np.zeros((m, n), np.float32)
+    lib().orc_flatmm_ref(_p(a, _u8p), _p(bshuf, _u8p), _p(sfa, _f32p), _p(sfb, _f32p), _p(c, _f32p),
+                         m, n, k, k, n)
+    return c
+
+
+def count_abs_mismatch(ref, out, thr=1e-3):
+    ref = _c(ref, np.float32)
+    out = _c(out, np.float32)
+    return lib().orc_count_abs_mismatch(_p(ref, _f32p), _p(out, _f32p), ref.size, thr)
+
+
+def num_threads():
+    return lib().orc_num_threads()
