@@ -1,0 +1,233 @@
+"""ctypes front end of the C ABI declared in include/mi355_a8w8.h.
+
+Argument names and meanings follow struct opus_gemm_kargs of the reference
+(opus_gemm/block_scale_gemm/gemm_a8w8_blockscale_common.h:4-25): element strides, A [M,K]
+and B [N,K] row-major E4M3 bytes, C [M,N].  Tensors are torch tensors used purely as
+device-memory handles (data_ptr) plus the current HIP stream.
+"""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libmi355a8w8.so")
+
+TENSOR, ROWCOL, BLOCK, MX = 0, 1, 2, 3
+BF16, FP32 = 0, 1
+OCP, FNUZ = 0, 1
+
+
+class A8W8Error(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        super().__init__(f"{where}: {status_string(status)} (status {status})")
+
+
+class GemmArgs(ctypes.Structure):
+    _fields_ = [
+        ("a", ctypes.c_void_p), ("b", ctypes.c_void_p), ("c", ctypes.c_void_p),
+        ("m", ctypes.c_int), ("n", ctypes.c_int), ("k", ctypes.c_int), ("batch", ctypes.c_int),
+        ("stride_a", ctypes.c_int), ("stride_b", ctypes.c_int), ("stride_c", ctypes.c_int),
+        ("stride_a_batch", ctypes.c_int), ("stride_b_batch", ctypes.c_int), ("stride_c_batch", ctypes.c_int),
+        ("sfa", ctypes.c_void_p), ("sfb", ctypes.c_void_p),
+        ("stride_sfa", ctypes.c_int), ("stride_sfb", ctypes.c_int),
+        ("stride_sfa_batch", ctypes.c_int), ("stride_sfb_batch", ctypes.c_int),
+        ("scale_mode", ctypes.c_int), ("c_dtype", ctypes.c_int), ("b_preshuffled", ctypes.c_int),
+    ]
+
+
+def library_path():
+    return _SO
+
+
+def build_library(verbose=False):
+    """Compile the HIP sources for gfx950 with hipcc (cross-compiles without a GPU)."""
+    subprocess.check_call(["make", "-C", os.path.join(_HERE, "csrc"), "-B"],
+                          stdout=None if verbose else subprocess.DEVNULL,
+                          stderr=None if verbose else subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    """The loaded C ABI.  Raises if the library has not been built; never substitutes a CPU path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            raise FileNotFoundError(
+                f"{_SO} is missing: build it with gcnasm_amd.build_library() or `make -C gcnasm_amd/csrc`")
+        L = ctypes.CDLL(_SO)
+        vp = ctypes.c_void_p
+        L.a8w8_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.a8w8_gemm_blockscale.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.a8w8_flatmm.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.a8w8_preshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
+        L.a8w8_unshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
+        L.a8w8_preshuffle_b_device.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, vp]
+        L.a8w8_cvt_f32_to_e4m3.restype = ctypes.c_size_t
+        L.a8w8_cvt_f32_to_e4m3.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, vp]
+        L.a8w8_cvt_e4m3_to_f32.restype = ctypes.c_size_t
+        L.a8w8_cvt_e4m3_to_f32.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, vp]
+        L.a8w8_quantize.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_int,
+                                    ctypes.c_int, vp]
+        L.a8w8_status_string.restype = ctypes.c_char_p
+        L.a8w8_status_string.argtypes = [ctypes.c_int]
+        L.a8w8_kernel_name.restype = ctypes.c_char_p
+        L.a8w8_kernel_name.argtypes = [ctypes.POINTER(GemmArgs)]
+        L.a8w8_version.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def status_string(status):
+    return lib().a8w8_status_string(int(status)).decode()
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(status, where):
+    if status != 0:
+        raise A8W8Error(status, where)
+
+
+def raw_gemm_args(a, b, c, sfa, sfb, m, n, k, scale_mode, c_dtype=BF16, batch=1, stride_a=None, stride_b=None,
+                  stride_c=None, stride_sfa=None, stride_sfb=None, b_preshuffled=0, batch_strides=None):
+    """Fill the C argument block from raw integers (device addresses)."""
+    g = GemmArgs()
+    g.a, g.b, g.c, g.sfa, g.sfb = a, b, c, sfa, sfb
+    g.m, g.n, g.k, g.batch = m, n, k, batch
+    g.stride_a = k if stride_a is None else stride_a
+    g.stride_b = k if stride_b is None else stride_b
+    g.stride_c = n if stride_c is None else stride_c
+    if stride_sfa is None:
+        stride_sfa = {TENSOR: 0, ROWCOL: 0, BLOCK: m, MX: k // 32}[scale_mode] if 0 <= scale_mode <= 3 else 0
+    if stride_sfb is None:
+        stride_sfb = {TENSOR: 0, ROWCOL: 1, BLOCK: k // 128, MX: k // 32}[scale_mode] if 0 <= scale_mode <= 3 else 0
+    g.stride_sfa, g.stride_sfb = stride_sfa, stride_sfb
+    if batch_strides is None:
+        sfa_b = {TENSOR: 1, ROWCOL: m, BLOCK: m * (k // 128), MX: m * (k // 32)}.get(scale_mode, 0)
+        sfb_b = {TENSOR: 1, ROWCOL: n, BLOCK: (n // 128) * (k // 128), MX: n * (k // 32)}.get(scale_mode, 0)
+        batch_strides = (m * g.stride_a, n * g.stride_b, m * g.stride_c, sfa_b, sfb_b)
+    (g.stride_a_batch, g.stride_b_batch, g.stride_c_batch, g.stride_sfa_batch, g.stride_sfb_batch) = batch_strides
+    g.scale_mode, g.c_dtype, g.b_preshuffled = scale_mode, c_dtype, b_preshuffled
+    return g
+
+
+def _out(c, shape, c_dtype, device):
+    import torch
+    if c is None:
+        c = torch.empty(shape, dtype=torch.bfloat16 if c_dtype == BF16 else torch.float32, device=device)
+    return c
+
+
+def _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, b_preshuffled, n=None):
+    batch = a.shape[0] if a.dim() == 3 else 1
+    m, k = a.shape[-2], a.shape[-1]
+    if n is None:
+        n = b.shape[-2]
+    shape = (batch, m, n) if a.dim() == 3 else (m, n)
+    c = _out(c, shape, c_dtype, a.device)
+    g = raw_gemm_args(a.data_ptr(), b.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, scale_mode,
+                      c_dtype, batch, stride_a=a.stride(-2), stride_b=(k if b_preshuffled else b.stride(-2)),
+                      stride_c=c.stride(-2), b_preshuffled=b_preshuffled)
+    if a.dim() == 3:
+        g.stride_a_batch, g.stride_c_batch = a.stride(0), c.stride(0)
+        g.stride_b_batch = b.stride(0) if b.dim() >= 2 and not b_preshuffled else n * k
+    return g, c
+
+
+def gemm(a, b, sfa, sfb, scale_mode, c=None, c_dtype=BF16):
+    """C = dequant(A) @ dequant(B)^T through a8w8_gemm.  a [.., M, K] u8, b [.., N, K] u8 on the GPU."""
+    g, c = _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, 0)
+    _check(lib().a8w8_gemm(ctypes.byref(g), _stream()), "a8w8_gemm")
+    return c
+
+
+def gemm_blockscale(a, b, sfa, sfb, c=None, c_dtype=FP32):
+    """The reference's block-scale GEMM (1x128 / 128x128 scales), fp32 C by default as there."""
+    g, c = _args_from_tensors(a, b, sfa, sfb, BLOCK, c, c_dtype, 0)
+    _check(lib().a8w8_gemm_blockscale(ctypes.byref(g), _stream()), "a8w8_gemm_blockscale")
+    return c
+
+
+def flatmm(a, b_shuffled, sfa, sfb, n, scale_mode=ROWCOL, c=None, c_dtype=BF16):
+    """Skinny-M GEMM over weights in the a8w8_preshuffle_b layout (flat u8 tensor of n*k bytes)."""
+    g, c = _args_from_tensors(a, b_shuffled, sfa, sfb, scale_mode, c, c_dtype, 1, n=n)
+    _check(lib().a8w8_flatmm(ctypes.byref(g), _stream()), "a8w8_flatmm")
+    return c
+
+
+def preshuffle_b(b_np):
+    """Host pre-shuffle of a numpy [N, K] uint8 weight; returns a flat uint8 array."""
+    import numpy as np
+    b_np = np.ascontiguousarray(b_np, dtype=np.uint8)
+    n, k = b_np.shape
+    out = np.empty(n * k, np.uint8)
+    _check(lib().a8w8_preshuffle_b(b_np.ctypes.data, out.ctypes.data, n, k), "a8w8_preshuffle_b")
+    return out
+
+
+def unshuffle_b(bs_np, n, k):
+    import numpy as np
+    bs_np = np.ascontiguousarray(bs_np, dtype=np.uint8)
+    out = np.empty((n, k), np.uint8)
+    _check(lib().a8w8_unshuffle_b(bs_np.ctypes.data, out.ctypes.data, n, k), "a8w8_unshuffle_b")
+    return out
+
+
+def preshuffle_b_device(b):
+    import torch
+    n, k = b.shape
+    out = torch.empty(n * k, dtype=torch.uint8, device=b.device)
+    _check(lib().a8w8_preshuffle_b_device(b.data_ptr(), out.data_ptr(), n, k, _stream()), "a8w8_preshuffle_b_device")
+    return out
+
+
+def cvt_f32_to_e4m3(x, dialect=OCP, clamp240=False):
+    import torch
+    x = x.contiguous()
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    done = lib().a8w8_cvt_f32_to_e4m3(x.data_ptr(), out.data_ptr(), x.numel(), dialect, int(clamp240), _stream())
+    if done != x.numel():
+        raise A8W8Error(-6, "a8w8_cvt_f32_to_e4m3")
+    return out
+
+
+def cvt_e4m3_to_f32(codes, dialect=OCP):
+    import torch
+    codes = codes.contiguous()
+    out = torch.empty(codes.shape, dtype=torch.float32, device=codes.device)
+    done = lib().a8w8_cvt_e4m3_to_f32(codes.data_ptr(), out.data_ptr(), codes.numel(), dialect, _stream())
+    if done != codes.numel():
+        raise A8W8Error(-6, "a8w8_cvt_e4m3_to_f32")
+    return out
+
+
+def quantize(x, scale_mode, group_rows=1):
+    """fp32 [rows, K] -> (E4M3 bytes [rows, K], scales in the layout a8w8_gemm reads)."""
+    import torch
+    rows, k = x.shape
+    q = torch.empty((rows, k), dtype=torch.uint8, device=x.device)
+    if scale_mode == ROWCOL:
+        s = torch.empty(rows, dtype=torch.float32, device=x.device)
+    elif scale_mode == BLOCK and group_rows == 1:
+        s = torch.empty((k // 128, rows), dtype=torch.float32, device=x.device)
+    elif scale_mode == BLOCK:
+        s = torch.empty((rows // 128, k // 128), dtype=torch.float32, device=x.device)
+    elif scale_mode == MX:
+        s = torch.empty((rows, k // 32), dtype=torch.uint8, device=x.device)
+    else:
+        raise A8W8Error(-6, "a8w8_quantize")
+    _check(lib().a8w8_quantize(x.data_ptr(), rows, k, x.stride(0), q.data_ptr(), s.data_ptr(), scale_mode, group_rows,
+                               _stream()), "a8w8_quantize")
+    return q, s
+
+
+def kernel_name(g):
+    r = lib().a8w8_kernel_name(ctypes.byref(g))
+    return r.decode() if r else None

@@ -1,0 +1,343 @@
+// C ABI of libmi355a8w8: argument validation, kernel selection, launches.
+#include "../../include/mi355_a8w8.h"
+
+#include <hip/hip_runtime.h>
+#include <string.h>
+
+#include "cvt.hpp"
+#include "flatmm.hpp"
+#include "gemm_general.hpp"
+#include "gemm_tile.hpp"
+
+using namespace a8w8;
+
+namespace {
+
+bool device_is_gfx950()
+{
+    static int cached[64];   // 0 unknown, 1 yes, -1 no
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    if (cached[dev] == 0) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return false;
+        cached[dev] = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
+    }
+    return cached[dev] == 1;
+}
+
+int launch_status()
+{
+    return hipGetLastError() == hipSuccess ? A8W8_OK : A8W8_ERR_LAUNCH;
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// Checks shared by every GEMM entry point (mirrors the reference harness's rejects,
+// gemm_a8w8_blockscale_host.cc:175-187, and adds the pointer/stride checks a library needs).
+int validate_common(const a8w8_gemm_args* g)
+{
+    if (!g) return A8W8_ERR_NULL_POINTER;
+    if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
+    if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (g->scale_mode < 0 || g->scale_mode > 3) return A8W8_ERR_BAD_MODE;
+    if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
+    if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128 && (g->n % 128 != 0 || g->k % 128 != 0))
+        return A8W8_ERR_BAD_GROUP;
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_1x32 && g->k % 32 != 0) return A8W8_ERR_BAD_GROUP;
+    if (g->stride_c < g->n) return A8W8_ERR_BAD_STRIDE;
+    if (g->stride_a < g->k) return A8W8_ERR_BAD_STRIDE;
+    if (!g->b_preshuffled && g->stride_b < g->k) return A8W8_ERR_BAD_STRIDE;
+    if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128 && (g->stride_sfa < g->m || g->stride_sfb < g->k / 128))
+        return A8W8_ERR_BAD_STRIDE;
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_1x32 && (g->stride_sfa < g->k / 32 || g->stride_sfb < g->k / 32))
+        return A8W8_ERR_BAD_STRIDE;
+    if (g->batch > 1 && (g->stride_a_batch < 0 || g->stride_b_batch < 0 || g->stride_c_batch < 0 ||
+                         g->stride_sfa_batch < 0 || g->stride_sfb_batch < 0))
+        return A8W8_ERR_BAD_STRIDE;
+    // the kernels address one batch of A / B with 32-bit byte offsets
+    const long long a_span = (long long)(g->m - 1) * g->stride_a + g->k;
+    const long long b_span = g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k;
+    if (a_span >= (1ll << 31) || b_span >= (1ll << 31)) return A8W8_ERR_TOO_LARGE;
+    if (g->batch > 65535) return A8W8_ERR_TOO_LARGE;
+    return A8W8_OK;
+}
+
+GemmParams make_params(const a8w8_gemm_args* g)
+{
+    GemmParams p;
+    p.a = (const uint8_t*)g->a;
+    p.b = (const uint8_t*)g->b;
+    p.c = g->c;
+    p.sfa = g->sfa;
+    p.sfb = g->sfb;
+    p.m = g->m; p.n = g->n; p.k = g->k;
+    p.lda = g->stride_a; p.ldb = g->stride_b; p.ldc = g->stride_c;
+    p.a_batch = g->stride_a_batch; p.b_batch = g->stride_b_batch; p.c_batch = g->stride_c_batch;
+    p.sfa_batch = g->stride_sfa_batch; p.sfb_batch = g->stride_sfb_batch;
+    p.stride_sfa = g->stride_sfa; p.stride_sfb = g->stride_sfb;
+    p.tiles_m = (g->m + BM - 1) / BM;
+    p.tiles_n = (g->n + BN - 1) / BN;
+    return p;
+}
+
+// The tiled kernels need whole 128-wide K steps and 16-byte aligned rows in A and B.
+bool tiled_ok(const a8w8_gemm_args* g)
+{
+    return g->k % BK == 0 && g->stride_a % 16 == 0 && g->stride_b % 16 == 0 && aligned16(g->a) && aligned16(g->b) &&
+           (g->batch == 1 || (g->stride_a_batch % 16 == 0 && g->stride_b_batch % 16 == 0)) &&
+           (long long)((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 31);
+}
+
+template <int MODE, int CDT>
+int launch_tiled(const GemmParams& p, int batch, hipStream_t stream)
+{
+    static bool attr_set[64];
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    auto kern = gemm_a8w8_tile256<MODE, CDT>;
+    if (!attr_set[dev & 63]) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES) !=
+            hipSuccess)
+            return A8W8_ERR_LAUNCH;
+        attr_set[dev & 63] = true;
+    }
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch);
+    hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), GEMM_LDS_BYTES, stream, p);
+    return launch_status();
+}
+
+template <int MODE, int CDT>
+int launch_general(const GemmParams& p, int batch, hipStream_t stream)
+{
+    dim3 grid((unsigned)((p.n + 15) / 16), (unsigned)((p.m + 15) / 16), (unsigned)batch);
+    hipLaunchKernelGGL((gemm_a8w8_general<MODE, CDT>), grid, dim3(256), 0, stream, p);
+    return launch_status();
+}
+
+
+#define A8W8_DISPATCH(FN, mode, cdt, ...)                                                   \
+    switch ((mode) * 2 + (cdt)) {                                                           \
+        case 0: return FN<MODE_TENSOR, C_BF16>(__VA_ARGS__);                                \
+        case 1: return FN<MODE_TENSOR, C_FP32>(__VA_ARGS__);                                \
+        case 2: return FN<MODE_ROWCOL, C_BF16>(__VA_ARGS__);                                \
+        case 3: return FN<MODE_ROWCOL, C_FP32>(__VA_ARGS__);                                \
+        case 4: return FN<MODE_BLOCK, C_BF16>(__VA_ARGS__);                                 \
+        case 5: return FN<MODE_BLOCK, C_FP32>(__VA_ARGS__);                                 \
+        case 6: return FN<MODE_MX, C_BF16>(__VA_ARGS__);                                    \
+        case 7: return FN<MODE_MX, C_FP32>(__VA_ARGS__);                                    \
+        default: return A8W8_ERR_BAD_MODE;                                                  \
+    }
+
+int dispatch_tiled(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
+{
+    A8W8_DISPATCH(launch_tiled, g->scale_mode, g->c_dtype, p, g->batch, s)
+}
+int dispatch_general(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
+{
+    A8W8_DISPATCH(launch_general, g->scale_mode, g->c_dtype, p, g->batch, s)
+}
+
+int validate_flat(const a8w8_gemm_args* g)
+{
+    if (!g) return A8W8_ERR_NULL_POINTER;
+    if (!g->b_preshuffled) return A8W8_ERR_BAD_MODE;
+    if (g->scale_mode != A8W8_SCALE_ROWCOL && g->scale_mode != A8W8_SCALE_TENSOR) return A8W8_ERR_BAD_MODE;
+    const int st = validate_common(g);
+    if (st != A8W8_OK) return st;
+    if (g->m > 64) return A8W8_ERR_BAD_SHAPE;
+    if (g->n % 16 != 0 || g->k % 64 != 0) return A8W8_ERR_BAD_GROUP;
+    if (!aligned16(g->a) || !aligned16(g->b) || g->stride_a % 16 != 0) return A8W8_ERR_MISALIGNED;
+    if (g->batch > 1 && (g->stride_a_batch % 16 != 0 || g->stride_b_batch % 16 != 0)) return A8W8_ERR_MISALIGNED;
+    return A8W8_OK;
+}
+
+constexpr int FLAT_NT = 2;
+
+template <int CDT, int MODE>
+int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
+{
+    const int n_tiles = p.n / 16;
+    dim3 grid((unsigned)((n_tiles + FLAT_NT - 1) / FLAT_NT), (unsigned)((p.m + 15) / 16), (unsigned)batch);
+    hipLaunchKernelGGL((flatmm_a8w8<FLAT_NT, CDT, MODE>), grid, dim3(FLAT_THREADS), 0, stream, p);
+    return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+int a8w8_gemm(const a8w8_gemm_args* g, void* hip_stream)
+{
+    const int st = validate_common(g);
+    if (st != A8W8_OK) return st;
+    if (g->b_preshuffled) return A8W8_ERR_BAD_MODE;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    const GemmParams p = make_params(g);
+    hipStream_t s = (hipStream_t)hip_stream;
+    return tiled_ok(g) ? dispatch_tiled(g, p, s) : dispatch_general(g, p, s);
+}
+
+int a8w8_gemm_blockscale(const a8w8_gemm_args* g, void* hip_stream)
+{
+    if (!g) return A8W8_ERR_NULL_POINTER;
+    a8w8_gemm_args local = *g;
+    local.scale_mode = A8W8_SCALE_BLOCK_1x128_128x128;
+    local.b_preshuffled = 0;
+    return a8w8_gemm(&local, hip_stream);
+}
+
+int a8w8_flatmm(const a8w8_gemm_args* g, void* hip_stream)
+{
+    const int st = validate_flat(g);
+    if (st != A8W8_OK) return st;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    const GemmParams p = make_params(g);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const bool tensor = g->scale_mode == A8W8_SCALE_TENSOR;
+    if (g->c_dtype == A8W8_C_BF16)
+        return tensor ? launch_flat<C_BF16, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_BF16, MODE_ROWCOL>(p, g->batch, s);
+    return tensor ? launch_flat<C_FP32, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_FP32, MODE_ROWCOL>(p, g->batch, s);
+}
+
+static size_t shuffled_index(int j, int p, int k)
+{
+    return (((size_t)(j / 16) * (k / 64) + p / 64) * 4 + (p % 64) / 16) * 256 + (size_t)(j % 16) * 16 + p % 16;
+}
+
+int a8w8_preshuffle_b(const void* b_host, void* out_host, int n, int k)
+{
+    if (!b_host || !out_host) return A8W8_ERR_NULL_POINTER;
+    if (n <= 0 || k <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (n % 16 != 0 || k % 64 != 0) return A8W8_ERR_BAD_GROUP;
+    const uint8_t* b = (const uint8_t*)b_host;
+    uint8_t* o = (uint8_t*)out_host;
+    for (int j = 0; j < n; ++j)
+        for (int p = 0; p < k; p += 16) memcpy(o + shuffled_index(j, p, k), b + (size_t)j * k + p, 16);
+    return A8W8_OK;
+}
+
+int a8w8_unshuffle_b(const void* bshuf_host, void* out_host, int n, int k)
+{
+    if (!bshuf_host || !out_host) return A8W8_ERR_NULL_POINTER;
+    if (n <= 0 || k <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (n % 16 != 0 || k % 64 != 0) return A8W8_ERR_BAD_GROUP;
+    const uint8_t* s = (const uint8_t*)bshuf_host;
+    uint8_t* o = (uint8_t*)out_host;
+    for (int j = 0; j < n; ++j)
+        for (int p = 0; p < k; p += 16) memcpy(o + (size_t)j * k + p, s + shuffled_index(j, p, k), 16);
+    return A8W8_OK;
+}
+
+int a8w8_preshuffle_b_device(const void* b_dev, void* out_dev, int n, int k, void* hip_stream)
+{
+    if (!b_dev || !out_dev) return A8W8_ERR_NULL_POINTER;
+    if (n <= 0 || k <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (n % 16 != 0 || k % 64 != 0) return A8W8_ERR_BAD_GROUP;
+    if (!aligned16(out_dev)) return A8W8_ERR_MISALIGNED;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    const long long units = (long long)n * k / 16;
+    hipLaunchKernelGGL(preshuffle_b_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)hip_stream, (const uint8_t*)b_dev, (uint8_t*)out_dev, n, k);
+    return launch_status();
+}
+
+size_t a8w8_cvt_f32_to_e4m3(const float* src, uint8_t* dst, size_t n, int dialect, int clamp240, void* hip_stream)
+{
+    if (!src || !dst || n == 0) return 0;
+    if (dialect != A8W8_E4M3_OCP && dialect != A8W8_E4M3_FNUZ) return 0;
+    if (!device_is_gfx950()) return 0;
+    hipStream_t s = (hipStream_t)hip_stream;
+    const dim3 grid((unsigned)(((n + 3) / 4 + 255) / 256)), block(256);
+    if (dialect == A8W8_E4M3_OCP) {
+        if (clamp240) hipLaunchKernelGGL((cvt_f32_to_e4m3_kernel<0, 1>), grid, block, 0, s, src, dst, n);
+        else hipLaunchKernelGGL((cvt_f32_to_e4m3_kernel<0, 0>), grid, block, 0, s, src, dst, n);
+    } else {
+        if (clamp240) hipLaunchKernelGGL((cvt_f32_to_e4m3_kernel<1, 1>), grid, block, 0, s, src, dst, n);
+        else hipLaunchKernelGGL((cvt_f32_to_e4m3_kernel<1, 0>), grid, block, 0, s, src, dst, n);
+    }
+    return launch_status() == A8W8_OK ? n : 0;
+}
+
+size_t a8w8_cvt_e4m3_to_f32(const uint8_t* src, float* dst, size_t n, int dialect, void* hip_stream)
+{
+    if (!src || !dst || n == 0) return 0;
+    if (dialect != A8W8_E4M3_OCP && dialect != A8W8_E4M3_FNUZ) return 0;
+    if (!device_is_gfx950()) return 0;
+    hipStream_t s = (hipStream_t)hip_stream;
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (dialect == A8W8_E4M3_OCP) hipLaunchKernelGGL((cvt_e4m3_to_f32_kernel<0>), grid, block, 0, s, src, dst, n);
+    else hipLaunchKernelGGL((cvt_e4m3_to_f32_kernel<1>), grid, block, 0, s, src, dst, n);
+    return launch_status() == A8W8_OK ? n : 0;
+}
+
+int a8w8_quantize(const float* src, int rows, int k, int ld, uint8_t* q, void* scale, int scale_mode, int group_rows,
+                  void* hip_stream)
+{
+    if (!src || !q || !scale) return A8W8_ERR_NULL_POINTER;
+    if (rows <= 0 || k <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (ld < k) return A8W8_ERR_BAD_STRIDE;
+    hipStream_t s = (hipStream_t)hip_stream;
+    switch (scale_mode) {
+        case A8W8_SCALE_ROWCOL:
+            if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+            hipLaunchKernelGGL(quant_rowwise_kernel, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
+            return launch_status();
+        case A8W8_SCALE_BLOCK_1x128_128x128:
+            if (k % 128 != 0) return A8W8_ERR_BAD_GROUP;
+            if (group_rows == 1) {
+                if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+                const long long waves = (long long)rows * (k / 128);
+                hipLaunchKernelGGL(quant_1x128_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, src, rows, k,
+                                   ld, q, (float*)scale);
+                return launch_status();
+            }
+            if (group_rows == 128) {
+                if (rows % 128 != 0) return A8W8_ERR_BAD_GROUP;
+                if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+                hipLaunchKernelGGL(quant_128x128_kernel, dim3((unsigned)(k / 128), (unsigned)(rows / 128)), dim3(256), 0,
+                                   s, src, k, ld, q, (float*)scale);
+                return launch_status();
+            }
+            return A8W8_ERR_BAD_MODE;
+        case A8W8_SCALE_MX_E8M0_1x32: {
+            if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
+            if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+            const long long threads = (long long)rows * k;
+            hipLaunchKernelGGL(quant_mx_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k,
+                               ld, q, (uint8_t*)scale);
+            return launch_status();
+        }
+        default:
+            return A8W8_ERR_BAD_MODE;
+    }
+}
+
+const char* a8w8_status_string(int status)
+{
+    switch (status) {
+        case A8W8_OK: return "ok";
+        case A8W8_ERR_NULL_POINTER: return "null pointer";
+        case A8W8_ERR_BAD_SHAPE: return "m, n, k and batch must be positive (and m <= 64 for flatmm)";
+        case A8W8_ERR_BAD_GROUP: return "m/n/k must be multiples of the scale group (or of the shuffle tile)";
+        case A8W8_ERR_BAD_STRIDE: return "a stride is smaller than the extent it spans";
+        case A8W8_ERR_MISALIGNED: return "pointer or stride not 16-byte aligned";
+        case A8W8_ERR_BAD_MODE: return "unsupported scale mode, output type or layout flag";
+        case A8W8_ERR_TOO_LARGE: return "matrix too large for 32-bit offsets";
+        case A8W8_ERR_LAUNCH: return "kernel launch failed";
+        case A8W8_ERR_NO_DEVICE: return "current device is not gfx950";
+        default: return "unknown status";
+    }
+}
+
+const char* a8w8_kernel_name(const a8w8_gemm_args* g)
+{
+    if (!g) return nullptr;
+    if (g->b_preshuffled) return validate_flat(g) == A8W8_OK ? "flatmm_a8w8" : nullptr;
+    if (validate_common(g) != A8W8_OK) return nullptr;
+    return tiled_ok(g) ? "gemm_a8w8_tile256" : "gemm_a8w8_general";
+}
+
+int a8w8_version(void) { return 100; }
+
+}  // extern "C"

@@ -1,0 +1,57 @@
+// Device-side building blocks shared by the gfx950 A8W8 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace a8w8 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned short v4u16 __attribute__((ext_vector_type(4)));
+
+#define A8W8_DEV __device__ __forceinline__
+#define A8W8_LDS __attribute__((address_space(3)))
+
+enum : int { MODE_TENSOR = 0, MODE_ROWCOL = 1, MODE_BLOCK = 2, MODE_MX = 3 };
+enum : int { C_BF16 = 0, C_FP32 = 1 };
+
+// Kernel parameters of the dense and flat GEMMs (strides in elements, as in the ABI).
+struct GemmParams {
+    const uint8_t* a;
+    const uint8_t* b;
+    void* c;
+    const void* sfa;
+    const void* sfb;
+    int m, n, k;
+    int lda, ldb, ldc;
+    long long a_batch, b_batch, c_batch, sfa_batch, sfb_batch;
+    int stride_sfa, stride_sfb;
+    int tiles_m, tiles_n;
+};
+
+// Raw buffer descriptor over [base, base + bytes): dword 3 = 0x00020000 selects the raw
+// 32-bit data format used for untyped loads on gfx9-family hardware.
+A8W8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+// 16 bytes per lane straight from global memory into LDS.  The hardware places lane i's
+// data at lds_base + 16*i, so lds_base must be wave-uniform.
+A8W8_DEV void load_to_lds_16(__amdgpu_buffer_rsrc_t rsrc, A8W8_LDS void* lds_base, int voffset, int soffset)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds_base, 16, voffset, soffset, 0, 0);
+}
+
+A8W8_DEV int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// fp32 -> bf16 bits, round to nearest even, through the hardware convert.
+A8W8_DEV unsigned short bf16_bits(float f)
+{
+    __bf16 h = (__bf16)f;
+    return __builtin_bit_cast(unsigned short, h);
+}
+
+}  // namespace a8w8

@@ -1,0 +1,220 @@
+// fp8 <-> fp32 conversion helpers, weight pre-shuffle and the quantisation front end (gfx950).
+#pragma once
+#include "a8w8_device.hpp"
+
+namespace a8w8 {
+
+// ---------------------------------------------------------------- software E4M3 FNUZ
+// The gfx942 dialect (bias 8, max 240, 0x80 = NaN, no -0) is not what gfx950 hardware
+// converts to, so it is computed with integer arithmetic on the fp32 bit pattern.
+A8W8_DEV uint8_t f32_to_e4m3_fnuz_sw(float x)
+{
+    const uint32_t u = __builtin_bit_cast(uint32_t, x);
+    const uint32_t sign = (u >> 31) << 7;
+    const uint32_t au = u & 0x7fffffffu;
+    if (au >= 0x7f800000u) return 0x80;                 // NaN and Inf have one code
+    if (au > 0x43700000u) return (uint8_t)(sign | 0x7f); // beyond 240: largest finite
+    const int e8 = (int)(au >> 23) - 127 + 8;           // exponent field in the fp8 format
+    uint32_t mant = au & 0x7fffffu;
+    uint32_t code, rem, half;
+    if (e8 >= 1) {
+        code = ((uint32_t)e8 << 3) | (mant >> 20);
+        rem = mant & 0xfffffu;
+        half = 0x80000u;
+    } else {
+        const int sh = 21 - e8;                          // 20 dropped bits + (1 - e8)
+        if (sh > 25) return 0;                           // below half of the smallest subnormal
+        mant |= 0x800000u;
+        code = mant >> sh;
+        rem = mant & ((1u << sh) - 1u);
+        half = 1u << (sh - 1);
+    }
+    if (rem > half || (rem == half && (code & 1u))) ++code;   // nearest, ties to even
+    if (code > 0x7fu) code = 0x7fu;
+    if (code == 0) return 0;
+    return (uint8_t)(sign | code);
+}
+
+A8W8_DEV float e4m3_fnuz_to_f32_sw(uint8_t c)
+{
+    if (c == 0) return 0.f;
+    if (c == 0x80) return __builtin_bit_cast(float, 0x7F800001u);
+    uint32_t sign = (uint32_t)(c >> 7) << 31;
+    int e = (c >> 3) & 15;
+    uint32_t m = c & 7;
+    if (e == 0) {                       // subnormal: shift the leading one into place
+        const int lz = __builtin_clz(m) - 29;   // 0 for m>=4, 1 for m>=2, 2 for m==1
+        m = (m << (lz + 1)) & 7;
+        e = -lz;
+    }
+    return __builtin_bit_cast(float, sign | ((uint32_t)(e + 127 - 8) << 23) | (m << 20));
+}
+
+// to_fp8_raw_from_fp32 of the reference (cvt_fp8/test.cpp:21-43) on this hardware.
+A8W8_DEV float clamp240_unless_special(float v)
+{
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    if ((u & 0x7F800000u) != 0x7F800000u) v = __builtin_amdgcn_fmed3f(v, 240.0f, -240.0f);
+    return v;
+}
+
+// One thread converts four consecutive floats into one packed word:
+// two packed hardware converts into the low halves, merged by a byte permute
+// (the sequence of pk_cvt_fp8x4_fp32x4_rne, pk_cvt/test.cpp:220-257).
+template <int DIALECT, int CLAMP>
+__global__ void __launch_bounds__(256) cvt_f32_to_e4m3_kernel(const float* src, uint8_t* dst, size_t n)
+{
+    const size_t q = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t i0 = q * 4;
+    if (i0 >= n) return;
+    float s[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        s[e] = i0 + e < n ? src[i0 + e] : 0.f;
+        if (CLAMP) s[e] = clamp240_unless_special(s[e]);
+    }
+    uint32_t word;
+    if (DIALECT == 0) {
+        const uint32_t x = __builtin_amdgcn_cvt_pk_fp8_f32(s[0], s[1], 0, false);
+        const uint32_t y = __builtin_amdgcn_cvt_pk_fp8_f32(s[2], s[3], 0, false);
+        word = __builtin_amdgcn_perm(y, x, 0x05040100);
+    } else {
+        word = (uint32_t)f32_to_e4m3_fnuz_sw(s[0]) | ((uint32_t)f32_to_e4m3_fnuz_sw(s[1]) << 8) |
+               ((uint32_t)f32_to_e4m3_fnuz_sw(s[2]) << 16) | ((uint32_t)f32_to_e4m3_fnuz_sw(s[3]) << 24);
+    }
+    if (i0 + 3 < n && ((uintptr_t)dst & 3) == 0) {
+        *(uint32_t*)(dst + i0) = word;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (i0 + e < n) dst[i0 + e] = (uint8_t)(word >> (8 * e));
+    }
+}
+
+template <int DIALECT>
+__global__ void __launch_bounds__(256) cvt_e4m3_to_f32_kernel(const uint8_t* src, float* dst, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const uint8_t c = src[i];
+    dst[i] = DIALECT == 0 ? __builtin_amdgcn_cvt_f32_fp8((int)c, 0) : e4m3_fnuz_to_f32_sw(c);
+}
+
+// Row-major B[n][k] -> Bshuf[n/16][k/64][4][16][16 B]; one thread moves 16 bytes.
+__global__ void __launch_bounds__(256) preshuffle_b_kernel(const uint8_t* b, uint8_t* out, int n, int k)
+{
+    const long long o = (long long)blockIdx.x * 256 + threadIdx.x;   // 16-byte unit in the output
+    const long long total = (long long)n * k / 16;
+    if (o >= total) return;
+    const int r = (int)(o & 15);
+    const int kq = (int)((o >> 4) & 3);
+    const long long blk = o >> 6;
+    const int k_tiles = k >> 6;
+    const int kt = (int)(blk % k_tiles);
+    const int nt = (int)(blk / k_tiles);
+    const uint8_t* src = b + (long long)(nt * 16 + r) * k + kt * 64 + kq * 16;
+    v4i v;
+    if (((uintptr_t)src & 15) == 0) v = *(const v4i*)src;
+    else __builtin_memcpy(&v, src, 16);
+    *(v4i*)(out + o * 16) = v;
+}
+
+// ------------------------------------------------------------ quantisation front end
+A8W8_DEV float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+A8W8_DEV uint8_t quant_one(float x, float scale)
+{
+    const float q = __fdiv_rn(x, scale);
+    const uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(q, q, 0, false);
+    return (uint8_t)w;
+}
+
+// per-row scale = amax(row)/448; one workgroup per row
+__global__ void __launch_bounds__(256) quant_rowwise_kernel(const float* src, int k, int ld, uint8_t* q, float* scale)
+{
+    __shared__ float part[4];
+    const int row = blockIdx.x;
+    const float* x = src + (long long)row * ld;
+    float amax = 0.f;
+    for (int i = threadIdx.x; i < k; i += 256) amax = fmaxf(amax, fabsf(x[i]));
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    const float s = __fdiv_rn(amax, 448.0f);
+    if (threadIdx.x == 0) scale[row] = s;
+    for (int i = threadIdx.x; i < k; i += 256) q[(long long)row * k + i] = quant_one(x[i], s);
+}
+
+// 1 x 128 blocks: one wave per (row, 128-group); scale stored [k/128][rows]
+__global__ void __launch_bounds__(256) quant_1x128_kernel(const float* src, int rows, int k, int ld, uint8_t* q,
+                                                          float* scale)
+{
+    const int groups = k >> 7;
+    const long long w = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (w >= (long long)rows * groups) return;
+    const int row = (int)(w / groups), g = (int)(w % groups);
+    const int lane = threadIdx.x & 63;
+    const float* x = src + (long long)row * ld + g * 128;
+    const float v0 = x[lane], v1 = x[lane + 64];
+    const float amax = wave_max(fmaxf(fabsf(v0), fabsf(v1)));
+    const float s = __fdiv_rn(amax, 448.0f);
+    if (lane == 0) scale[(long long)g * rows + row] = s;
+    uint8_t* o = q + (long long)row * k + g * 128;
+    o[lane] = quant_one(v0, s);
+    o[lane + 64] = quant_one(v1, s);
+}
+
+// 128 x 128 blocks: one workgroup per block; scale stored [rows/128][k/128]
+__global__ void __launch_bounds__(256) quant_128x128_kernel(const float* src, int k, int ld, uint8_t* q, float* scale)
+{
+    __shared__ float part[4];
+    const int gk = blockIdx.x, gr = blockIdx.y;
+    const float* x = src + (long long)gr * 128 * ld + gk * 128;
+    float amax = 0.f;
+    for (int i = threadIdx.x; i < 128 * 128; i += 256) amax = fmaxf(amax, fabsf(x[(long long)(i >> 7) * ld + (i & 127)]));
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    const float s = __fdiv_rn(amax, 448.0f);
+    if (threadIdx.x == 0) scale[(long long)gr * gridDim.x + gk] = s;
+    uint8_t* o = q + (long long)gr * 128 * k + gk * 128;
+    for (int i = threadIdx.x; i < 128 * 128; i += 256)
+        o[(long long)(i >> 7) * k + (i & 127)] = quant_one(x[(long long)(i >> 7) * ld + (i & 127)], s);
+}
+
+// MX: one E8M0 exponent per 32 K-elements, e = ceil(log2(amax/448)) clamped to [-127, 127]
+// computed exactly from the fp32 exponent/mantissa fields; 32 lanes per block.
+__global__ void __launch_bounds__(256) quant_mx_kernel(const float* src, int rows, int k, int ld, uint8_t* q,
+                                                       uint8_t* scale)
+{
+    const int blocks = k >> 5;
+    const long long idx = ((long long)blockIdx.x * 256 + threadIdx.x) >> 5;
+    if (idx >= (long long)rows * blocks) return;
+    const int row = (int)(idx / blocks), g = (int)(idx % blocks);
+    const int l = threadIdx.x & 31;
+    const float v = src[(long long)row * ld + g * 32 + l];
+    float amax = fabsf(v);
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float t = __fdiv_rn(amax, 448.0f);
+    int e = -127;
+    if (t > 0.f) {
+        int ex;
+        const float f = frexpf(t, &ex);          // t = f * 2^ex, f in [0.5, 1)
+        e = (f == 0.5f) ? ex - 1 : ex;
+        e = max(-127, min(127, e));
+    }
+    if (l == 0) scale[(long long)row * blocks + g] = (uint8_t)(e + 127);
+    const float qv = ldexpf(v, -e);
+    const uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(qv, qv, 0, false);
+    q[(long long)row * k + g * 32 + l] = (uint8_t)w;
+}
+
+}  // namespace a8w8

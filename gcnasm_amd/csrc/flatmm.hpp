@@ -1,0 +1,131 @@
+// Skinny-M ("flat") A8W8 GEMM over pre-shuffled weights for gfx950.
+//
+// B arrives as Bshuf[n/16][k/64][4][16][16 B]: one 1 KiB block per (16 rows of B, 64 K),
+// ordered so that a 64-lane load of 16 bytes per lane is one contiguous 1 KiB read and lane
+// (kq = lane/16, r = lane%16) receives K bytes [16kq, 16kq+16) of row r -- half of a
+// 16 x 16 x 128 MFMA operand.  Two consecutive K blocks make one MFMA; the activation
+// fragment is gathered with the same K order, so no data ever moves through LDS.
+//
+// The kernel is bound by HBM: B is read exactly once with non-temporal 16-byte loads.
+// A workgroup is 8 waves that split K eight ways for the same NT weight tiles (all waves
+// stream B concurrently); the partial 16 x 16 accumulators are reduced through LDS and
+// the dequantisation scales are applied in fp32 before the bf16 store.
+#pragma once
+#include "a8w8_device.hpp"
+
+namespace a8w8 {
+
+constexpr int FLAT_WAVES = 8;
+constexpr int FLAT_THREADS = FLAT_WAVES * 64;
+
+template <int NT, int CDT, int MODE>
+__global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
+{
+    __shared__ v4f red[FLAT_WAVES][NT][64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = wave_uniform(tid >> 6);
+    const int batch = blockIdx.z;
+    const int r16 = lane & 15, kq = lane >> 4;
+
+    const int n_tiles = p.n >> 4;
+    const int k_tiles = p.k >> 6;
+    const int nt0 = blockIdx.x * NT;
+    const int m0 = blockIdx.y * 16;
+
+    const uint8_t* a_row = p.a + (long long)batch * p.a_batch + (long long)min(m0 + r16, p.m - 1) * p.lda + kq * 16;
+    const uint8_t* b_base = p.b + (long long)batch * p.b_batch + lane * 16;
+    const uint8_t* b_tile[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) b_tile[t] = b_base + (long long)min(nt0 + t, n_tiles - 1) * k_tiles * 1024;
+
+    // K blocks are consumed in pairs; this wave's share of the pairs
+    const int pairs = (k_tiles + 1) >> 1;
+    const int pp_begin = wave * pairs / FLAT_WAVES;
+    const int pp_end = (wave + 1) * pairs / FLAT_WAVES;
+
+    v4f acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    struct Frag {
+        v4i a[2];
+        v4i b[NT][2];
+    };
+    auto load = [&](int pp, Frag& f) {
+        const int kt0 = 2 * pp, kt1 = 2 * pp + 1;
+        const bool has1 = kt1 < k_tiles;
+        f.a[0] = *(const v4i*)(a_row + kt0 * 64);
+        f.a[1] = has1 ? *(const v4i*)(a_row + kt1 * 64) : v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            f.b[t][0] = __builtin_nontemporal_load((const v4i*)(b_tile[t] + (long long)kt0 * 1024));
+            f.b[t][1] = has1 ? __builtin_nontemporal_load((const v4i*)(b_tile[t] + (long long)kt1 * 1024))
+                             : v4i{0, 0, 0, 0};
+        }
+    };
+    auto mma = [&](const Frag& f) {
+        const v8i fa = v8i{f.a[0].x, f.a[0].y, f.a[0].z, f.a[0].w, f.a[1].x, f.a[1].y, f.a[1].z, f.a[1].w};
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const v8i fb = v8i{f.b[t][0].x, f.b[t][0].y, f.b[t][0].z, f.b[t][0].w,
+                               f.b[t][1].x, f.b[t][1].y, f.b[t][1].z, f.b[t][1].w};
+            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[t], 0, 0, 0, 0, 0, 0);
+        }
+    };
+
+    if (pp_begin < pp_end) {
+        Frag f0, f1;
+        load(pp_begin, f0);
+        int pp = pp_begin;
+        // two register stages, loads of the next pair in flight while the current one is used
+        while (true) {
+            if (pp + 1 < pp_end) load(pp + 1, f1);
+            mma(f0);
+            if (++pp >= pp_end) break;
+            if (pp + 1 < pp_end) load(pp + 1, f0);
+            mma(f1);
+            if (++pp >= pp_end) break;
+        }
+    }
+
+#pragma unroll
+    for (int t = 0; t < NT; ++t) red[wave][t][lane] = acc[t];
+    __syncthreads();
+
+    // lane holds C[m = r16][n = tile*16 + 4*kq .. +3]
+    if (tid < NT * 64) {
+        const int t = tid >> 6;
+        v4f s = red[0][t][lane];
+#pragma unroll
+        for (int w = 1; w < FLAT_WAVES; ++w) s += red[w][t][lane];
+        const int cm = m0 + r16;
+        const int cn = (nt0 + t) * 16 + 4 * kq;
+        if (cm < p.m && nt0 + t < n_tiles) {
+            const float* sfa = (const float*)p.sfa + (long long)batch * p.sfa_batch;
+            const float* sfb = (const float*)p.sfb + (long long)batch * p.sfb_batch;
+            if constexpr (MODE == MODE_TENSOR) {
+                s *= sfa[0] * sfb[0];
+            } else {
+                const v4f sb = v4f{sfb[cn], sfb[cn + 1], sfb[cn + 2], sfb[cn + 3]};
+                s *= sb * sfa[cm];
+            }
+            const long long ci = (long long)batch * p.c_batch + (long long)cm * p.ldc + cn;
+            if constexpr (CDT == C_BF16) {
+                unsigned short* dst = (unsigned short*)p.c + ci;
+                if ((p.ldc & 3) == 0 && (((uintptr_t)p.c + 2 * (long long)batch * p.c_batch) & 7) == 0) {
+                    *(v4u16*)dst = v4u16{bf16_bits(s.x), bf16_bits(s.y), bf16_bits(s.z), bf16_bits(s.w)};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dst[e] = bf16_bits(s[e]);
+                }
+            } else {
+                float* dst = (float*)p.c + ci;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[e] = s[e];
+            }
+        }
+    }
+}
+
+}  // namespace a8w8

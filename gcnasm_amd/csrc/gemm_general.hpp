@@ -1,0 +1,57 @@
+// General-shape A8W8 GEMM for gfx950: any m, n, k, strides and alignment, every scale mode.
+// One thread per element of C, sequential K, one product-times-scale per MAC without fused
+// multiply-add, i.e. the arithmetic order of the reference CPU GEMM
+// (opus_gemm/block_scale_gemm/gemm_a8w8_blockscale_host.cc:66-90).  It is the path for
+// shapes the tiled kernels do not take (k % 128 != 0, unaligned rows); it is not fast.
+#pragma once
+#include "a8w8_device.hpp"
+
+namespace a8w8 {
+
+A8W8_DEV float e4m3_to_f32_hw(uint8_t code) { return __builtin_amdgcn_cvt_f32_fp8((int)code, 0); }
+
+A8W8_DEV float e8m0_pair_scale(uint8_t ea, uint8_t eb)
+{
+    if (ea == 255 || eb == 255) return __builtin_nanf("");
+    return __builtin_ldexpf(1.0f, (int)ea + (int)eb - 254);
+}
+
+template <int MODE, int CDT>
+__global__ void __launch_bounds__(256) gemm_a8w8_general(GemmParams p)
+{
+#pragma clang fp contract(off)   // separate multiply and add, as the reference's host code rounds
+    const int j = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int i = blockIdx.y * 16 + (threadIdx.x >> 4);
+    const int batch = blockIdx.z;
+    if (i >= p.m || j >= p.n) return;
+    const uint8_t* a = p.a + (long long)batch * p.a_batch + (long long)i * p.lda;
+    const uint8_t* b = p.b + (long long)batch * p.b_batch + (long long)j * p.ldb;
+    const float* sfa_f = (const float*)p.sfa + (long long)batch * p.sfa_batch;
+    const float* sfb_f = (const float*)p.sfb + (long long)batch * p.sfb_batch;
+    const uint8_t* sfa_e = (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
+    const uint8_t* sfb_e = (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch;
+
+    const int group_k = MODE == MODE_BLOCK ? 128 : (MODE == MODE_MX ? 32 : p.k);
+    float sum = 0.f;
+    for (int k0 = 0; k0 < p.k; k0 += group_k) {
+        const int g = k0 / group_k;
+        float scale;
+        if constexpr (MODE == MODE_TENSOR) scale = sfa_f[0] * sfb_f[0];
+        if constexpr (MODE == MODE_ROWCOL) scale = sfa_f[i] * sfb_f[j];
+        if constexpr (MODE == MODE_BLOCK)
+            scale = sfa_f[(long long)g * p.stride_sfa + i] * sfb_f[(long long)(j >> 7) * p.stride_sfb + g];
+        if constexpr (MODE == MODE_MX)
+            scale = e8m0_pair_scale(sfa_e[(long long)i * p.stride_sfa + g], sfb_e[(long long)j * p.stride_sfb + g]);
+        const int k1 = min(k0 + group_k, p.k);
+        for (int k = k0; k < k1; ++k) {
+            const float prod = e4m3_to_f32_hw(a[k]) * e4m3_to_f32_hw(b[k]);
+            const float term = prod * scale;
+            sum = sum + term;
+        }
+    }
+    const long long ci = (long long)batch * p.c_batch + (long long)i * p.ldc + j;
+    if constexpr (CDT == C_BF16) ((unsigned short*)p.c)[ci] = bf16_bits(sum);
+    else ((float*)p.c)[ci] = sum;
+}
+
+}  // namespace a8w8

@@ -1,0 +1,148 @@
+/*
+ * libmi355a8w8 -- A8W8 (FP8 E4M3 x FP8 E4M3) quantised GEMM for MI355X (gfx950), C ABI.
+ *
+ * Plain pointers and sizes only.  Every device pointer is memory the caller owns on the
+ * current HIP device; the library allocates nothing and never frees caller memory.
+ * Calls are asynchronous on the supplied hipStream_t (passed as void*, NULL = the default
+ * stream, which is what the reference launches on); they do not synchronise.  Errors are
+ * returned as negative a8w8_status values; nothing throws or exits across this boundary.
+ *
+ * The entry points stand in for the kernel-launch contract of carlushuang/gcnasm's FP8
+ * GEMM demos.  Citations give the reference file:line (relative to its checkout) that
+ * each one replaces.
+ */
+#ifndef MI355_A8W8_H
+#define MI355_A8W8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define A8W8_API __attribute__((visibility("default")))
+
+typedef enum {
+    A8W8_OK = 0,
+    A8W8_ERR_NULL_POINTER = -1,   /* a required pointer is NULL                            */
+    A8W8_ERR_BAD_SHAPE = -2,      /* non-positive m/n/k/batch (host.cc:175-178)            */
+    A8W8_ERR_BAD_GROUP = -3,      /* n or k not a multiple of the scale group (host.cc:183-187) */
+    A8W8_ERR_BAD_STRIDE = -4,     /* a leading dimension smaller than the row it spans      */
+    A8W8_ERR_MISALIGNED = -5,     /* pointer or stride not aligned as the kernel needs      */
+    A8W8_ERR_BAD_MODE = -6,       /* unknown scale_mode / c_dtype / dialect, or a combination
+                                     the entry point does not implement                    */
+    A8W8_ERR_TOO_LARGE = -7,      /* an offset would not fit the 32-bit addressing in use   */
+    A8W8_ERR_LAUNCH = -8,         /* hipGetLastError() reported a failed launch             */
+    A8W8_ERR_NO_DEVICE = -9       /* no gfx950 device is current                            */
+} a8w8_status;
+
+/* How the dequantisation scales are laid out.  All fp32 unless stated.
+ *   TENSOR  sfa[1], sfb[1]
+ *   ROWCOL  sfa[m] (per row of A, "per token"), sfb[n] (per row of B, "per channel")
+ *   BLOCK   the reference layout (host.cc:78-79, 244-245):
+ *             sfa[g*stride_sfa + i]          one scale per 1 x 128 block of A, g = k/128
+ *             sfb[(j/128)*stride_sfb + g]    one scale per 128 x 128 block of B
+ *   MX      uint8 E8M0 exponents, one per 32 K-elements, value 2^(e-127):
+ *             sfa[i*stride_sfa + k/32], sfb[j*stride_sfb + k/32]                        */
+typedef enum {
+    A8W8_SCALE_TENSOR = 0,
+    A8W8_SCALE_ROWCOL = 1,
+    A8W8_SCALE_BLOCK_1x128_128x128 = 2,
+    A8W8_SCALE_MX_E8M0_1x32 = 3
+} a8w8_scale_mode;
+
+typedef enum { A8W8_C_BF16 = 0, A8W8_C_FP32 = 1 } a8w8_c_dtype;
+typedef enum { A8W8_E4M3_OCP = 0, A8W8_E4M3_FNUZ = 1 } a8w8_fp8_dialect;
+
+/* Argument block.  A superset of struct opus_gemm_kargs
+ * (opus_gemm/block_scale_gemm/gemm_a8w8_blockscale_common.h:4-25) with the same field
+ * meanings: A is [batch, m, k] row-major, B is [batch, n, k] row-major (the column-major
+ * K x N weight), C is [batch, m, n]; every stride counts ELEMENTS (common.h:12-17).
+ * A and B hold OCP E4M3 bytes.  C[i,j] = sum_k A[i,k] * B[j,k] * scale. */
+typedef struct {
+    const void* a;
+    const void* b;
+    void* c;
+    int m, n, k, batch;
+    int stride_a, stride_b, stride_c;
+    int stride_a_batch, stride_b_batch, stride_c_batch;
+    const void* sfa;
+    const void* sfb;
+    int stride_sfa, stride_sfb;
+    int stride_sfa_batch, stride_sfb_batch;
+    int scale_mode;      /* a8w8_scale_mode                                        */
+    int c_dtype;         /* a8w8_c_dtype                                           */
+    int b_preshuffled;   /* non-zero: b is in the a8w8_preshuffle_b layout (flatmm) */
+} a8w8_gemm_args;
+
+/* Dense GEMM, any scale mode.  Replaces the launch
+ *   gemm_a8w8_blockscale_kernel<Traits><<<grid, 512>>>(kargs)   (host.cc:14-15, 249-257)
+ * and the launches of the absent siblings gemm_a8w8_8wave (opus_gemm/rebuild.sh:3) for the
+ * per-tensor and row/column modes.  Needs k % 128 == 0 and 16-byte aligned A/B rows for
+ * the tiled kernels; other shapes run on a slower general kernel.  m, n edges are handled. */
+A8W8_API int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream);
+
+/* The block-scale entry point with exactly the reference's preconditions: scale_mode is
+ * taken as BLOCK_1x128_128x128, n % 128 == 0 and k % 128 == 0 are required
+ * (host.cc:179-187); c_dtype may be fp32 (the reference's output, common.h / host.cc:216)
+ * or bf16. */
+A8W8_API int a8w8_gemm_blockscale(const a8w8_gemm_args* args, void* hip_stream);
+
+/* Skinny-M GEMM over pre-shuffled weights (the flatmm_a8w8_gfx950 program listed at
+ * opus_fmm/README.md:9, built by opus_fmm/rebuild.sh:3-13).  Requires b_preshuffled != 0,
+ * scale_mode ROWCOL or TENSOR, m <= 64, n % 16 == 0, k % 64 == 0.  B is streamed once with
+ * 16-byte non-temporal loads. */
+A8W8_API int a8w8_flatmm(const a8w8_gemm_args* args, void* hip_stream);
+
+/* Host-side weight pre-shuffle, row-major b[n][k] -> Bshuf[n/16][k/64][4][16][16 bytes]:
+ * byte (j, p) moves to ((j/16*(k/64) + p/64)*4 + (p%64)/16)*256 + (j%16)*16 + p%16.
+ * The reference's own layout did not survive (source absent); this one is defined here.
+ * a8w8_unshuffle_b is its inverse.  Both work on host memory. */
+A8W8_API int a8w8_preshuffle_b(const void* b_host, void* out_host, int n, int k);
+A8W8_API int a8w8_unshuffle_b(const void* bshuf_host, void* out_host, int n, int k);
+/* The same permutation on device memory (src and dst must not overlap). */
+A8W8_API int a8w8_preshuffle_b_device(const void* b_dev, void* out_dev, int n, int k, void* hip_stream);
+
+/* fp32 -> E4M3, device buffers, one byte per element.
+ *   clamp240 != 0: to_fp8_raw_from_fp32 (cvt_fp8/test.cpp:21-43): finite inputs are
+ *       clamped to [-240, 240] by a median-of-three and then converted by the hardware
+ *       instruction; NaN/Inf bypass the clamp.
+ *   clamp240 == 0: the unclamped packed convert of pk_cvt_fp8x4_fp32x4_rne
+ *       (pk_cvt/test.cpp:220-257): elements 4i..4i+3 become the four bytes of word i,
+ *       little-endian, saturating to the largest finite value.
+ * dialect OCP uses the gfx950 hardware convert; FNUZ reproduces the gfx942 hardware result
+ * (bias 8, max 240, NaN 0x80) in software on the device.  Returns the element count
+ * converted, or 0 on error. */
+A8W8_API size_t a8w8_cvt_f32_to_e4m3(const float* src_dev, uint8_t* dst_dev, size_t n, int dialect,
+                                     int clamp240, void* hip_stream);
+/* E4M3 -> fp32, device buffers: fp8_e4m3fnuz_to_fp32_raw (cvt_fp8/test.cpp:59-90) and
+ * run_cast_from_f8<fp8, float, true> (pk_cvt/test.cpp:340-421) for FNUZ (0x80 -> NaN with
+ * bits 0x7F800001); the hardware convert for OCP. */
+A8W8_API size_t a8w8_cvt_e4m3_to_f32(const uint8_t* src_dev, float* dst_dev, size_t n, int dialect,
+                                     void* hip_stream);
+
+/* Quantisation front end: fp32 rows [rows, k] (leading dimension ld, elements) -> OCP E4M3
+ * bytes [rows, k] plus scales, in the layouts a8w8_gemm consumes.
+ *   ROWCOL: scale[r] = amax(row r)/448 (fp32)
+ *   BLOCK : group_rows = 1   -> scale[(p/128)*rows + r]       (the SFA layout)
+ *           group_rows = 128 -> scale[(r/128)*(k/128) + p/128] (the SFB layout)
+ *   MX    : uint8 e = clamp(ceil(log2(amax32/448)), -127, 127) + 127 at scale[r*(k/32) + p/32]
+ * TENSOR needs a grid-wide reduction first and is provided as ROWCOL followed by the
+ * caller's own max; it returns A8W8_ERR_BAD_MODE here. */
+A8W8_API int a8w8_quantize(const float* src_dev, int rows, int k, int ld, uint8_t* q_dev, void* scale_dev,
+                           int scale_mode, int group_rows, void* hip_stream);
+
+A8W8_API const char* a8w8_status_string(int status);
+
+/* Name of the kernel variant a8w8_gemm / a8w8_flatmm would launch for these arguments
+ * (for logs and profiles); NULL if the arguments are rejected. */
+A8W8_API const char* a8w8_kernel_name(const a8w8_gemm_args* args);
+
+/* Library version, major*10000 + minor*100 + patch. */
+A8W8_API int a8w8_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_A8W8_H */

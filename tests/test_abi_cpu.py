@@ -1,0 +1,106 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports every symbol
+the header declares, and rejects bad arguments with the documented status codes (argument
+validation runs before any device call, mirroring the reference harness's rejects at
+opus_gemm/block_scale_gemm/gemm_a8w8_blockscale_host.cc:175-187)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import gcnasm_amd as g
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_every_declared_symbol_is_exported():
+    text = open(os.path.join(ROOT, "include", "mi355_a8w8.h")).read()
+    names = set(re.findall(r"A8W8_API\s+[\w\s\*]+?\b(a8w8_\w+)\s*\(", text))
+    assert {"a8w8_gemm", "a8w8_gemm_blockscale", "a8w8_flatmm", "a8w8_preshuffle_b", "a8w8_cvt_f32_to_e4m3",
+            "a8w8_cvt_e4m3_to_f32", "a8w8_status_string"} <= names
+    L = ctypes.CDLL(g.library_path())
+    for n in names:
+        assert hasattr(L, n), n
+
+
+def _ok_args(mode=g.BLOCK, m=256, n=256, k=256, **kw):
+    # device addresses are never dereferenced on the host; any aligned non-null value will do
+    return g.raw_gemm_args(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, m, n, k, mode, **kw)
+
+
+@pytest.mark.parametrize("mutate,want", [
+    (lambda a: setattr(a, "a", None), -1),
+    (lambda a: setattr(a, "sfb", None), -1),
+    (lambda a: setattr(a, "m", 0), -2),
+    (lambda a: setattr(a, "batch", -1), -2),
+    (lambda a: setattr(a, "n", 200), -3),          # N % 128 for block scales
+    (lambda a: setattr(a, "k", 192), -3),          # K % 128 for block scales
+    (lambda a: setattr(a, "stride_a", 128), -4),
+    (lambda a: setattr(a, "stride_c", 100), -4),
+    (lambda a: setattr(a, "stride_sfa", 8), -4),
+    (lambda a: setattr(a, "scale_mode", 7), -6),
+    (lambda a: setattr(a, "c_dtype", 3), -6),
+    (lambda a: setattr(a, "b_preshuffled", 1), -6),
+])
+def test_gemm_rejects_bad_arguments(mutate, want):
+    a = _ok_args()
+    mutate(a)
+    assert g.lib().a8w8_gemm(ctypes.byref(a), None) == want
+    assert g.kernel_name(a) is None
+    assert g.status_string(want) != "unknown status"
+
+
+def test_null_struct_and_mx_group():
+    assert g.lib().a8w8_gemm(None, None) == -1
+    assert g.lib().a8w8_gemm_blockscale(None, None) == -1
+    a = _ok_args(mode=g.MX, k=48)
+    assert g.lib().a8w8_gemm(ctypes.byref(a), None) == -3
+    a = _ok_args(mode=g.ROWCOL, m=70000, k=32768, n=16)     # 2.29e9 bytes of A
+    assert g.lib().a8w8_gemm(ctypes.byref(a), None) == -7
+
+
+def test_flatmm_preconditions():
+    a = _ok_args(mode=g.ROWCOL, m=16, n=256, k=256, b_preshuffled=1)
+    assert g.kernel_name(a) == "flatmm_a8w8"
+    for mutate, want in [(lambda x: setattr(x, "b_preshuffled", 0), -6), (lambda x: setattr(x, "scale_mode", g.BLOCK), -6),
+                         (lambda x: setattr(x, "m", 65), -2), (lambda x: setattr(x, "n", 250), -3),
+                         (lambda x: setattr(x, "k", 96), -3), (lambda x: setattr(x, "a", 0x1001), -5)]:
+        b = _ok_args(mode=g.ROWCOL, m=16, n=256, k=256, b_preshuffled=1)
+        mutate(b)
+        if b.k == 96:
+            b.stride_a = 96
+        assert g.lib().a8w8_flatmm(ctypes.byref(b), None) == want
+
+
+def test_kernel_selection():
+    assert g.kernel_name(_ok_args()) == "gemm_a8w8_tile256"
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=200)) == "gemm_a8w8_general"
+    a = _ok_args(mode=g.ROWCOL)
+    a.a = 0x1004
+    assert g.kernel_name(a) == "gemm_a8w8_general"
+
+
+def test_good_arguments_pass_validation_and_stop_at_the_device():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("GPU present: the call would launch")
+    assert g.lib().a8w8_gemm(ctypes.byref(_ok_args()), None) == -9
+    assert "gfx950" in g.status_string(-9)
+
+
+def test_host_preshuffle_matches_oracle(orc):
+    rng = np.random.Generator(np.random.Philox(1))
+    b = rng.integers(0, 256, (48, 192)).astype(np.uint8)
+    bs = g.preshuffle_b(b)
+    assert (bs == orc.preshuffle_b(b)).all()
+    assert (g.unshuffle_b(bs, 48, 192) == b).all()
+    assert g.lib().a8w8_preshuffle_b(b.ctypes.data, bs.ctypes.data, 40, 192) == -3
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    import gcnasm_amd.api as api
+    monkeypatch.setattr(api, "_lib", None)
+    monkeypatch.setattr(api, "_SO", str(tmp_path / "nope.so"))
+    with pytest.raises(FileNotFoundError):
+        api.lib()
