@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""Benchmark of the A8W8 FP8 GEMM path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-extra]
+
+One "step" is one launch of the hot path over one batch of synthetic, already-quantised
+inputs resident in HBM.  The headline workload is the MXFP8 GEMM M=N=K=8192 (E4M3 elements,
+one E8M0 exponent per 32 K-elements, bf16 out); the other configurations and the M=16
+flatmm are timed after it and reported in the same JSON line under "other_workloads".
+Timing uses HIP events recorded on the stream the kernels are launched on, W untimed
+warm-up launches, then exactly K timed launches.  The CPU baseline is the oracle (a port
+of the reference's host GEMM) timed on a bounded slab of the same problem.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "FP8 GEMM TFLOPS & % gfx950 FP8 MFMA peak; HBM GB/s for M=16 flatmm"
+PEAK_FP8_TFLOPS = 5000.0      # MI355X dense FP8 MFMA, published
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: (mode, m, n, k, algorithmic bytes per launch)
+    "mxfp8_8192": ("mx", 8192, 8192, 8192, 272629760),
+    "rowcol_4096": ("rowcol", 4096, 4096, 4096, 67141632),
+    "block_4096x7168x2048": ("block", 4096, 7168, 2048, 82054656),
+    "tensor_256": ("tensor", 256, 256, 256, 262152),
+    "flatmm_16x16384x7168": ("flat", 16, 16384, 7168, 118145088),
+}
+
+
+def make_inputs(name, torch, g, seed):
+    """Synthetic operands of the workload's shape, quantised on the GPU by the library's own
+    front end (values N(0,1); the MX case multiplies each 32-block by 2^U(-4,4))."""
+    mode, m, n, k, _ = WORKLOADS[name]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+
+    def normal(rows):
+        return torch.randn((rows, k), generator=gen, device="cuda", dtype=torch.float32)
+
+    if mode == "mx":
+        out = []
+        for rows in (m, n):
+            x = normal(rows).view(rows, k // 32, 32)
+            x = x * torch.exp2(torch.rand((rows, k // 32, 1), generator=gen, device="cuda") * 8 - 4)
+            out.append(g.quantize(x.view(rows, k).contiguous(), g.MX))
+            del x
+        (a, sfa), (b, sfb) = out
+        return dict(a=a, b=b, sfa=sfa, sfb=sfb, mode=g.MX)
+    if mode == "block":
+        a, sfa = g.quantize(normal(m), g.BLOCK, 1)
+        b, sfb = g.quantize(normal(n), g.BLOCK, 128)
+        return dict(a=a, b=b, sfa=sfa, sfb=sfb, mode=g.BLOCK)
+    a, sfa = g.quantize(normal(m), g.ROWCOL)
+    b, sfb = g.quantize(normal(n), g.ROWCOL)
+    if mode == "tensor":
+        # one scale per tensor: requantise with the largest row scale
+        sa, sb = sfa.max().reshape(1), sfb.max().reshape(1)
+        a = g.cvt_f32_to_e4m3(g.cvt_e4m3_to_f32(a) * (sfa[:, None] / sa))
+        b = g.cvt_f32_to_e4m3(g.cvt_e4m3_to_f32(b) * (sfb[:, None] / sb))
+        return dict(a=a, b=b, sfa=sa.contiguous(), sfb=sb.contiguous(), mode=g.TENSOR)
+    if mode == "flat":
+        return dict(a=a, b=b, sfa=sfa, sfb=sfb, mode=g.ROWCOL, bshuf=g.preshuffle_b_device(b))
+    return dict(a=a, b=b, sfa=sfa, sfb=sfb, mode=g.ROWCOL)
+
+
+def time_launches(torch, fn, steps, warmup):
+    """Average launch duration in ms: W warm-up launches, then K launches between two HIP
+    events on the current stream (the stream the library is handed)."""
+    for _ in range(warmup):
+        fn(0)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1) / steps, wall_ms / steps
+
+
+def run_workload(name, torch, g, steps, warmup, seed):
+    mode, m, n, k, abytes = WORKLOADS[name]
+    inp = make_inputs(name, torch, g, seed)
+    flops = 2.0 * m * n * k
+    c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    res = {"workload": name, "m": m, "n": n, "k": k}
+    if mode == "flat":
+        # B (117 MB) fits the 256 MB Infinity Cache: rotate four copies so every launch reads HBM
+        copies = [inp["bshuf"]] + [inp["bshuf"].clone() for _ in range(3)]
+
+        def fn_rot(i):
+            g.flatmm(inp["a"], copies[i % 4], inp["sfa"], inp["sfb"], n, c=c)
+
+        def fn_same(i):
+            g.flatmm(inp["a"], copies[0], inp["sfa"], inp["sfb"], n, c=c)
+
+        ms, wall = time_launches(torch, fn_rot, steps, warmup)
+        ms_same, _ = time_launches(torch, fn_same, steps, warmup)
+        res.update(ms_per_launch=ms, wall_ms_per_launch=wall, gbs=abytes / ms / 1e6, gbs_same_buffer=abytes / ms_same / 1e6,
+                   tflops=flops / ms / 1e9, frac_hbm_peak=abytes / ms / 1e6 / PEAK_HBM_GBS,
+                   note="four rotating copies of B (470 MB) defeat the 256 MB Infinity Cache; gbs_same_buffer re-reads one copy")
+        fn = fn_rot
+    else:
+        def fn(i):
+            g.gemm(inp["a"], inp["b"], inp["sfa"], inp["sfb"], inp["mode"], c=c)
+
+        ms, wall = time_launches(torch, fn, steps, warmup)
+        res.update(ms_per_launch=ms, wall_ms_per_launch=wall, tflops=flops / ms / 1e9,
+                   frac_fp8_peak=flops / ms / 1e9 / PEAK_FP8_TFLOPS, gbs=abytes / ms / 1e6)
+    fn(0)
+    torch.cuda.synchronize()
+    return res, inp, c
+
+
+def cpu_baseline(name, inp, c_gpu, torch, budget_s=15.0):
+    """Times the oracle (port of the reference's host GEMM: per-MAC software fp8 decode,
+    OpenMP over (i, j), gemm_a8w8_blockscale_host.cc:66-90) on the first rows of the same
+    problem, sized to about budget_s seconds, and checks the GPU result on that slab."""
+    import numpy as np
+    import oracle
+    mode, m, n, k, _ = WORKLOADS[name]
+    a = inp["a"].cpu().numpy()
+    b = inp["b"].cpu().numpy()
+    sfa = inp["sfa"].cpu().numpy()
+    sfb = inp["sfb"].cpu().numpy()
+    omode = {"mx": oracle.MX, "rowcol": oracle.ROWCOL, "block": oracle.BLOCK, "tensor": oracle.TENSOR,
+             "flat": oracle.ROWCOL}[mode]
+    t0 = time.perf_counter()
+    oracle.gemm_ref(a, b, sfa, sfb, omode, rows=(0, 1), decode_per_mac=True)
+    t_row = time.perf_counter() - t0
+    rows = int(max(1, min(m, 256, budget_s / max(t_row, 1e-4))))
+    t0 = time.perf_counter()
+    ref = oracle.gemm_ref(a, b, sfa, sfb, omode, rows=(0, rows), decode_per_mac=True)
+    dt = time.perf_counter() - t0
+    got = c_gpu[:rows].float().cpu().numpy()
+    ok = np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-2
+    return {
+        "value": 2.0 * rows * n * k / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+        "sample": f"first {rows} of {m} rows of C (all N, all K), {dt:.2f} s; full problem extrapolates to "
+                  f"{dt * m / rows:.0f} s",
+        "gpu_slab_within_tolerance": float(ok.mean()),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="mxfp8_8192", choices=sorted(WORKLOADS))
+    ap.add_argument("--seed", type=int, default=0xA8A80004)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="time only the selected workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+
+    import torch
+    import gcnasm_amd as g
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    g.lib()     # raises if the HIP library has not been built; there is no fallback path
+    torch.cuda.set_device(0)
+
+    res, inp, c = run_workload(args.workload, torch, g, args.steps, args.warmup, args.seed)
+    mode, m, n, k, abytes = WORKLOADS[args.workload]
+    if mode == "flat":
+        value, unit = res["gbs"], "GB/s"
+        roof = {"bound": "hbm", "achieved": res["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": res["gbs"] / PEAK_HBM_GBS, "traffic": None, "kernel": "flatmm_a8w8"}
+    else:
+        value, unit = res["tflops"], "TFLOP/s"
+        roof = {"bound": "mfma", "achieved": res["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                "frac": res["tflops"] / PEAK_FP8_TFLOPS, "traffic": None, "kernel": "gemm_a8w8_tile256"}
+    line = {
+        "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": res["ms_per_launch"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3", "data": "synthetic",
+        "config": {"workload": args.workload, "m": m, "n": n, "k": k, "out": "bf16", "accumulate": "fp32",
+                   "algorithmic_bytes": abytes, "flop": 2 * m * n * k},
+        "roofline": roof,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(args.workload, inp, c, torch)
+    del inp, c
+    torch.cuda.empty_cache()
+    if not args.no_extra:
+        others = []
+        for name in WORKLOADS:
+            if name == args.workload:
+                continue
+            r, i2, c2 = run_workload(name, torch, g, args.steps, args.warmup, args.seed + 1)
+            others.append(r)
+            del i2, c2
+            torch.cuda.empty_cache()
+        line["other_workloads"] = others
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

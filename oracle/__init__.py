@@ -57,7 +57,7 @@ def lib():
         L.orc_encode_vec.argtypes = [_f32p, _u8p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int]
         L.orc_bf16_vec.argtypes = [_f32p, _u16p, ctypes.c_size_t]
         L.orc_gemm_ref.argtypes = [_u8p, _u8p, _f32p, _f32p, _f32p] + [ctypes.c_int] * 14
-        L.orc_gemm_ref_mx.argtypes = [_u8p, _u8p, _u8p, _u8p, _f32p] + [ctypes.c_int] * 10
+        L.orc_gemm_ref_mx.argtypes = [_u8p, _u8p, _u8p, _u8p, _f32p] + [ctypes.c_int] * 11
         L.orc_gemm_probe.argtypes = ([_u8p, _u8p, ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 9
                                      + [_i32p, _i32p, ctypes.c_int, _f32p])
         L.orc_preshuffle_index.restype = ctypes.c_size_t
@@ -154,7 +154,7 @@ def gemm_ref(a, b, sfa, sfb, mode, rows=None, decode_per_mac=False):
         sfa = _c(sfa, np.uint8)
         sfb = _c(sfb, np.uint8)
         lib().orc_gemm_ref_mx(_p(a, _u8p), _p(b, _u8p), _p(sfa, _u8p), _p(sfb, _u8p), _p(c, _f32p),
-                              m, n, k, k, k, n, sfa.shape[-1], sfb.shape[-1], r0, r1)
+                              m, n, k, k, k, n, sfa.shape[-1], sfb.shape[-1], r0, r1, int(decode_per_mac))
     else:
         sfa = _c(sfa, np.float32)
         sfb = _c(sfb, np.float32)

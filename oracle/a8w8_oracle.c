@@ -261,7 +261,7 @@ ORC_API void orc_gemm_ref(const uint8_t* a, const uint8_t* b, const float* sfa, 
  * (host.cc:66-90) with the scale decode of opus.hpp:1786. */
 ORC_API void orc_gemm_ref_mx(const uint8_t* a, const uint8_t* b, const uint8_t* ea, const uint8_t* eb,
                              float* c, int m, int n, int k, int lda, int ldb, int ldc,
-                             int stride_sfa, int stride_sfb, int row_begin, int row_end)
+                             int stride_sfa, int stride_sfb, int row_begin, int row_end, int decode_per_mac)
 {
     init_lut();
     (void)m;
@@ -275,7 +275,12 @@ ORC_API void orc_gemm_ref_mx(const uint8_t* a, const uint8_t* b, const uint8_t* 
                 uint8_t xa = ea[(size_t)i * stride_sfa + g], xb = eb[(size_t)j * stride_sfb + g];
                 float scale = (xa == 255 || xb == 255) ? u2f(0x7fc00000u)
                                                        : ldexpf(1.0f, (int)xa + (int)xb - 254);
-                for (int p = g * 32; p < g * 32 + 32; ++p) sum += lut_ocp[a_row[p]] * lut_ocp[b_row[p]] * scale;
+                if (decode_per_mac) {
+                    for (int p = g * 32; p < g * 32 + 32; ++p)
+                        sum += orc_e4m3_ocp_decode(a_row[p]) * orc_e4m3_ocp_decode(b_row[p]) * scale;
+                } else {
+                    for (int p = g * 32; p < g * 32 + 32; ++p) sum += lut_ocp[a_row[p]] * lut_ocp[b_row[p]] * scale;
+                }
             }
             c[(size_t)i * ldc + j] = sum;
         }
