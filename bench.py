@@ -155,8 +155,8 @@ def cpu_baseline(name, inp, c_gpu, torch, budget_s=15.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="mxfp8_8192", choices=sorted(WORKLOADS))
     ap.add_argument("--seed", type=int, default=0xA8A80004)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

@@ -81,9 +81,14 @@ GemmParams make_params(const a8w8_gemm_args* g)
     return p;
 }
 
-// The tiled kernels need whole 128-wide K steps and 16-byte aligned rows in A and B.
+// The tiled kernels need whole 128-wide K steps and 16-byte aligned rows in A and B; the MX
+// variant also stages its scale bytes with dword-granular loads.
 bool tiled_ok(const a8w8_gemm_args* g)
 {
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_1x32 &&
+        (g->stride_sfa % 4 != 0 || g->stride_sfb % 4 != 0 || ((uintptr_t)g->sfa & 3) || ((uintptr_t)g->sfb & 3) ||
+         (g->batch > 1 && (g->stride_sfa_batch % 4 != 0 || g->stride_sfb_batch % 4 != 0))))
+        return false;
     return g->k % BK == 0 && g->stride_a % 16 == 0 && g->stride_b % 16 == 0 && aligned16(g->a) && aligned16(g->b) &&
            (g->batch == 1 || (g->stride_a_batch % 16 == 0 && g->stride_b_batch % 16 == 0)) &&
            (long long)((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 31);
@@ -96,14 +101,14 @@ int launch_tiled(const GemmParams& p, int batch, hipStream_t stream)
     int dev = 0;
     (void)hipGetDevice(&dev);
     auto kern = gemm_a8w8_tile256<MODE, CDT>;
+    constexpr int lds_bytes = MODE == MODE_MX ? GEMM_LDS_BYTES_MX : GEMM_LDS_BYTES;
     if (!attr_set[dev & 63]) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES) !=
-            hipSuccess)
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
             return A8W8_ERR_LAUNCH;
         attr_set[dev & 63] = true;
     }
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch);
-    hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), GEMM_LDS_BYTES, stream, p);
+    hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), lds_bytes, stream, p);
     return launch_status();
 }
 
@@ -152,7 +157,7 @@ int validate_flat(const a8w8_gemm_args* g)
     return A8W8_OK;
 }
 
-constexpr int FLAT_NT = 2;
+constexpr int FLAT_NT = 4;   // weight tiles per wave: the activation fragment is re-used 4 times
 
 template <int CDT, int MODE>
 int launch_flat(const GemmParams& p, int batch, hipStream_t stream)

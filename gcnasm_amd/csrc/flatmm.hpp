@@ -8,7 +8,7 @@
 //
 // The kernel is bound by HBM: B is read exactly once with non-temporal 16-byte loads.
 // A workgroup is 8 waves that split K eight ways for the same NT weight tiles (all waves
-// stream B concurrently); the partial 16 x 16 accumulators are reduced through LDS and
+// stream B concurrently, the activation fragment of a K block is shared by the NT tiles); the partial 16 x 16 accumulators are reduced through LDS and
 // the dequantisation scales are applied in fp32 before the bf16 store.
 #pragma once
 #include "a8w8_device.hpp"
@@ -21,6 +21,7 @@ constexpr int FLAT_THREADS = FLAT_WAVES * 64;
 template <int NT, int CDT, int MODE>
 __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 {
+    static_assert(NT <= FLAT_WAVES, "wave t finishes weight tile t");
     __shared__ v4f red[FLAT_WAVES][NT][64];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -32,6 +33,24 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     const int k_tiles = p.k >> 6;
     const int nt0 = blockIdx.x * NT;
     const int m0 = blockIdx.y * 16;
+
+    // Wave t < NT writes tile t at the end: its lane holds C[m = r16][n = tile*16 + 4*kq .. +3].
+    // Its scales are fetched now, so that the tail of the kernel is only reduce + store.
+    const int cm = m0 + r16;
+    const int cn = (nt0 + wave) * 16 + 4 * kq;
+    const bool finisher = wave < NT && cm < p.m && nt0 + wave < n_tiles;
+    float sa = 1.f;
+    v4f sb = v4f{1.f, 1.f, 1.f, 1.f};
+    if (finisher) {
+        const float* sfa = (const float*)p.sfa + (long long)batch * p.sfa_batch;
+        const float* sfb = (const float*)p.sfb + (long long)batch * p.sfb_batch;
+        if constexpr (MODE == MODE_TENSOR) {
+            sa = sfa[0] * sfb[0];
+        } else {
+            sa = sfa[cm];
+            sb = v4f{sfb[cn], sfb[cn + 1], sfb[cn + 2], sfb[cn + 3]};
+        }
+    }
 
     const uint8_t* a_row = p.a + (long long)batch * p.a_batch + (long long)min(m0 + r16, p.m - 1) * p.lda + kq * 16;
     const uint8_t* b_base = p.b + (long long)batch * p.b_batch + lane * 16;
@@ -93,37 +112,24 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     for (int t = 0; t < NT; ++t) red[wave][t][lane] = acc[t];
     __syncthreads();
 
-    // lane holds C[m = r16][n = tile*16 + 4*kq .. +3]
-    if (tid < NT * 64) {
-        const int t = tid >> 6;
-        v4f s = red[0][t][lane];
+    if (finisher) {
+        v4f s = red[0][wave][lane];
 #pragma unroll
-        for (int w = 1; w < FLAT_WAVES; ++w) s += red[w][t][lane];
-        const int cm = m0 + r16;
-        const int cn = (nt0 + t) * 16 + 4 * kq;
-        if (cm < p.m && nt0 + t < n_tiles) {
-            const float* sfa = (const float*)p.sfa + (long long)batch * p.sfa_batch;
-            const float* sfb = (const float*)p.sfb + (long long)batch * p.sfb_batch;
-            if constexpr (MODE == MODE_TENSOR) {
-                s *= sfa[0] * sfb[0];
+        for (int w = 1; w < FLAT_WAVES; ++w) s += red[w][wave][lane];
+        s *= sb * sa;
+        const long long ci = (long long)batch * p.c_batch + (long long)cm * p.ldc + cn;
+        if constexpr (CDT == C_BF16) {
+            unsigned short* dst = (unsigned short*)p.c + ci;
+            if ((p.ldc & 3) == 0 && (((uintptr_t)p.c + 2 * (long long)batch * p.c_batch) & 7) == 0) {
+                *(v4u16*)dst = v4u16{bf16_bits(s.x), bf16_bits(s.y), bf16_bits(s.z), bf16_bits(s.w)};
             } else {
-                const v4f sb = v4f{sfb[cn], sfb[cn + 1], sfb[cn + 2], sfb[cn + 3]};
-                s *= sb * sfa[cm];
-            }
-            const long long ci = (long long)batch * p.c_batch + (long long)cm * p.ldc + cn;
-            if constexpr (CDT == C_BF16) {
-                unsigned short* dst = (unsigned short*)p.c + ci;
-                if ((p.ldc & 3) == 0 && (((uintptr_t)p.c + 2 * (long long)batch * p.c_batch) & 7) == 0) {
-                    *(v4u16*)dst = v4u16{bf16_bits(s.x), bf16_bits(s.y), bf16_bits(s.z), bf16_bits(s.w)};
-                } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) dst[e] = bf16_bits(s[e]);
-                }
-            } else {
-                float* dst = (float*)p.c + ci;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) dst[e] = s[e];
+                for (int e = 0; e < 4; ++e) dst[e] = bf16_bits(s[e]);
             }
+        } else {
+            float* dst = (float*)p.c + ci;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[e] = s[e];
         }
     }
 }

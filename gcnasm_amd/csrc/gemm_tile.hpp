@@ -20,6 +20,9 @@ constexpr int BM = 256, BN = 256, BK = 128;
 constexpr int GEMM_THREADS = 512;
 constexpr int STAGE_BYTES = (BM + BN) * BK;          // 65536
 constexpr int GEMM_LDS_BYTES = 2 * STAGE_BYTES;      // 131072
+// MX only: E8M0 scales of 4 K steps (16 bytes per row, 256 A rows then 256 B rows), two buffers
+constexpr int MX_GROUP_BYTES = (BM + BN) * 16;       // 8192
+constexpr int GEMM_LDS_BYTES_MX = GEMM_LDS_BYTES + 2 * MX_GROUP_BYTES;
 constexpr int WAVE_M = 64, WAVE_N = 128;
 constexpr int TM = WAVE_M / 16, TN = WAVE_N / 16;    // 4 x 8 MFMA tiles per wave
 
@@ -120,17 +123,29 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
     const uint8_t* sfa_e = (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
     const uint8_t* sfb_e = (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch;
     float blk_sa[TM], blk_sa_next[TM];
-    float blk_sb = 0.f, blk_sb_next = 0.f;
+    float blk_sb_next = 0.f;
     int mx_sa[TM], mx_sb[TN], mx_sa_next[TM], mx_sb_next[TN];
-    int mx_row_a[TM], mx_row_b[TN];
+    // MX: thread t stages the 16 scale bytes (4 K steps) of A row m0+t (t < 256) or B row
+    // n0+t-256 with one direct-to-LDS load per group of 4 K steps; lanes then pick single
+    // bytes with ds_read_u8, one K step ahead of their use.
+    __amdgpu_buffer_rsrc_t rsrc_sf = rsrc_a;
+    int voff_sf = 0, rd_sfa = 0, rd_sfb = 0;
     if constexpr (MODE == MODE_MX) {
-#pragma unroll
-        for (int t = 0; t < TM; ++t)
-            mx_row_a[t] = min(m0 + wave_m * WAVE_M + t * 16 + r16, p.m - 1) * p.stride_sfa + g;
-#pragma unroll
-        for (int t = 0; t < TN; ++t)
-            mx_row_b[t] = min(n0 + wave_n * WAVE_N + t * 16 + r16, p.n - 1) * p.stride_sfb + g;
+        const bool is_b = wave >= 4;                      // wave-uniform: waves 0-3 stage A rows, 4-7 B rows
+        const int rows = is_b ? p.n : p.m;
+        const int stride = is_b ? p.stride_sfb : p.stride_sfa;
+        rsrc_sf = make_rsrc(is_b ? sfb_e : sfa_e, (uint32_t)(rows - 1) * stride + (uint32_t)(p.k >> 5));
+        voff_sf = min((is_b ? n0 : m0) + (wave & 3) * 64 + lane, rows - 1) * stride;
+        rd_sfa = GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16 + g;
+        rd_sfb = GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + r16) * 16 + g;
     }
+    auto issue_mx_group = [&](int group) {
+        if constexpr (MODE == MODE_MX) {
+            A8W8_LDS char* s = (A8W8_LDS char*)smem + GEMM_LDS_BYTES + (group & 1) * MX_GROUP_BYTES + wave * 1024;
+            // the resource of the wave's matrix (waves 0-3 stage A rows, 4-7 B rows) is wave-uniform
+            load_to_lds_16(rsrc_sf, s, voff_sf, group * 16);
+        }
+    };
     auto fetch_scales = [&](int kstep) {
         if constexpr (MODE == MODE_BLOCK) {
 #pragma unroll
@@ -140,17 +155,17 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
             blk_sb_next = sfb_f[(long long)nb * p.stride_sfb + kstep];
         }
         if constexpr (MODE == MODE_MX) {
+            const unsigned char* s = (const unsigned char*)smem + ((kstep >> 2) & 1) * MX_GROUP_BYTES + (kstep & 3) * 4;
 #pragma unroll
-            for (int t = 0; t < TM; ++t) mx_sa_next[t] = sfa_e[mx_row_a[t] + kstep * 4];
+            for (int t = 0; t < TM; ++t) mx_sa_next[t] = s[rd_sfa + t * 256];
 #pragma unroll
-            for (int t = 0; t < TN; ++t) mx_sb_next[t] = sfb_e[mx_row_b[t] + kstep * 4];
+            for (int t = 0; t < TN; ++t) mx_sb_next[t] = s[rd_sfb + t * 256];
         }
     };
     auto rotate_scales = [&]() {
         if constexpr (MODE == MODE_BLOCK) {
 #pragma unroll
             for (int t = 0; t < TM; ++t) blk_sa[t] = blk_sa_next[t] * blk_sb_next;
-            blk_sb = blk_sb_next;
         }
         if constexpr (MODE == MODE_MX) {
 #pragma unroll
@@ -159,39 +174,43 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
             for (int t = 0; t < TN; ++t) mx_sb[t] = mx_sb_next[t];
         }
     };
-    (void)blk_sb;
 
     issue_stage(0, 0);
-    fetch_scales(0);
+    issue_mx_group(0);
+    if constexpr (MODE == MODE_BLOCK) fetch_scales(0);
     __builtin_amdgcn_s_waitcnt(0);          // everything issued so far has landed
     __syncthreads();
+    if constexpr (MODE == MODE_MX) fetch_scales(0);
 
     for (int ks = 0; ks < nk; ++ks) {
         const int cur = ks & 1;
         rotate_scales();
         if (ks + 1 < nk) {
             issue_stage(cur ^ 1, ks + 1);
+            if ((ks & 3) == 0 && ks + 4 < nk) issue_mx_group((ks >> 2) + 1);
             fetch_scales(ks + 1);
         }
 
-        v8i fa[TM];
+        // all A fragments of the step, B fragments one tile ahead of the MFMAs that use them
+        v8i fa[TM], fb[2];
 #pragma unroll
         for (int t = 0; t < TM; ++t) fa[t] = read_frag(cur, rd_a, t);
+        fb[0] = read_frag(cur, rd_b, 0);
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const v8i fb = read_frag(cur, rd_b, j);
+            if (j + 1 < TN) fb[(j + 1) & 1] = read_frag(cur, rd_b, j + 1);
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 if constexpr (MODE == MODE_MX) {
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        fb, fa[i], acc[i][j], 0, 0, 0, mx_sb[j], 0, mx_sa[i]);
+                        fb[j & 1], fa[i], acc[i][j], 0, 0, 0, mx_sb[j], 0, mx_sa[i]);
                 } else if constexpr (MODE == MODE_BLOCK) {
                     const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        fb, fa[i], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                        fb[j & 1], fa[i], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
                     acc[i][j] += part * blk_sa[i];
                 } else {
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        fb, fa[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+                        fb[j & 1], fa[i], acc[i][j], 0, 0, 0, 0, 0, 0);
                 }
             }
         }
