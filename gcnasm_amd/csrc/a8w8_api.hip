@@ -7,11 +7,14 @@
 #include "cvt.hpp"
 #include "flatmm.hpp"
 #include "gemm_general.hpp"
+#include "gemm_persist.hpp"
 #include "gemm_tile.hpp"
 
 using namespace a8w8;
 
 namespace {
+
+int g_num_cus[64];
 
 bool device_is_gfx950()
 {
@@ -21,6 +24,7 @@ bool device_is_gfx950()
     if (cached[dev] == 0) {
         hipDeviceProp_t prop;
         if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return false;
+        g_num_cus[dev] = prop.multiProcessorCount;
         cached[dev] = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
     }
     return cached[dev] == 1;
@@ -94,6 +98,15 @@ bool tiled_ok(const a8w8_gemm_args* g)
            (long long)((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 31);
 }
 
+// The persistent kernel pipelines two K steps ahead and indexes work items with an int.  The
+// block-scale mode stays on the plain tiled kernel, which is the faster of the two for it
+// (its per-step fp32 rescale leaves no registers for the second fragment set).
+bool persist_ok(const a8w8_gemm_args* g)
+{
+    return g->scale_mode != A8W8_SCALE_BLOCK_1x128_128x128 && g->k >= 2 * BK &&
+           (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 30);
+}
+
 template <int MODE, int CDT>
 int launch_tiled(const GemmParams& p, int batch, hipStream_t stream)
 {
@@ -109,6 +122,30 @@ int launch_tiled(const GemmParams& p, int batch, hipStream_t stream)
     }
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch);
     hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), lds_bytes, stream, p);
+    return launch_status();
+}
+
+// Persistent pipelined kernel: one workgroup per CU walks the (batch, tile) list.
+template <int MODE, int CDT>
+int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
+{
+    static bool attr_set[64];
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    auto kern = gemm_a8w8_persist<MODE, CDT>;
+    constexpr int lds_bytes = MODE == MODE_MX ? PERSIST_LDS_BYTES_MX : PERSIST_LDS_BYTES;
+    if (!attr_set[dev & 63]) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+            return A8W8_ERR_LAUNCH;
+        attr_set[dev & 63] = true;
+    }
+    PersistParams pp;
+    pp.g = p;
+    pp.batch = batch;
+    pp.items = batch * p.tiles_m * p.tiles_n;
+    const int cus = g_num_cus[dev & 63] > 0 ? g_num_cus[dev & 63] : 256;
+    dim3 grid((unsigned)(pp.items < cus ? pp.items : cus), 1, 1);
+    hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), lds_bytes, stream, pp);
     return launch_status();
 }
 
@@ -137,6 +174,10 @@ int launch_general(const GemmParams& p, int batch, hipStream_t stream)
 int dispatch_tiled(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
 {
     A8W8_DISPATCH(launch_tiled, g->scale_mode, g->c_dtype, p, g->batch, s)
+}
+int dispatch_persist(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
+{
+    A8W8_DISPATCH(launch_persist, g->scale_mode, g->c_dtype, p, g->batch, s)
 }
 int dispatch_general(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
 {
@@ -180,7 +221,8 @@ int a8w8_gemm(const a8w8_gemm_args* g, void* hip_stream)
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
     const GemmParams p = make_params(g);
     hipStream_t s = (hipStream_t)hip_stream;
-    return tiled_ok(g) ? dispatch_tiled(g, p, s) : dispatch_general(g, p, s);
+    if (!tiled_ok(g)) return dispatch_general(g, p, s);
+    return persist_ok(g) ? dispatch_persist(g, p, s) : dispatch_tiled(g, p, s);
 }
 
 int a8w8_gemm_blockscale(const a8w8_gemm_args* g, void* hip_stream)
@@ -340,7 +382,8 @@ const char* a8w8_kernel_name(const a8w8_gemm_args* g)
     if (!g) return nullptr;
     if (g->b_preshuffled) return validate_flat(g) == A8W8_OK ? "flatmm_a8w8" : nullptr;
     if (validate_common(g) != A8W8_OK) return nullptr;
-    return tiled_ok(g) ? "gemm_a8w8_tile256" : "gemm_a8w8_general";
+    if (!tiled_ok(g)) return "gemm_a8w8_general";
+    return persist_ok(g) ? "gemm_a8w8_persist" : "gemm_a8w8_tile256";
 }
 
 int a8w8_version(void) { return 100; }

@@ -1,0 +1,377 @@
+// Persistent, software-pipelined dense A8W8 GEMM for gfx950 (the fast path of a8w8_gemm).
+//
+// Tile 256 x 256 x 128, 8 waves (4 along M x 2 along N), wave tile 64 x 128 = 4 x 8 MFMA
+// tiles of 16 x 16 x 128, operands staged global -> LDS with 16-byte direct-to-LDS loads,
+// two LDS stages of 64 KiB, rows XOR-swizzled with (row & 7) exactly as in gemm_tile.hpp.
+//
+// What differs from the plain kernel:
+//  * One workgroup per CU walks a list of tiles; the K loop runs continuously across tile
+//    boundaries, so the loads of the next tile's first K steps are already in flight while
+//    the finished tile is scaled, converted and stored.
+//  * An LDS stage is handed back in two parts.  After MFMA group 3 of a step every wave has
+//    the step's A fragments and B tiles 0-3 in registers ("mid" barrier): the A half and the
+//    low B half of the stage are free and the loads of the step after next start landing
+//    there.  After group 6 all B tiles have been read ("end" barrier) and the high B half
+//    follows.  Every byte therefore has about 1.5 K steps to arrive instead of one.
+//  * The eight loads of a stage are issued one or two per MFMA group instead of as a burst,
+//    and the next step's A fragments are fetched from LDS in the shadow of the last group.
+//  * Barriers are raw s_barrier instructions with hand-placed s_waitcnt: the compiler's
+//    workgroup fence would wait for every outstanding direct-to-LDS load at each barrier.
+//    Loads complete in issue order, so "all but the newest four" (vmcnt(4)) at the end
+//    barrier is exactly "the stage about to be read has landed".
+#pragma once
+#include <utility>
+
+#include "gemm_tile.hpp"
+
+namespace a8w8 {
+
+// LDS: two operand stages, then (MX only) two scale groups of 4 K steps.
+constexpr int PERSIST_LDS_BYTES = GEMM_LDS_BYTES;
+constexpr int PERSIST_LDS_BYTES_MX = GEMM_LDS_BYTES_MX;
+
+#define A8W8_RAW_BARRIER() asm volatile("s_barrier" ::: "memory")
+#ifndef A8W8_PERSIST_SB
+#define A8W8_PERSIST_SB 0
+#endif
+#if A8W8_PERSIST_SB
+#define A8W8_PERSIST_SCHED_BARRIER() __builtin_amdgcn_sched_barrier(0)
+#else
+#define A8W8_PERSIST_SCHED_BARRIER() (void)0
+#endif
+
+struct PersistParams {
+    GemmParams g;
+    int batch;        // work items = batch * tiles_m * tiles_n, walked with stride gridDim.x
+    int items;
+};
+
+template <int MODE, int CDT>
+__global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistParams pp)
+{
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const GemmParams& p = pp.g;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = wave_uniform(tid >> 6);
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int nk = p.k / BK;                       // >= 2 (checked by the host)
+    const int tiles = p.tiles_m * p.tiles_n;
+
+    // ---------------------------------------------------------------- load side state
+    // position of the stage whose loads are being issued: (item, k step), two steps ahead
+    int ld_item = blockIdx.x, ld_ks = 0;
+    const int groups_per_tile = (nk + 3) >> 2;      // MX scale groups (4 K steps each) per tile
+    int ld_gbase = 0, cur_gbase = 0;                // running group count: picks the scale buffer
+    __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_sf;
+    int voff_a[4], voff_b[4], voff_sf = 0;
+    const int ld_row = wave * 8 + (lane >> 3);
+    const int ld_piece = (lane & 7) ^ (lane >> 3);
+    auto point_loads_at = [&](int item) __attribute__((always_inline)) {
+        item = min(item, pp.items - 1);            // past the end: keep loading valid data nobody reads
+        const int batch = item / tiles;
+        int tm, tn;
+        tile_of_block(item - batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+        const int m0 = tm * BM, n0 = tn * BN;
+        rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
+        rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, (uint32_t)(p.n - 1) * p.ldb + p.k);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            voff_a[j] = min(m0 + ld_row + 64 * j, p.m - 1) * p.lda + ld_piece * 16;
+            voff_b[j] = min(n0 + ld_row + 64 * j, p.n - 1) * p.ldb + ld_piece * 16;
+        }
+        if constexpr (MODE == MODE_MX) {
+            const bool is_b = wave >= 4;           // waves 0-3 stage A-row scales, 4-7 B-row scales
+            const int rows = is_b ? p.n : p.m;
+            const int stride = is_b ? p.stride_sfb : p.stride_sfa;
+            const uint8_t* base = is_b ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
+                                       : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
+            rsrc_sf = make_rsrc(base, (uint32_t)(rows - 1) * stride + (uint32_t)(p.k >> 5));
+            voff_sf = min((is_b ? n0 : m0) + (wave & 3) * 64 + lane, rows - 1) * stride;
+        }
+    };
+    // one of the eight loads of a stage: 0..3 = A chunks, 4,5 = low B chunks, 6,7 = high B chunks.
+    // Wave w fills rows 8w + 64j (+0..7) of each matrix; for B, j = 0, 2 are the rows of MFMA
+    // tiles 0-3 of the two wave columns ("low"), j = 1, 3 those of tiles 4-7 ("high").
+    auto issue_one = [&](int stage, int kstep, int which) __attribute__((always_inline)) {
+        A8W8_LDS char* s = (A8W8_LDS char*)smem + stage * STAGE_BYTES + wave * 1024;
+        const int koff = kstep * BK;
+        if (which < 4) {
+            load_to_lds_16(rsrc_a, s + which * 8192, voff_a[which], koff);
+        } else {
+            const int j = which == 4 ? 0 : which == 5 ? 2 : which == 6 ? 1 : 3;
+            load_to_lds_16(rsrc_b, s + BM * BK + j * 8192, voff_b[j], koff);
+        }
+    };
+    auto issue_mx_group = [&](int group) __attribute__((always_inline)) {
+        if constexpr (MODE == MODE_MX) {
+            A8W8_LDS char* s =
+                (A8W8_LDS char*)smem + GEMM_LDS_BYTES + ((ld_gbase + group) & 1) * MX_GROUP_BYTES + wave * 1024;
+            load_to_lds_16(rsrc_sf, s, voff_sf, group * 16);
+        }
+    };
+    auto advance_ld = [&]() __attribute__((always_inline)) {                      // the load position moves one K step
+        if (++ld_ks == nk) {
+            ld_ks = 0;
+            ld_item += gridDim.x;
+            ld_gbase += groups_per_tile;
+            point_loads_at(ld_item);
+        }
+    };
+
+    // ---------------------------------------------------------------- compute side state
+    int rd_a[2], rd_b[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int slot = (g + 4 * h) ^ (lane & 7);
+        rd_a[h] = (wave_m * WAVE_M + r16) * BK + (slot << 4);
+        rd_b[h] = BM * BK + (wave_n * WAVE_N + r16) * BK + (slot << 4);
+    }
+    auto read_frag = [&](int stage, const int (&base)[2], int t) -> v8i {
+        const char* s = smem + stage * STAGE_BYTES + t * (16 * BK);
+        const v4i lo = *(const v4i*)(s + base[0]);
+        const v4i hi = *(const v4i*)(s + base[1]);
+        return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    };
+    const int rd_sfa = GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16;
+    const int rd_sfb = GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + r16) * 16;
+
+    int cur_item = blockIdx.x, cur_ks = 0;         // the step being multiplied
+    int cur_batch = 0, m0 = 0, n0 = 0;
+    auto point_compute_at = [&](int item) __attribute__((always_inline)) {
+        cur_batch = item / tiles;
+        int tm, tn;
+        tile_of_block(item - cur_batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+        m0 = tm * BM;
+        n0 = tn * BN;
+    };
+
+    v4f acc[TM][TN];
+    auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    };
+
+    // scales consumed by the MFMAs of a step (BLOCK: fp32 per row x per column block, MX: E8M0 bytes)
+    float blk_s[TM], blk_s_next[TM];
+    int mx_sa[TM], mx_sb[TN], mx_sa_next[TM], mx_sb_next[TN];
+    auto fetch_step_scales = [&](int batch, int mm0, int nn0, int kstep, int gbase) __attribute__((always_inline)) {
+        (void)gbase;
+        if constexpr (MODE == MODE_BLOCK) {
+            const float* sfa_f = (const float*)p.sfa + (long long)batch * p.sfa_batch;
+            const float* sfb_f = (const float*)p.sfb + (long long)batch * p.sfb_batch;
+            const int nb = min(nn0 + wave_n * WAVE_N, p.n - 1) >> 7;
+            const float sb = sfb_f[(long long)nb * p.stride_sfb + kstep];
+#pragma unroll
+            for (int t = 0; t < TM; ++t)
+                blk_s_next[t] =
+                    sfa_f[(long long)kstep * p.stride_sfa + min(mm0 + wave_m * WAVE_M + r16 + 16 * t, p.m - 1)] * sb;
+        }
+        if constexpr (MODE == MODE_MX) {
+            // one dword per (row, K step) holds the four block exponents; lane group g extracts
+            // byte g when the step begins, so nothing waits on these reads in the step issuing them
+            const char* s = smem + ((gbase + (kstep >> 2)) & 1) * MX_GROUP_BYTES + (kstep & 3) * 4;
+#pragma unroll
+            for (int t = 0; t < TM; ++t)
+                mx_sa_next[t] = *(const int*)(s + rd_sfa + t * 256);
+#pragma unroll
+            for (int t = 0; t < TN; ++t)
+                mx_sb_next[t] = *(const int*)(s + rd_sfb + t * 256);
+        }
+    };
+    auto rotate_step_scales = [&]() __attribute__((always_inline)) {
+        if constexpr (MODE == MODE_BLOCK) {
+#pragma unroll
+            for (int t = 0; t < TM; ++t) blk_s[t] = blk_s_next[t];
+        }
+        if constexpr (MODE == MODE_MX) {
+#pragma unroll
+            for (int t = 0; t < TM; ++t) mx_sa[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sa_next[t], 8 * g, 8);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sb_next[t], 8 * g, 8);
+        }
+    };
+
+    // ---------------------------------------------------------------- epilogue of one tile
+    auto store_tile = [&]() __attribute__((always_inline)) {
+        const float* sfa_f = (const float*)p.sfa + (long long)cur_batch * p.sfa_batch;
+        const float* sfb_f = (const float*)p.sfb + (long long)cur_batch * p.sfb_batch;
+        const int cm_base = m0 + wave_m * WAVE_M + r16;
+        const int cn_base = n0 + wave_n * WAVE_N + 4 * g;
+        float sa[TM];
+        float ts = 1.f;
+        if constexpr (MODE == MODE_TENSOR) ts = sfa_f[0] * sfb_f[0];
+        if constexpr (MODE == MODE_ROWCOL) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) sa[i] = sfa_f[min(cm_base + 16 * i, p.m - 1)];
+        }
+        char* c_base = (char*)p.c + (long long)cur_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
+        const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 7) == 0)
+                                            : ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 15) == 0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int cn = cn_base + 16 * j;
+            v4f sb = v4f{1.f, 1.f, 1.f, 1.f};
+            if constexpr (MODE == MODE_ROWCOL) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sb[e] = sfb_f[min(cn + e, p.n - 1)];
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int cm = cm_base + 16 * i;
+                v4f v = acc[i][j];
+                if constexpr (MODE == MODE_TENSOR) v *= ts;
+                if constexpr (MODE == MODE_ROWCOL) v *= sb * sa[i];
+                if (cm >= p.m) continue;
+                if constexpr (CDT == C_BF16) {
+                    unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
+                    if (vec_ok && cn + 3 < p.n) {
+                        A8W8_STORE_C((v4u16*)dst, (v4u16{bf16_bits(v.x), bf16_bits(v.y), bf16_bits(v.z), bf16_bits(v.w)}));
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (cn + e < p.n) dst[e] = bf16_bits(v[e]);
+                    }
+                } else {
+                    float* dst = (float*)c_base + (long long)cm * p.ldc + cn;
+                    if (vec_ok && cn + 3 < p.n) {
+                        A8W8_STORE_C((v4f*)dst, v);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (cn + e < p.n) dst[e] = v[e];
+                    }
+                }
+            }
+        }
+    };
+
+    // ---------------------------------------------------------------- prologue
+    struct Frags {
+        v8i a[TM];
+        v8i b0;
+    };
+    Frags F[2];
+    const int my_items = (pp.items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int total_steps = my_items * nk;
+
+    if (my_items == 0) return;
+    point_loads_at(ld_item);
+    point_compute_at(cur_item);
+    // the stages of steps 0 and 1 in full and MX scale group 0; the load position stays at step 1,
+    // whose last two loads the first step re-issues (same data, nobody is reading that stage yet)
+#pragma unroll
+    for (int w = 0; w < 8; ++w) issue_one(0, 0, w);
+    issue_mx_group(0);
+    advance_ld();
+#pragma unroll
+    for (int w = 0; w < 8; ++w) issue_one(1, ld_ks, w);
+    if constexpr (MODE == MODE_BLOCK) fetch_step_scales(cur_batch, m0, n0, 0, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    A8W8_RAW_BARRIER();
+    if constexpr (MODE == MODE_MX) fetch_step_scales(cur_batch, m0, n0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < TM; ++t) F[0].a[t] = read_frag(0, rd_a, t);
+    F[0].b0 = read_frag(0, rd_b, 0);
+    zero_acc();
+
+    // ---------------------------------------------------------------- one K step
+    // Loads of the stage at the load position X: A chunks after MFMA groups 3..6 of step X-2,
+    // first low/high B chunks after group 7, the second ones after groups 0 and 1 of step X-1;
+    // the position advances after group 2.
+    auto step = [&](auto parity) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity)::value;
+        Frags& cur = F[P];
+        Frags& nxt = F[P ^ 1];
+        rotate_step_scales();
+        // where the next step lives (it may be the first step of this workgroup's next tile)
+        const bool last_of_tile = cur_ks + 1 == nk;
+        int nx_batch = cur_batch, nx_m0 = m0, nx_n0 = n0, nx_gbase = cur_gbase;
+        const int nx_ks = last_of_tile ? 0 : cur_ks + 1;
+        if (last_of_tile) {
+            const int item = min(cur_item + (int)gridDim.x, pp.items - 1);
+            nx_batch = item / tiles;
+            int tm, tn;
+            tile_of_block(item - nx_batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+            nx_m0 = tm * BM;
+            nx_n0 = tn * BN;
+            nx_gbase = cur_gbase + groups_per_tile;
+        }
+
+        v8i fb[TN];
+        fb[0] = cur.b0;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if (j + 1 < TN) fb[j + 1] = read_frag(P, rd_b, j + 1);
+            A8W8_PERSIST_SCHED_BARRIER();
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                if constexpr (MODE == MODE_MX) {
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], cur.a[i], acc[i][j], 0, 0, 0,
+                                                                                 mx_sb[j], 0, mx_sa[i]);
+                } else if constexpr (MODE == MODE_BLOCK) {
+                    const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                        fb[j], cur.a[i], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                    acc[i][j] += part * blk_s[i];
+                } else {
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], cur.a[i], acc[i][j], 0, 0, 0,
+                                                                                 0, 0, 0);
+                }
+            }
+            A8W8_PERSIST_SCHED_BARRIER();
+
+            if (j == 0) issue_one(P ^ 1, ld_ks, 5);
+            if (j == 1) issue_one(P ^ 1, ld_ks, 7);
+            if (j == 2) {
+                advance_ld();
+                if constexpr (MODE == MODE_MX) {
+                    if ((ld_ks & 3) == 0) issue_mx_group(ld_ks >> 2);   // scales of steps ld_ks .. ld_ks+3
+                }
+                if constexpr (MODE == MODE_BLOCK) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, 0);
+            }
+            if (j == 3) {
+                __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): A fragments and B tiles 0..4 are in registers
+                A8W8_RAW_BARRIER();                   // mid: the A half and low B half of stage P are free
+                issue_one(P, ld_ks, 0);
+            }
+            if (j == 4) issue_one(P, ld_ks, 1);
+            if (j == 5) issue_one(P, ld_ks, 2);
+            if (j == 6) {
+                issue_one(P, ld_ks, 3);
+                __builtin_amdgcn_s_waitcnt(0x0074);   // vmcnt(4) lgkmcnt(0): the next stage has landed
+                A8W8_RAW_BARRIER();                   // end: all of stage P is free
+#pragma unroll
+                for (int t = 0; t < TM; ++t) nxt.a[t] = read_frag(P ^ 1, rd_a, t);
+                nxt.b0 = read_frag(P ^ 1, rd_b, 0);
+                if constexpr (MODE == MODE_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
+            }
+            if (j == 7) {
+                issue_one(P, ld_ks, 4);
+                issue_one(P, ld_ks, 6);
+            }
+        }
+        if (last_of_tile) {
+            store_tile();
+            zero_acc();
+            cur_item += gridDim.x;
+            cur_ks = 0;
+            cur_batch = nx_batch;
+            m0 = nx_m0;
+            n0 = nx_n0;
+            cur_gbase = nx_gbase;
+        } else {
+            ++cur_ks;
+        }
+    };
+
+    for (int s = 0; s < total_steps; s += 2) {
+        step(std::integral_constant<int, 0>{});
+        if (s + 1 < total_steps) step(std::integral_constant<int, 1>{});
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // no direct-to-LDS load may outlive the workgroup's LDS allocation
+}
+
+}  // namespace a8w8

@@ -136,8 +136,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
         const int stride = is_b ? p.stride_sfb : p.stride_sfa;
         rsrc_sf = make_rsrc(is_b ? sfb_e : sfa_e, (uint32_t)(rows - 1) * stride + (uint32_t)(p.k >> 5));
         voff_sf = min((is_b ? n0 : m0) + (wave & 3) * 64 + lane, rows - 1) * stride;
-        rd_sfa = GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16 + g;
-        rd_sfb = GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + r16) * 16 + g;
+        rd_sfa = GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16;
+        rd_sfb = GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + r16) * 16;
     }
     auto issue_mx_group = [&](int group) {
         if constexpr (MODE == MODE_MX) {
@@ -155,11 +155,16 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
             blk_sb_next = sfb_f[(long long)nb * p.stride_sfb + kstep];
         }
         if constexpr (MODE == MODE_MX) {
-            const unsigned char* s = (const unsigned char*)smem + ((kstep >> 2) & 1) * MX_GROUP_BYTES + (kstep & 3) * 4;
+            // one dword per (row, K step) holds the four block exponents (four lanes reading one
+            // dword is a broadcast); lane group g extracts byte g when the step begins, so that
+            // nothing waits on these reads inside the step that issues them
+            const char* s = smem + ((kstep >> 2) & 1) * MX_GROUP_BYTES + (kstep & 3) * 4;
 #pragma unroll
-            for (int t = 0; t < TM; ++t) mx_sa_next[t] = s[rd_sfa + t * 256];
+            for (int t = 0; t < TM; ++t)
+                mx_sa_next[t] = *(const int*)(s + rd_sfa + t * 256);
 #pragma unroll
-            for (int t = 0; t < TN; ++t) mx_sb_next[t] = s[rd_sfb + t * 256];
+            for (int t = 0; t < TN; ++t)
+                mx_sb_next[t] = *(const int*)(s + rd_sfb + t * 256);
         }
     };
     auto rotate_scales = [&]() {
@@ -169,9 +174,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
         }
         if constexpr (MODE == MODE_MX) {
 #pragma unroll
-            for (int t = 0; t < TM; ++t) mx_sa[t] = mx_sa_next[t];
+            for (int t = 0; t < TM; ++t) mx_sa[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sa_next[t], 8 * g, 8);
 #pragma unroll
-            for (int t = 0; t < TN; ++t) mx_sb[t] = mx_sb_next[t];
+            for (int t = 0; t < TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sb_next[t], 8 * g, 8);
         }
     };
 
@@ -247,7 +252,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
             if constexpr (CDT == C_BF16) {
                 unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
                 if (vec_ok && cn + 3 < p.n) {
-                    *(v4u16*)dst = v4u16{bf16_bits(v.x), bf16_bits(v.y), bf16_bits(v.z), bf16_bits(v.w)};
+                    A8W8_STORE_C((v4u16*)dst, (v4u16{bf16_bits(v.x), bf16_bits(v.y), bf16_bits(v.z), bf16_bits(v.w)}));
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
@@ -256,7 +261,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
             } else {
                 float* dst = (float*)c_base + (long long)cm * p.ldc + cn;
                 if (vec_ok && cn + 3 < p.n) {
-                    *(v4f*)dst = v;
+                    A8W8_STORE_C((v4f*)dst, v);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
