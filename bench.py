@@ -88,33 +88,69 @@ def time_launches(torch, fn, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall_ms / steps
 
 
-def run_workload(name, torch, g, steps, warmup, seed):
+def time_best_of(torch, fn, steps, warmup, rounds=3):
+    """For the secondary workloads: bring the clocks up with at least 100 ms of warm-up launches,
+    then report the best of `rounds` timed regions of `steps` launches each."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.1:
+        for _ in range(20):
+            fn(0)
+        torch.cuda.synchronize()
+    best = None
+    for _ in range(rounds):
+        r = time_launches(torch, fn, steps, warmup)
+        if best is None or r[0] < best[0]:
+            best = r
+    return best
+
+
+def run_workload(name, torch, g, steps, warmup, seed, headline=True):
     mode, m, n, k, abytes = WORKLOADS[name]
     inp = make_inputs(name, torch, g, seed)
     flops = 2.0 * m * n * k
     c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     res = {"workload": name, "m": m, "n": n, "k": k}
+    res["kernel"] = "flatmm_a8w8" if mode == "flat" else None
+    import ctypes
+    L = g.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def args_for(b_tensor, preshuffled):
+        # the C argument block is filled once; the timed loop is only the C-ABI call
+        return g.raw_gemm_args(inp["a"].data_ptr(), b_tensor.data_ptr(), c.data_ptr(), inp["sfa"].data_ptr(),
+                               inp["sfb"].data_ptr(), m, n, k, inp["mode"], g.BF16, b_preshuffled=preshuffled)
+
     if mode == "flat":
         # B (117 MB) fits the 256 MB Infinity Cache: rotate four copies so every launch reads HBM
         copies = [inp["bshuf"]] + [inp["bshuf"].clone() for _ in range(3)]
+        flat_args = [ctypes.byref(args_for(x, 1)) for x in copies]
+        keep = [a._obj for a in flat_args]   # noqa: F841  (keeps the structs alive)
 
         def fn_rot(i):
-            g.flatmm(inp["a"], copies[i % 4], inp["sfa"], inp["sfb"], n, c=c)
+            if L.a8w8_flatmm(flat_args[i & 3], stream) != 0:
+                raise RuntimeError("a8w8_flatmm failed")
 
         def fn_same(i):
-            g.flatmm(inp["a"], copies[0], inp["sfa"], inp["sfb"], n, c=c)
+            if L.a8w8_flatmm(flat_args[0], stream) != 0:
+                raise RuntimeError("a8w8_flatmm failed")
 
-        ms, wall = time_launches(torch, fn_rot, steps, warmup)
-        ms_same, _ = time_launches(torch, fn_same, steps, warmup)
+        timer = time_launches if headline else time_best_of
+        ms, wall = timer(torch, fn_rot, steps, warmup)
+        ms_same, _ = timer(torch, fn_same, steps, warmup)
         res.update(ms_per_launch=ms, wall_ms_per_launch=wall, gbs=abytes / ms / 1e6, gbs_same_buffer=abytes / ms_same / 1e6,
                    tflops=flops / ms / 1e9, frac_hbm_peak=abytes / ms / 1e6 / PEAK_HBM_GBS,
                    note="four rotating copies of B (470 MB) defeat the 256 MB Infinity Cache; gbs_same_buffer re-reads one copy")
         fn = fn_rot
     else:
-        def fn(i):
-            g.gemm(inp["a"], inp["b"], inp["sfa"], inp["sfb"], inp["mode"], c=c)
+        gemm_args = args_for(inp["b"], 0)
+        gemm_ref_ = ctypes.byref(gemm_args)
 
-        ms, wall = time_launches(torch, fn, steps, warmup)
+        def fn(i):
+            if L.a8w8_gemm(gemm_ref_, stream) != 0:
+                raise RuntimeError("a8w8_gemm failed")
+
+        res["kernel"] = g.kernel_name(gemm_args)
+        ms, wall = (time_launches if headline else time_best_of)(torch, fn, steps, warmup)
         res.update(ms_per_launch=ms, wall_ms_per_launch=wall, tflops=flops / ms / 1e9,
                    frac_fp8_peak=flops / ms / 1e9 / PEAK_FP8_TFLOPS, gbs=abytes / ms / 1e6)
     fn(0)
@@ -181,7 +217,7 @@ def main():
     else:
         value, unit = res["tflops"], "TFLOP/s"
         roof = {"bound": "mfma", "achieved": res["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                "frac": res["tflops"] / PEAK_FP8_TFLOPS, "traffic": None, "kernel": "gemm_a8w8_tile256"}
+                "frac": res["tflops"] / PEAK_FP8_TFLOPS, "traffic": None, "kernel": res.get("kernel")}
     line = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": res["ms_per_launch"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -199,7 +235,8 @@ def main():
         for name in WORKLOADS:
             if name == args.workload:
                 continue
-            r, i2, c2 = run_workload(name, torch, g, args.steps, args.warmup, args.seed + 1)
+            r, i2, c2 = run_workload(name, torch, g, args.steps, args.warmup, args.seed + 1, headline=False)
+            r["timing"] = "best of 3 regions of K launches after 100 ms of warm-up"
             others.append(r)
             del i2, c2
             torch.cuda.empty_cache()

@@ -98,12 +98,10 @@ bool tiled_ok(const a8w8_gemm_args* g)
            (long long)((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 31);
 }
 
-// The persistent kernel pipelines two K steps ahead and indexes work items with an int.  The
-// block-scale mode stays on the plain tiled kernel, which is the faster of the two for it
-// (its per-step fp32 rescale leaves no registers for the second fragment set).
+// The persistent kernel pipelines two K steps ahead and indexes work items with an int.
 bool persist_ok(const a8w8_gemm_args* g)
 {
-    return g->scale_mode != A8W8_SCALE_BLOCK_1x128_128x128 && g->k >= 2 * BK &&
+    return g->k >= 2 * BK &&
            (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 30);
 }
 

@@ -250,11 +250,15 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     };
 
     // ---------------------------------------------------------------- prologue
+    // The next step's A fragments and first B fragment are fetched in the shadow of the last MFMA
+    // group; the block-scale mode has no registers to spare for that second set and reads them
+    // when the step begins.
+    constexpr bool PREFETCH_FRAGS = MODE != MODE_BLOCK;
     struct Frags {
         v8i a[TM];
         v8i b0;
     };
-    Frags F[2];
+    Frags F[PREFETCH_FRAGS ? 2 : 1];
     const int my_items = (pp.items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
     const int total_steps = my_items * nk;
 
@@ -273,9 +277,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     __builtin_amdgcn_s_waitcnt(0);
     A8W8_RAW_BARRIER();
     if constexpr (MODE == MODE_MX) fetch_step_scales(cur_batch, m0, n0, 0, 0);
+    if constexpr (PREFETCH_FRAGS) {
 #pragma unroll
-    for (int t = 0; t < TM; ++t) F[0].a[t] = read_frag(0, rd_a, t);
-    F[0].b0 = read_frag(0, rd_b, 0);
+        for (int t = 0; t < TM; ++t) F[0].a[t] = read_frag(0, rd_a, t);
+        F[0].b0 = read_frag(0, rd_b, 0);
+    }
     zero_acc();
 
     // ---------------------------------------------------------------- one K step
@@ -284,9 +290,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     // the position advances after group 2.
     auto step = [&](auto parity) __attribute__((always_inline)) {
         constexpr int P = decltype(parity)::value;
-        Frags& cur = F[P];
-        Frags& nxt = F[P ^ 1];
+        Frags& cur = F[PREFETCH_FRAGS ? P : 0];
+        Frags& nxt = F[PREFETCH_FRAGS ? P ^ 1 : 0];
         rotate_step_scales();
+        if constexpr (!PREFETCH_FRAGS) {
+#pragma unroll
+            for (int t = 0; t < TM; ++t) cur.a[t] = read_frag(P, rd_a, t);
+            cur.b0 = read_frag(P, rd_b, 0);
+        }
         // where the next step lives (it may be the first step of this workgroup's next tile)
         const bool last_of_tile = cur_ks + 1 == nk;
         int nx_batch = cur_batch, nx_m0 = m0, nx_n0 = n0, nx_gbase = cur_gbase;
@@ -303,6 +314,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
 
         v8i fb[TN];
         fb[0] = cur.b0;
+        // block scales: acc += part * scale trails the MFMA that made `part` by BLK_LAG tiles
+        constexpr int BLK_LAG = 4;
+        v4f part[BLK_LAG + 1];
+        (void)part;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             if (j + 1 < TN) fb[j + 1] = read_frag(P, rd_b, j + 1);
@@ -313,9 +328,20 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], cur.a[i], acc[i][j], 0, 0, 0,
                                                                                  mx_sb[j], 0, mx_sa[i]);
                 } else if constexpr (MODE == MODE_BLOCK) {
-                    const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    const int t = j * TM + i;
+                    part[t % (BLK_LAG + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                         fb[j], cur.a[i], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                    acc[i][j] += part * blk_s[i];
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (t >= BLK_LAG) {
+                        const int u = t - BLK_LAG;
+                        acc[u % TM][u / TM] += part[u % (BLK_LAG + 1)] * blk_s[u % TM];
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (t == TM * TN - 1) {
+#pragma unroll
+                        for (int u = TM * TN - BLK_LAG; u < TM * TN; ++u)
+                            acc[u % TM][u / TM] += part[u % (BLK_LAG + 1)] * blk_s[u % TM];
+                    }
                 } else {
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], cur.a[i], acc[i][j], 0, 0, 0,
                                                                                  0, 0, 0);
@@ -343,9 +369,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                 issue_one(P, ld_ks, 3);
                 __builtin_amdgcn_s_waitcnt(0x0074);   // vmcnt(4) lgkmcnt(0): the next stage has landed
                 A8W8_RAW_BARRIER();                   // end: all of stage P is free
+                if constexpr (PREFETCH_FRAGS) {
 #pragma unroll
-                for (int t = 0; t < TM; ++t) nxt.a[t] = read_frag(P ^ 1, rd_a, t);
-                nxt.b0 = read_frag(P ^ 1, rd_b, 0);
+                    for (int t = 0; t < TM; ++t) nxt.a[t] = read_frag(P ^ 1, rd_a, t);
+                    nxt.b0 = read_frag(P ^ 1, rd_b, 0);
+                }
                 if constexpr (MODE == MODE_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
             }
             if (j == 7) {

@@ -201,21 +201,43 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
 #pragma unroll
         for (int t = 0; t < TM; ++t) fa[t] = read_frag(cur, rd_a, t);
         fb[0] = read_frag(cur, rd_b, 0);
+        if constexpr (MODE == MODE_BLOCK) {
+            // Each 128-wide K step yields a partial tile that is rescaled into the running sum:
+            // acc += part * (sfa * sfb).  The multiply-adds trail the MFMAs by BLK_LAG tiles so
+            // that they never wait on a matrix-core result that is still in flight.
+#ifndef A8W8_BLK_LAG
+#define A8W8_BLK_LAG 4
+#endif
+            constexpr int BLK_LAG = A8W8_BLK_LAG;
+            v4f part[BLK_LAG + 1];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            if (j + 1 < TN) fb[(j + 1) & 1] = read_frag(cur, rd_b, j + 1);
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                if constexpr (MODE == MODE_MX) {
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        fb[j & 1], fa[i], acc[i][j], 0, 0, 0, mx_sb[j], 0, mx_sa[i]);
-                } else if constexpr (MODE == MODE_BLOCK) {
-                    const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+            for (int t = 0; t < TM * TN + BLK_LAG; ++t) {
+                if (t < TM * TN) {
+                    const int j = t / TM, i = t % TM;
+                    if (i == 0 && j + 1 < TN) fb[(j + 1) & 1] = read_frag(cur, rd_b, j + 1);
+                    part[t % (BLK_LAG + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                         fb[j & 1], fa[i], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                    acc[i][j] += part * blk_sa[i];
-                } else {
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        fb[j & 1], fa[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);   // keep the lag: the scheduler would pull the FMAs up
+                if (t >= BLK_LAG) {
+                    const int u = t - BLK_LAG;
+                    acc[u % TM][u / TM] += part[u % (BLK_LAG + 1)] * blk_sa[u % TM];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                if (j + 1 < TN) fb[(j + 1) & 1] = read_frag(cur, rd_b, j + 1);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    if constexpr (MODE == MODE_MX) {
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                            fb[j & 1], fa[i], acc[i][j], 0, 0, 0, mx_sb[j], 0, mx_sa[i]);
+                    } else {
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                            fb[j & 1], fa[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+                    }
                 }
             }
         }

@@ -74,7 +74,7 @@ def test_flatmm_preconditions():
 
 
 def test_kernel_selection():
-    assert g.kernel_name(_ok_args()) == "gemm_a8w8_tile256"                  # block scales: plain tiled kernel
+    assert g.kernel_name(_ok_args()) == "gemm_a8w8_persist"
     assert g.kernel_name(_ok_args(mode=g.MX)) == "gemm_a8w8_persist"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL)) == "gemm_a8w8_persist"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=128)) == "gemm_a8w8_tile256"
