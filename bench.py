@@ -23,6 +23,9 @@ sys.path.insert(0, ROOT)
 METRIC = "FP8 GEMM TFLOPS & % gfx950 FP8 MFMA peak; HBM GB/s for M=16 flatmm"
 PEAK_FP8_TFLOPS = 5000.0      # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E, published
+# Bytes that crossed the L2 <-> fabric boundary per launch, from two rocprofv3 --pmc runs of this file
+# (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 117 MB device copy calibrates; profiles/).
+MEASURED_TRAFFIC = {"mxfp8_8192": 1.10e9, "flatmm_16x16384x7168": 1.190e8}
 
 WORKLOADS = {
     # name: (mode, m, n, k, algorithmic bytes per launch)
@@ -213,11 +216,12 @@ def main():
     if mode == "flat":
         value, unit = res["gbs"], "GB/s"
         roof = {"bound": "hbm", "achieved": res["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": res["gbs"] / PEAK_HBM_GBS, "traffic": None, "kernel": "flatmm_a8w8"}
+                "frac": res["gbs"] / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC.get(args.workload), "kernel": "flatmm_a8w8"}
     else:
         value, unit = res["tflops"], "TFLOP/s"
         roof = {"bound": "mfma", "achieved": res["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                "frac": res["tflops"] / PEAK_FP8_TFLOPS, "traffic": None, "kernel": res.get("kernel")}
+                "frac": res["tflops"] / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC.get(args.workload),
+                "kernel": res.get("kernel")}
     line = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": res["ms_per_launch"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
