@@ -2,7 +2,7 @@
 //
 // Tile 256 x 256 x 128, 8 waves (4 along M x 2 along N), wave tile 64 x 128 = 4 x 8 MFMA
 // tiles of 16 x 16 x 128, operands staged global -> LDS with 16-byte direct-to-LDS loads,
-// two LDS stages of 64 KiB, rows XOR-swizzled with (row & 7) exactly as in gemm_tile.hpp.
+// two LDS stages of 64 KiB, 128-byte rows whose 16-byte slots are XOR-swizzled (see swz_key below).
 //
 // What differs from the plain kernel:
 //  * One workgroup per CU walks a list of tiles; the K loop runs continuously across tile
@@ -31,6 +31,9 @@ constexpr int PERSIST_LDS_BYTES = GEMM_LDS_BYTES;
 constexpr int PERSIST_LDS_BYTES_MX = GEMM_LDS_BYTES_MX;
 
 #define A8W8_RAW_BARRIER() asm volatile("s_barrier" ::: "memory")
+#ifndef A8W8_PREFETCH_FRAGS
+#define A8W8_PREFETCH_FRAGS(mode) ((mode) == MODE_TENSOR)
+#endif
 #ifndef A8W8_PERSIST_SB
 #define A8W8_PERSIST_SB 0
 #endif
@@ -67,7 +70,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_sf;
     int voff_a[4], voff_b[4], voff_sf = 0;
     const int ld_row = wave * 8 + (lane >> 3);
-    const int ld_piece = (lane & 7) ^ (lane >> 3);
+    // lane i of a 1 KiB chunk lands on row (i>>3), slot (i&7) of the chunk's 8 rows; the slot holds
+    // K-piece slot ^ key(row) with key(row) = (row & 7) ^ (((row >> 3) & 3) << 1), and bits 3-4 of the
+    // tile row are (chunk & 3) = (wave & 3) for every chunk this wave fills
+    const int ld_piece = (lane & 7) ^ (((lane >> 3) ^ ((wave & 3) << 1)) & 7);
     auto point_loads_at = [&](int item) __attribute__((always_inline)) {
         item = min(item, pp.items - 1);            // past the end: keep loading valid data nobody reads
         const int batch = item / tiles;
@@ -121,21 +127,37 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     };
 
     // ---------------------------------------------------------------- compute side state
-    int rd_a[2], rd_b[2];
+    // LDS rows of the operands.  A: MFMA tile t, operand row r16 <- tile row 16t + r16.  B: the rows
+    // of each 32-row group are dealt to a tile pair so that a lane ends up with eight consecutive n
+    // (one 16-byte bf16 store, 64 contiguous bytes per C row and instruction):
+    //     tile j, operand row 4g' + i  <-  row 32*(j/2) + 8g' + 4*(j%2) + i.
+    // The swizzle key (row & 7) ^ (((row >> 3) & 3) << 1) keeps both read patterns free of LDS bank
+    // conflicts (measured).  Only the tile's parity enters the key, the rest is an immediate offset.
+    auto swz_key = [](int row) __attribute__((always_inline)) { return ((row & 7) ^ (((row >> 3) & 3) << 1)) & 7; };
+    int rd_a[2][2], rd_b[2][2];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int slot = (g + 4 * h) ^ (lane & 7);
-        rd_a[h] = (wave_m * WAVE_M + r16) * BK + (slot << 4);
-        rd_b[h] = BM * BK + (wave_n * WAVE_N + r16) * BK + (slot << 4);
-    }
-    auto read_frag = [&](int stage, const int (&base)[2], int t) -> v8i {
-        const char* s = smem + stage * STAGE_BYTES + t * (16 * BK);
+    for (int par = 0; par < 2; ++par)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int row_a = 16 * par + r16;
+            const int row_b = 8 * (r16 >> 2) + 4 * par + (r16 & 3);
+            rd_a[par][h] = (wave_m * WAVE_M + row_a) * BK + ((((g + 4 * h) ^ swz_key(row_a)) & 7) << 4);
+            rd_b[par][h] = BM * BK + (wave_n * WAVE_N + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
+        }
+    auto read_frag_at = [&](int stage, const int (&base)[2], int byte_off) __attribute__((always_inline)) -> v8i {
+        const char* s = smem + stage * STAGE_BYTES + byte_off;
         const v4i lo = *(const v4i*)(s + base[0]);
         const v4i hi = *(const v4i*)(s + base[1]);
         return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     };
+    auto read_frag_a = [&](int stage, int t) __attribute__((always_inline)) -> v8i {
+        return read_frag_at(stage, rd_a[t & 1], (t >> 1) * (32 * BK));
+    };
+    auto read_frag_b = [&](int stage, int j) __attribute__((always_inline)) -> v8i {
+        return read_frag_at(stage, rd_b[j & 1], (j >> 1) * (32 * BK));
+    };
     const int rd_sfa = GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16;
-    const int rd_sfb = GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + r16) * 16;
+    const int rd_sfb = GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + 8 * (r16 >> 2) + (r16 & 3)) * 16;
 
     int cur_item = blockIdx.x, cur_ks = 0;         // the step being multiplied
     int cur_batch = 0, m0 = 0, n0 = 0;
@@ -179,7 +201,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                 mx_sa_next[t] = *(const int*)(s + rd_sfa + t * 256);
 #pragma unroll
             for (int t = 0; t < TN; ++t)
-                mx_sb_next[t] = *(const int*)(s + rd_sfb + t * 256);
+                mx_sb_next[t] = *(const int*)(s + rd_sfb + (t >> 1) * 512 + (t & 1) * 64);
         }
     };
     auto rotate_step_scales = [&]() __attribute__((always_inline)) {
@@ -200,7 +222,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         const float* sfa_f = (const float*)p.sfa + (long long)cur_batch * p.sfa_batch;
         const float* sfb_f = (const float*)p.sfb + (long long)cur_batch * p.sfb_batch;
         const int cm_base = m0 + wave_m * WAVE_M + r16;
-        const int cn_base = n0 + wave_n * WAVE_N + 4 * g;
+        const int cn_base = n0 + wave_n * WAVE_N + 8 * g;      // + 32 * (tile pair): eight consecutive n
         float sa[TM];
         float ts = 1.f;
         if constexpr (MODE == MODE_TENSOR) ts = sfa_f[0] * sfb_f[0];
@@ -209,39 +231,63 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             for (int i = 0; i < TM; ++i) sa[i] = sfa_f[min(cm_base + 16 * i, p.m - 1)];
         }
         char* c_base = (char*)p.c + (long long)cur_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
-        const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 7) == 0)
+        const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 7) == 0 && (((uintptr_t)c_base) & 15) == 0)
                                             : ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 15) == 0);
+        // every scale is fetched before the first store: a wait for a load issued after a store would
+        // also wait for that store to be acknowledged (one counter, in issue order)
+        float sb[TN / 2][8];
+        if constexpr (MODE == MODE_ROWCOL) {
+            const bool sfb_vec = (((uintptr_t)sfb_f) & 15) == 0;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int cn = cn_base + 16 * j;
-            v4f sb = v4f{1.f, 1.f, 1.f, 1.f};
-            if constexpr (MODE == MODE_ROWCOL) {
+            for (int jp = 0; jp < TN / 2; ++jp) {
+                const int cn = cn_base + 32 * jp;
+                if (sfb_vec && cn + 7 < p.n) {
+                    const v4f lo = *(const v4f*)(sfb_f + cn), hi = *(const v4f*)(sfb_f + cn + 4);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) sb[e] = sfb_f[min(cn + e, p.n - 1)];
+                    for (int e = 0; e < 4; ++e) { sb[jp][e] = lo[e]; sb[jp][4 + e] = hi[e]; }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sb[jp][e] = sfb_f[min(cn + e, p.n - 1)];
+                }
             }
+        }
+        // ... and waited for here, once, so that no wait ends up between the stores
+        if constexpr (MODE == MODE_ROWCOL) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+#pragma unroll
+        for (int jp = 0; jp < TN / 2; ++jp) {
+            const int cn = cn_base + 32 * jp;
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 const int cm = cm_base + 16 * i;
-                v4f v = acc[i][j];
-                if constexpr (MODE == MODE_TENSOR) v *= ts;
-                if constexpr (MODE == MODE_ROWCOL) v *= sb * sa[i];
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    v[e] = acc[i][2 * jp + (e >> 2)][e & 3];
+                    if constexpr (MODE == MODE_TENSOR) v[e] *= ts;
+                    if constexpr (MODE == MODE_ROWCOL) v[e] *= sb[jp][e] * sa[i];
+                }
                 if (cm >= p.m) continue;
                 if constexpr (CDT == C_BF16) {
                     unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
-                    if (vec_ok && cn + 3 < p.n) {
-                        A8W8_STORE_C((v4u16*)dst, (v4u16{bf16_bits(v.x), bf16_bits(v.y), bf16_bits(v.z), bf16_bits(v.w)}));
-                    } else {
+                    if (vec_ok && cn + 7 < p.n) {
+                        v4i w;
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
+                            w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+                        A8W8_STORE_C((v4i*)dst, w);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
                             if (cn + e < p.n) dst[e] = bf16_bits(v[e]);
                     }
                 } else {
                     float* dst = (float*)c_base + (long long)cm * p.ldc + cn;
-                    if (vec_ok && cn + 3 < p.n) {
-                        A8W8_STORE_C((v4f*)dst, v);
+                    if (vec_ok && cn + 7 < p.n) {
+                        A8W8_STORE_C((v4f*)dst, (v4f{v[0], v[1], v[2], v[3]}));
+                        A8W8_STORE_C((v4f*)(dst + 4), (v4f{v[4], v[5], v[6], v[7]}));
                     } else {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
+                        for (int e = 0; e < 8; ++e)
                             if (cn + e < p.n) dst[e] = v[e];
                     }
                 }
@@ -253,7 +299,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     // The next step's A fragments and first B fragment are fetched in the shadow of the last MFMA
     // group; the block-scale mode has no registers to spare for that second set and reads them
     // when the step begins.
-    constexpr bool PREFETCH_FRAGS = MODE != MODE_BLOCK;
+    constexpr bool PREFETCH_FRAGS = A8W8_PREFETCH_FRAGS(MODE);
     struct Frags {
         v8i a[TM];
         v8i b0;
@@ -279,8 +325,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     if constexpr (MODE == MODE_MX) fetch_step_scales(cur_batch, m0, n0, 0, 0);
     if constexpr (PREFETCH_FRAGS) {
 #pragma unroll
-        for (int t = 0; t < TM; ++t) F[0].a[t] = read_frag(0, rd_a, t);
-        F[0].b0 = read_frag(0, rd_b, 0);
+        for (int t = 0; t < TM; ++t) F[0].a[t] = read_frag_a(0, t);
+        F[0].b0 = read_frag_b(0, 0);
     }
     zero_acc();
 
@@ -295,8 +341,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         rotate_step_scales();
         if constexpr (!PREFETCH_FRAGS) {
 #pragma unroll
-            for (int t = 0; t < TM; ++t) cur.a[t] = read_frag(P, rd_a, t);
-            cur.b0 = read_frag(P, rd_b, 0);
+            for (int t = 0; t < TM; ++t) cur.a[t] = read_frag_a(P, t);
+            cur.b0 = read_frag_b(P, 0);
         }
         // where the next step lives (it may be the first step of this workgroup's next tile)
         const bool last_of_tile = cur_ks + 1 == nk;
@@ -320,7 +366,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         (void)part;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            if (j + 1 < TN) fb[j + 1] = read_frag(P, rd_b, j + 1);
+            if (j + 1 < TN) fb[j + 1] = read_frag_b(P, j + 1);
             A8W8_PERSIST_SCHED_BARRIER();
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
@@ -371,8 +417,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                 A8W8_RAW_BARRIER();                   // end: all of stage P is free
                 if constexpr (PREFETCH_FRAGS) {
 #pragma unroll
-                    for (int t = 0; t < TM; ++t) nxt.a[t] = read_frag(P ^ 1, rd_a, t);
-                    nxt.b0 = read_frag(P ^ 1, rd_b, 0);
+                    for (int t = 0; t < TM; ++t) nxt.a[t] = read_frag_a(P ^ 1, t);
+                    nxt.b0 = read_frag_b(P ^ 1, 0);
                 }
                 if constexpr (MODE == MODE_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
             }
