@@ -44,11 +44,12 @@ int validate_common(const a8w8_gemm_args* g)
     if (!g) return A8W8_ERR_NULL_POINTER;
     if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
     if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0) return A8W8_ERR_BAD_SHAPE;
-    if (g->scale_mode < 0 || g->scale_mode > 3) return A8W8_ERR_BAD_MODE;
+    if (g->scale_mode < 0 || g->scale_mode > A8W8_SCALE_MX_E8M0_TILED) return A8W8_ERR_BAD_MODE;
     if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
     if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128 && (g->n % 128 != 0 || g->k % 128 != 0))
         return A8W8_ERR_BAD_GROUP;
-    if (g->scale_mode == A8W8_SCALE_MX_E8M0_1x32 && g->k % 32 != 0) return A8W8_ERR_BAD_GROUP;
+    if ((g->scale_mode == A8W8_SCALE_MX_E8M0_1x32 || g->scale_mode == A8W8_SCALE_MX_E8M0_TILED) && g->k % 32 != 0)
+        return A8W8_ERR_BAD_GROUP;
     if (g->stride_c < g->n) return A8W8_ERR_BAD_STRIDE;
     if (g->stride_a < g->k) return A8W8_ERR_BAD_STRIDE;
     if (!g->b_preshuffled && g->stride_b < g->k) return A8W8_ERR_BAD_STRIDE;
@@ -93,6 +94,10 @@ bool tiled_ok(const a8w8_gemm_args* g)
         (g->stride_sfa % 4 != 0 || g->stride_sfb % 4 != 0 || ((uintptr_t)g->sfa & 3) || ((uintptr_t)g->sfb & 3) ||
          (g->batch > 1 && (g->stride_sfa_batch % 4 != 0 || g->stride_sfb_batch % 4 != 0))))
         return false;
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED &&
+        (!aligned16(g->sfa) || !aligned16(g->sfb) ||
+         (g->batch > 1 && (g->stride_sfa_batch % 16 != 0 || g->stride_sfb_batch % 16 != 0))))
+        return false;
     return g->k % BK == 0 && g->stride_a % 16 == 0 && g->stride_b % 16 == 0 && aligned16(g->a) && aligned16(g->b) &&
            (g->batch == 1 || (g->stride_a_batch % 16 == 0 && g->stride_b_batch % 16 == 0)) &&
            (long long)((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 31);
@@ -106,11 +111,16 @@ bool persist_ok(const a8w8_gemm_args* g)
 }
 
 template <int MODE, int CDT>
+int launch_general(const GemmParams& p, int batch, hipStream_t stream);
+
+template <int MODE, int CDT>
 int launch_tiled(const GemmParams& p, int batch, hipStream_t stream)
 {
     static bool attr_set[64];
     int dev = 0;
     (void)hipGetDevice(&dev);
+    if constexpr (MODE == MODE_MXT) return launch_general<MODE, CDT>(p, batch, stream);   // single K step: rare
+    else {
     auto kern = gemm_a8w8_tile256<MODE, CDT>;
     constexpr int lds_bytes = MODE == MODE_MX ? GEMM_LDS_BYTES_MX : GEMM_LDS_BYTES;
     if (!attr_set[dev & 63]) {
@@ -121,6 +131,7 @@ int launch_tiled(const GemmParams& p, int batch, hipStream_t stream)
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch);
     hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), lds_bytes, stream, p);
     return launch_status();
+    }
 }
 
 // Persistent pipelined kernel: one workgroup per CU walks the (batch, tile) list.
@@ -131,7 +142,7 @@ int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
     int dev = 0;
     (void)hipGetDevice(&dev);
     auto kern = gemm_a8w8_persist<MODE, CDT>;
-    constexpr int lds_bytes = MODE == MODE_MX ? PERSIST_LDS_BYTES_MX : PERSIST_LDS_BYTES;
+    constexpr int lds_bytes = (MODE == MODE_MX || MODE == MODE_MXT) ? PERSIST_LDS_BYTES_MX : PERSIST_LDS_BYTES;
     if (!attr_set[dev & 63]) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
             return A8W8_ERR_LAUNCH;
@@ -166,6 +177,8 @@ int launch_general(const GemmParams& p, int batch, hipStream_t stream)
         case 5: return FN<MODE_BLOCK, C_FP32>(__VA_ARGS__);                                 \
         case 6: return FN<MODE_MX, C_BF16>(__VA_ARGS__);                                    \
         case 7: return FN<MODE_MX, C_FP32>(__VA_ARGS__);                                    \
+        case 8: return FN<MODE_MXT, C_BF16>(__VA_ARGS__);                                   \
+        case 9: return FN<MODE_MXT, C_FP32>(__VA_ARGS__);                                   \
         default: return A8W8_ERR_BAD_MODE;                                                  \
     }
 
@@ -349,13 +362,45 @@ int a8w8_quantize(const float* src, int rows, int k, int ld, uint8_t* q, void* s
             if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
             if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
             const long long threads = (long long)rows * k;
-            hipLaunchKernelGGL(quant_mx_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k,
+            hipLaunchKernelGGL(quant_mx_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k,
                                ld, q, (uint8_t*)scale);
+            return launch_status();
+        }
+        case A8W8_SCALE_MX_E8M0_TILED: {
+            if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
+            if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+            const long long threads = (long long)rows * k;
+            const int pad_blocks = ((k + 511) / 512) * 16 - k / 32;   // blocks of the last, partial K group
+            if (pad_blocks > 0)
+                hipLaunchKernelGGL(mx_tiled_pad_kernel, dim3((unsigned)(((long long)rows * pad_blocks + 255) / 256)),
+                                   dim3(256), 0, s, (uint8_t*)scale, rows, k);
+            hipLaunchKernelGGL(quant_mx_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows,
+                               k, ld, q, (uint8_t*)scale);
             return launch_status();
         }
         default:
             return A8W8_ERR_BAD_MODE;
     }
+}
+
+int a8w8_mx_tile_scales(const uint8_t* sf, int rows, int k, int stride, uint8_t* out, void* hip_stream)
+{
+    if (!sf || !out) return A8W8_ERR_NULL_POINTER;
+    if (rows <= 0 || k <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
+    if (stride < k / 32) return A8W8_ERR_BAD_STRIDE;
+    if (!aligned16(out)) return A8W8_ERR_MISALIGNED;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    const long long units = (long long)rows * ((k + 511) / 512);
+    hipLaunchKernelGGL(mx_tile_scales_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)hip_stream, sf, rows, k, stride, out);
+    return launch_status();
+}
+
+size_t a8w8_mx_tiled_bytes(int rows, int k)
+{
+    if (rows <= 0 || k <= 0) return 0;
+    return (size_t)rows * 16 * (size_t)((k + 511) / 512);
 }
 
 const char* a8w8_status_string(int status)
@@ -381,9 +426,10 @@ const char* a8w8_kernel_name(const a8w8_gemm_args* g)
     if (g->b_preshuffled) return validate_flat(g) == A8W8_OK ? "flatmm_a8w8" : nullptr;
     if (validate_common(g) != A8W8_OK) return nullptr;
     if (!tiled_ok(g)) return "gemm_a8w8_general";
-    return persist_ok(g) ? "gemm_a8w8_persist" : "gemm_a8w8_tile256";
+    if (persist_ok(g)) return "gemm_a8w8_persist";
+    return g->scale_mode == A8W8_SCALE_MX_E8M0_TILED ? "gemm_a8w8_general" : "gemm_a8w8_tile256";
 }
 
-int a8w8_version(void) { return 100; }
+int a8w8_version(void) { return 200; }
 
 }  // extern "C"

@@ -14,7 +14,16 @@ typedef unsigned short v4u16 __attribute__((ext_vector_type(4)));
 #define A8W8_DEV __device__ __forceinline__
 #define A8W8_LDS __attribute__((address_space(3)))
 
-enum : int { MODE_TENSOR = 0, MODE_ROWCOL = 1, MODE_BLOCK = 2, MODE_MX = 3 };
+enum : int { MODE_TENSOR = 0, MODE_ROWCOL = 1, MODE_BLOCK = 2, MODE_MX = 3, MODE_MXT = 4 };
+
+// Byte position of the E8M0 exponent of (row, 32-wide K block kblk) in the tiled MX scale layout:
+// [K/512][rows][4 blocks of a 128-wide K step][4 consecutive K steps].  One 16-byte unit holds the
+// sixteen exponents of a row for 512 K elements, transposed so that the four steps of one block
+// position share a dword (the dword a lane of the scaled MFMA keeps for four K steps).
+__host__ __device__ inline size_t mx_tiled_index(int rows, int row, int kblk)
+{
+    return ((size_t)(kblk >> 4) * rows + row) * 16 + (kblk & 3) * 4 + ((kblk >> 2) & 3);
+}
 enum : int { C_BF16 = 0, C_FP32 = 1 };
 
 // Kernel parameters of the dense and flat GEMMs (strides in elements, as in the ABI).

@@ -191,6 +191,7 @@ __global__ void __launch_bounds__(256) quant_128x128_kernel(const float* src, in
 
 // MX: one E8M0 exponent per 32 K-elements, e = ceil(log2(amax/448)) clamped to [-127, 127]
 // computed exactly from the fp32 exponent/mantissa fields; 32 lanes per block.
+template <bool TILED>
 __global__ void __launch_bounds__(256) quant_mx_kernel(const float* src, int rows, int k, int ld, uint8_t* q,
                                                        uint8_t* scale)
 {
@@ -211,10 +212,45 @@ __global__ void __launch_bounds__(256) quant_mx_kernel(const float* src, int row
         e = (f == 0.5f) ? ex - 1 : ex;
         e = max(-127, min(127, e));
     }
-    if (l == 0) scale[(long long)row * blocks + g] = (uint8_t)(e + 127);
+    if (l == 0) scale[TILED ? mx_tiled_index(rows, row, g) : (size_t)row * blocks + g] = (uint8_t)(e + 127);
     const float qv = ldexpf(v, -e);
     const uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(qv, qv, 0, false);
     q[(long long)row * k + g * 32 + l] = (uint8_t)w;
+}
+
+// natural [rows][k/32] E8M0 scales (row stride `stride` bytes) -> the tiled layout of mx_tiled_index.
+// One thread per 16-byte unit (row, 512-wide K group); consecutive threads take consecutive rows,
+// so the writes are contiguous.  Blocks past k get 127 (scale 1.0; their products are never formed).
+__global__ void __launch_bounds__(256) mx_tile_scales_kernel(const uint8_t* sf, int rows, int k, int stride,
+                                                             uint8_t* out)
+{
+    const long long u = (long long)blockIdx.x * 256 + threadIdx.x;
+    const int groups = (k + 511) >> 9, blocks = k >> 5;
+    if (u >= (long long)rows * groups) return;
+    const int row = (int)(u % rows), kg = (int)(u / rows);
+    const uint8_t* src = sf + (size_t)row * stride + kg * 16;
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int kblk = kg * 16 + s * 4 + g;
+            const uint32_t e = kblk < blocks ? src[s * 4 + g] : 127u;
+            w[g] |= e << (8 * s);
+        }
+    *(v4i*)(out + (size_t)u * 16) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+}
+
+// 127 into the blocks of the last K group that lie past k (tiled layout), for producers that
+// write only the real blocks.
+__global__ void __launch_bounds__(256) mx_tiled_pad_kernel(uint8_t* scale, int rows, int k)
+{
+    const int blocks = k >> 5, total = ((k + 511) >> 9) * 16;
+    const int pad = total - blocks;
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)rows * pad) return;
+    const int row = (int)(idx % rows), kblk = blocks + (int)(idx / rows);
+    scale[mx_tiled_index(rows, row, kblk)] = 127;
 }
 
 }  // namespace a8w8

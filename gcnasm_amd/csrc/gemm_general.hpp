@@ -31,7 +31,7 @@ __global__ void __launch_bounds__(256) gemm_a8w8_general(GemmParams p)
     const uint8_t* sfa_e = (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
     const uint8_t* sfb_e = (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch;
 
-    const int group_k = MODE == MODE_BLOCK ? 128 : (MODE == MODE_MX ? 32 : p.k);
+    const int group_k = MODE == MODE_BLOCK ? 128 : ((MODE == MODE_MX || MODE == MODE_MXT) ? 32 : p.k);
     float sum = 0.f;
     for (int k0 = 0; k0 < p.k; k0 += group_k) {
         const int g = k0 / group_k;
@@ -42,6 +42,8 @@ __global__ void __launch_bounds__(256) gemm_a8w8_general(GemmParams p)
             scale = sfa_f[(long long)g * p.stride_sfa + i] * sfb_f[(long long)(j >> 7) * p.stride_sfb + g];
         if constexpr (MODE == MODE_MX)
             scale = e8m0_pair_scale(sfa_e[(long long)i * p.stride_sfa + g], sfb_e[(long long)j * p.stride_sfb + g]);
+        if constexpr (MODE == MODE_MXT)
+            scale = e8m0_pair_scale(sfa_e[mx_tiled_index(p.m, i, g)], sfb_e[mx_tiled_index(p.n, j, g)]);
         const int k1 = min(k0 + group_k, p.k);
         for (int k = k0; k < k1; ++k) {
             const float prod = e4m3_to_f32_hw(a[k]) * e4m3_to_f32_hw(b[k]);

@@ -58,6 +58,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     const int lane = tid & 63;
     const int wave = wave_uniform(tid >> 6);
     const int wave_m = wave >> 1, wave_n = wave & 1;
+    constexpr bool IS_MX = MODE == MODE_MX || MODE == MODE_MXT;
     const int r16 = lane & 15, g = lane >> 4;
     const int nk = p.k / BK;                       // >= 2 (checked by the host)
     const int tiles = p.tiles_m * p.tiles_n;
@@ -69,6 +70,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     int ld_gbase = 0, cur_gbase = 0;                // running group count: picks the scale buffer
     __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_sf;
     int voff_a[4], voff_b[4], voff_sf = 0;
+    int sf_group_stride = 16;                       // bytes from one scale group of a row set to the next
     const int ld_row = wave * 8 + (lane >> 3);
     // lane i of a 1 KiB chunk lands on row (i>>3), slot (i&7) of the chunk's 8 rows; the slot holds
     // K-piece slot ^ key(row) with key(row) = (row & 7) ^ (((row >> 3) & 3) << 1), and bits 3-4 of the
@@ -96,6 +98,21 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             rsrc_sf = make_rsrc(base, (uint32_t)(rows - 1) * stride + (uint32_t)(p.k >> 5));
             voff_sf = min((is_b ? n0 : m0) + (wave & 3) * 64 + lane, rows - 1) * stride;
         }
+        if constexpr (MODE == MODE_MXT) {
+            // tiled scales: the 16-byte units of 64 rows of a group are contiguous in memory, so one
+            // load instruction reads eight whole cache lines.  LDS slot (wave & 3) * 64 + lane takes
+            // tile row `slot` for A; for B the rows are dealt as the MFMA tiles read them (slot
+            // 16 j + r16 holds the row that lane r16 supplies to tile j).
+            const bool is_b = wave >= 4;
+            const int rows = is_b ? p.n : p.m;
+            const uint8_t* base = is_b ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
+                                       : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
+            rsrc_sf = make_rsrc(base, (uint32_t)rows * 16u * (uint32_t)((p.k + 511) >> 9));
+            const int slot = (wave & 3) * 64 + lane;
+            const int trow = is_b ? ((slot & ~31) | (((slot >> 2) & 3) << 3) | (((slot >> 4) & 1) << 2) | (slot & 3)) : slot;
+            voff_sf = min((is_b ? n0 : m0) + trow, rows - 1) * 16;
+            sf_group_stride = wave_uniform(rows * 16);
+        }
     };
     // one of the eight loads of a stage: 0..3 = A chunks, 4,5 = low B chunks, 6,7 = high B chunks.
     // Wave w fills rows 8w + 64j (+0..7) of each matrix; for B, j = 0, 2 are the rows of MFMA
@@ -111,10 +128,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         }
     };
     auto issue_mx_group = [&](int group) __attribute__((always_inline)) {
-        if constexpr (MODE == MODE_MX) {
+        if constexpr (IS_MX) {
             A8W8_LDS char* s =
                 (A8W8_LDS char*)smem + GEMM_LDS_BYTES + ((ld_gbase + group) & 1) * MX_GROUP_BYTES + wave * 1024;
-            load_to_lds_16(rsrc_sf, s, voff_sf, group * 16);
+            load_to_lds_16(rsrc_sf, s, voff_sf, group * sf_group_stride);
         }
     };
     auto advance_ld = [&]() __attribute__((always_inline)) {                      // the load position moves one K step
@@ -156,8 +173,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     auto read_frag_b = [&](int stage, int j) __attribute__((always_inline)) -> v8i {
         return read_frag_at(stage, rd_b[j & 1], (j >> 1) * (32 * BK));
     };
-    const int rd_sfa = GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16;
-    const int rd_sfb = GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + 8 * (r16 >> 2) + (r16 & 3)) * 16;
+    // natural MX scales: B tile t at + (t >> 1) * 512 + (t & 1) * 64; tiled: tile t at + t * 256, dword g
+    const int rd_sfa = GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16 + (MODE == MODE_MXT ? 4 * g : 0);
+    const int rd_sfb = MODE == MODE_MXT
+                           ? GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + r16) * 16 + 4 * g
+                           : GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + 8 * (r16 >> 2) + (r16 & 3)) * 16;
 
     int cur_item = blockIdx.x, cur_ks = 0;         // the step being multiplied
     int cur_batch = 0, m0 = 0, n0 = 0;
@@ -203,6 +223,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             for (int t = 0; t < TN; ++t)
                 mx_sb_next[t] = *(const int*)(s + rd_sfb + (t >> 1) * 512 + (t & 1) * 64);
         }
+        if constexpr (MODE == MODE_MXT) {
+            // the dword of (row, block position g) holds the exponents of the group's four K steps
+            const char* s = smem + ((gbase + (kstep >> 2)) & 1) * MX_GROUP_BYTES;
+#pragma unroll
+            for (int t = 0; t < TM; ++t) mx_sa_next[t] = *(const int*)(s + rd_sfa + t * 256);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) mx_sb_next[t] = *(const int*)(s + rd_sfb + t * 256);
+        }
     };
     auto rotate_step_scales = [&]() __attribute__((always_inline)) {
         if constexpr (MODE == MODE_BLOCK) {
@@ -214,6 +242,13 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             for (int t = 0; t < TM; ++t) mx_sa[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sa_next[t], 8 * g, 8);
 #pragma unroll
             for (int t = 0; t < TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sb_next[t], 8 * g, 8);
+        }
+        if constexpr (MODE == MODE_MXT) {
+            const int sh = (cur_ks & 3) * 8;
+#pragma unroll
+            for (int t = 0; t < TM; ++t) mx_sa[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sa_next[t], sh, 8);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sb_next[t], sh, 8);
         }
     };
 
@@ -322,7 +357,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     if constexpr (MODE == MODE_BLOCK) fetch_step_scales(cur_batch, m0, n0, 0, 0);
     __builtin_amdgcn_s_waitcnt(0);
     A8W8_RAW_BARRIER();
-    if constexpr (MODE == MODE_MX) fetch_step_scales(cur_batch, m0, n0, 0, 0);
+    if constexpr (IS_MX) fetch_step_scales(cur_batch, m0, n0, 0, 0);
     if constexpr (PREFETCH_FRAGS) {
 #pragma unroll
         for (int t = 0; t < TM; ++t) F[0].a[t] = read_frag_a(0, t);
@@ -370,7 +405,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             A8W8_PERSIST_SCHED_BARRIER();
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                if constexpr (MODE == MODE_MX) {
+                if constexpr (IS_MX) {
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], cur.a[i], acc[i][j], 0, 0, 0,
                                                                                  mx_sb[j], 0, mx_sa[i]);
                 } else if constexpr (MODE == MODE_BLOCK) {
@@ -399,7 +434,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             if (j == 1) issue_one(P ^ 1, ld_ks, 7);
             if (j == 2) {
                 advance_ld();
-                if constexpr (MODE == MODE_MX) {
+                if constexpr (IS_MX) {
                     if ((ld_ks & 3) == 0) issue_mx_group(ld_ks >> 2);   // scales of steps ld_ks .. ld_ks+3
                 }
                 if constexpr (MODE == MODE_BLOCK) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, 0);
@@ -420,7 +455,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                     for (int t = 0; t < TM; ++t) nxt.a[t] = read_frag_a(P ^ 1, t);
                     nxt.b0 = read_frag_b(P ^ 1, 0);
                 }
-                if constexpr (MODE == MODE_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
+                if constexpr (IS_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
             }
             if (j == 7) {
                 issue_one(P, ld_ks, 4);

@@ -44,12 +44,18 @@ typedef enum {
  *             sfa[g*stride_sfa + i]          one scale per 1 x 128 block of A, g = k/128
  *             sfb[(j/128)*stride_sfb + g]    one scale per 128 x 128 block of B
  *   MX      uint8 E8M0 exponents, one per 32 K-elements, value 2^(e-127):
- *             sfa[i*stride_sfa + k/32], sfb[j*stride_sfb + k/32]                        */
+ *             sfa[i*stride_sfa + k/32], sfb[j*stride_sfb + k/32]
+ *   MX_TILED  the same exponents re-arranged by a8w8_mx_tile_scales (or written that way by
+ *             a8w8_quantize) so that the GEMM reads them as whole cache lines:
+ *             sf[((kb/16)*rows + r)*16 + (kb%4)*4 + (kb/4)%4],  kb = k/32, rows = m or n;
+ *             stride_sfa / stride_sfb are ignored, ceil(k/512)*rows*16 bytes each.  With row-major
+ *             scales every 16 bytes the kernel needs sit in a different 128-byte line.       */
 typedef enum {
     A8W8_SCALE_TENSOR = 0,
     A8W8_SCALE_ROWCOL = 1,
     A8W8_SCALE_BLOCK_1x128_128x128 = 2,
-    A8W8_SCALE_MX_E8M0_1x32 = 3
+    A8W8_SCALE_MX_E8M0_1x32 = 3,
+    A8W8_SCALE_MX_E8M0_TILED = 4
 } a8w8_scale_mode;
 
 typedef enum { A8W8_C_BF16 = 0, A8W8_C_FP32 = 1 } a8w8_c_dtype;
@@ -128,10 +134,19 @@ A8W8_API size_t a8w8_cvt_e4m3_to_f32(const uint8_t* src_dev, float* dst_dev, siz
  *   BLOCK : group_rows = 1   -> scale[(p/128)*rows + r]       (the SFA layout)
  *           group_rows = 128 -> scale[(r/128)*(k/128) + p/128] (the SFB layout)
  *   MX    : uint8 e = clamp(ceil(log2(amax32/448)), -127, 127) + 127 at scale[r*(k/32) + p/32]
+ *   MX_TILED : the same bytes at their MX_TILED positions (a8w8_mx_tiled_bytes(rows, k) bytes)
  * TENSOR needs a grid-wide reduction first and is provided as ROWCOL followed by the
  * caller's own max; it returns A8W8_ERR_BAD_MODE here. */
 A8W8_API int a8w8_quantize(const float* src_dev, int rows, int k, int ld, uint8_t* q_dev, void* scale_dev,
                            int scale_mode, int group_rows, void* hip_stream);
+
+/* E8M0 scales, row-major sf[r*stride + k/32] -> the MX_TILED layout, device buffers
+ * (a8w8_mx_tiled_bytes(rows, k) bytes at out, 16-byte aligned).  No counterpart in the
+ * reference, which has no MXFP8 program; weights' scales are converted once, activations'
+ * scales can be produced in this layout directly by a8w8_quantize. */
+A8W8_API int a8w8_mx_tile_scales(const uint8_t* sf_dev, int rows, int k, int stride, uint8_t* out_dev,
+                                 void* hip_stream);
+A8W8_API size_t a8w8_mx_tiled_bytes(int rows, int k);
 
 A8W8_API const char* a8w8_status_string(int status);
 
