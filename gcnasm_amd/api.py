@@ -12,7 +12,7 @@ import subprocess
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libmi355a8w8.so")
 
-TENSOR, ROWCOL, BLOCK, MX = 0, 1, 2, 3
+TENSOR, ROWCOL, BLOCK, MX, MX_TILED = 0, 1, 2, 3, 4
 BF16, FP32 = 0, 1
 OCP, FNUZ = 0, 1
 
@@ -72,6 +72,9 @@ def lib():
         L.a8w8_cvt_e4m3_to_f32.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, vp]
         L.a8w8_quantize.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_int,
                                     ctypes.c_int, vp]
+        L.a8w8_mx_tile_scales.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp]
+        L.a8w8_mx_tiled_bytes.restype = ctypes.c_size_t
+        L.a8w8_mx_tiled_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
         L.a8w8_status_string.restype = ctypes.c_char_p
         L.a8w8_status_string.argtypes = [ctypes.c_int]
         L.a8w8_kernel_name.restype = ctypes.c_char_p
@@ -110,12 +113,19 @@ def raw_gemm_args(a, b, c, sfa, sfb, m, n, k, scale_mode, c_dtype=BF16, batch=1,
         stride_sfb = {TENSOR: 0, ROWCOL: 1, BLOCK: k // 128, MX: k // 32}[scale_mode] if 0 <= scale_mode <= 3 else 0
     g.stride_sfa, g.stride_sfb = stride_sfa, stride_sfb
     if batch_strides is None:
-        sfa_b = {TENSOR: 1, ROWCOL: m, BLOCK: m * (k // 128), MX: m * (k // 32)}.get(scale_mode, 0)
-        sfb_b = {TENSOR: 1, ROWCOL: n, BLOCK: (n // 128) * (k // 128), MX: n * (k // 32)}.get(scale_mode, 0)
+        sfa_b = {TENSOR: 1, ROWCOL: m, BLOCK: m * (k // 128), MX: m * (k // 32),
+                 MX_TILED: mx_tiled_bytes(m, k)}.get(scale_mode, 0)
+        sfb_b = {TENSOR: 1, ROWCOL: n, BLOCK: (n // 128) * (k // 128), MX: n * (k // 32),
+                 MX_TILED: mx_tiled_bytes(n, k)}.get(scale_mode, 0)
         batch_strides = (m * g.stride_a, n * g.stride_b, m * g.stride_c, sfa_b, sfb_b)
     (g.stride_a_batch, g.stride_b_batch, g.stride_c_batch, g.stride_sfa_batch, g.stride_sfb_batch) = batch_strides
     g.scale_mode, g.c_dtype, g.b_preshuffled = scale_mode, c_dtype, b_preshuffled
     return g
+
+
+def mx_tiled_bytes(rows, k):
+    """Size of one matrix's E8M0 scales in the MX_TILED layout."""
+    return ((k + 511) // 512) * ((rows + 63) // 64) * 1024
 
 
 def _out(c, shape, c_dtype, device):
@@ -221,11 +231,24 @@ def quantize(x, scale_mode, group_rows=1):
         s = torch.empty((rows // 128, k // 128), dtype=torch.float32, device=x.device)
     elif scale_mode == MX:
         s = torch.empty((rows, k // 32), dtype=torch.uint8, device=x.device)
+    elif scale_mode == MX_TILED:
+        s = torch.empty(mx_tiled_bytes(rows, k), dtype=torch.uint8, device=x.device)
     else:
         raise A8W8Error(-6, "a8w8_quantize")
     _check(lib().a8w8_quantize(x.data_ptr(), rows, k, x.stride(0), q.data_ptr(), s.data_ptr(), scale_mode, group_rows,
                                _stream()), "a8w8_quantize")
     return q, s
+
+
+def mx_tile_scales(sf, out=None):
+    """Row-major E8M0 scales [rows, K/32] (u8, on the GPU) -> the MX_TILED layout (flat u8 tensor)."""
+    import torch
+    rows, kb = sf.shape
+    if out is None:
+        out = torch.empty(mx_tiled_bytes(rows, kb * 32), dtype=torch.uint8, device=sf.device)
+    _check(lib().a8w8_mx_tile_scales(sf.data_ptr(), rows, kb * 32, sf.stride(0), out.data_ptr(), _stream()),
+           "a8w8_mx_tile_scales")
+    return out
 
 
 def kernel_name(g):

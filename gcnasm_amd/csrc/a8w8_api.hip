@@ -106,6 +106,8 @@ bool tiled_ok(const a8w8_gemm_args* g)
 // The persistent kernel pipelines two K steps ahead and indexes work items with an int.
 bool persist_ok(const a8w8_gemm_args* g)
 {
+    // tiled MX scales come in pairs of K steps (one dword serves two steps)
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED && (g->k / BK) % 2 != 0) return false;
     return g->k >= 2 * BK &&
            (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 30);
 }
@@ -369,11 +371,13 @@ int a8w8_quantize(const float* src, int rows, int k, int ld, uint8_t* q, void* s
         case A8W8_SCALE_MX_E8M0_TILED: {
             if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
             if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+            if (((uintptr_t)scale & 3) != 0) return A8W8_ERR_MISALIGNED;
             const long long threads = (long long)rows * k;
-            const int pad_blocks = ((k + 511) / 512) * 16 - k / 32;   // blocks of the last, partial K group
-            if (pad_blocks > 0)
-                hipLaunchKernelGGL(mx_tiled_pad_kernel, dim3((unsigned)(((long long)rows * pad_blocks + 255) / 256)),
-                                   dim3(256), 0, s, (uint8_t*)scale, rows, k);
+            if (rows % 64 != 0 || k % 512 != 0) {   // positions no (row, block) owns: 127 first
+                const size_t dwords = mx_tiled_bytes(rows, k) / 4;
+                hipLaunchKernelGGL(mx_tiled_fill_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0, s,
+                                   (uint32_t*)scale, dwords);
+            }
             hipLaunchKernelGGL(quant_mx_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows,
                                k, ld, q, (uint8_t*)scale);
             return launch_status();
@@ -391,8 +395,8 @@ int a8w8_mx_tile_scales(const uint8_t* sf, int rows, int k, int stride, uint8_t*
     if (stride < k / 32) return A8W8_ERR_BAD_STRIDE;
     if (!aligned16(out)) return A8W8_ERR_MISALIGNED;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-    const long long units = (long long)rows * ((k + 511) / 512);
-    hipLaunchKernelGGL(mx_tile_scales_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0,
+    const size_t dwords = mx_tiled_bytes(rows, k) / 4;
+    hipLaunchKernelGGL(mx_tile_scales_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0,
                        (hipStream_t)hip_stream, sf, rows, k, stride, out);
     return launch_status();
 }
@@ -400,7 +404,7 @@ int a8w8_mx_tile_scales(const uint8_t* sf, int rows, int k, int stride, uint8_t*
 size_t a8w8_mx_tiled_bytes(int rows, int k)
 {
     if (rows <= 0 || k <= 0) return 0;
-    return (size_t)rows * 16 * (size_t)((k + 511) / 512);
+    return mx_tiled_bytes(rows, k);
 }
 
 const char* a8w8_status_string(int status)

@@ -16,14 +16,25 @@ typedef unsigned short v4u16 __attribute__((ext_vector_type(4)));
 
 enum : int { MODE_TENSOR = 0, MODE_ROWCOL = 1, MODE_BLOCK = 2, MODE_MX = 3, MODE_MXT = 4 };
 
-// Byte position of the E8M0 exponent of (row, 32-wide K block kblk) in the tiled MX scale layout:
-// [K/512][rows][4 blocks of a 128-wide K step][4 consecutive K steps].  One 16-byte unit holds the
-// sixteen exponents of a row for 512 K elements, transposed so that the four steps of one block
-// position share a dword (the dword a lane of the scaled MFMA keeps for four K steps).
+// Byte position of the E8M0 exponent of (row, 32-wide K block kblk) in the tiled MX scale layout
+//   [K/512][ceil(rows/64)][pair of K steps: 2][r16: 16][g: 4][jp: 2][par: 2][s: 2]       (1 byte each)
+// where, inside a 64-row block, row = 32 jp + 8 (r16 >> 2) + 4 par + (r16 & 3) is the row that lane
+// r16 supplies to MFMA tile 2 jp + par of the block, g = kblk & 3 is the 32-block inside a 128-wide
+// K step and s the step inside the pair.  The eight bytes of (r16, g) are what one lane of the
+// scaled MFMA needs for two K steps of a 64-row block: two dwords, each holding two tiles x two
+// steps, selected per instruction through op_sel.  A 64-row block takes 1 KiB per 512 of K.
 __host__ __device__ inline size_t mx_tiled_index(int rows, int row, int kblk)
 {
-    return ((size_t)(kblk >> 4) * rows + row) * 16 + (kblk & 3) * 4 + ((kblk >> 2) & 3);
+    const int nblk = (rows + 63) >> 6, blk = row >> 6, rr = row & 63;
+    const int jp = rr >> 5, x = (rr >> 3) & 3, par = (rr >> 2) & 1, y = rr & 3;
+    const int g = kblk & 3, s = (kblk >> 2) & 1, pair = (kblk >> 3) & 1;
+    return ((((size_t)(kblk >> 4) * nblk + blk) * 2 + pair) * 64 + (4 * x + y) * 4 + g) * 8 + jp * 4 + par * 2 + s;
 }
+__host__ __device__ inline size_t mx_tiled_bytes(int rows, int k)
+{
+    return (size_t)((k + 511) >> 9) * ((rows + 63) >> 6) * 1024;
+}
+
 enum : int { C_BF16 = 0, C_FP32 = 1 };
 
 // Kernel parameters of the dense and flat GEMMs (strides in elements, as in the ABI).

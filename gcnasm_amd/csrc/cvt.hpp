@@ -219,38 +219,36 @@ __global__ void __launch_bounds__(256) quant_mx_kernel(const float* src, int row
 }
 
 // natural [rows][k/32] E8M0 scales (row stride `stride` bytes) -> the tiled layout of mx_tiled_index.
-// One thread per 16-byte unit (row, 512-wide K group); consecutive threads take consecutive rows,
-// so the writes are contiguous.  Blocks past k get 127 (scale 1.0; their products are never formed).
+// One thread per output dword: two tiles x two K steps of one (64-row block, r16, g, jp).
+// Consecutive threads write consecutive dwords.  Rows past `rows` and blocks past k get 127
+// (scale 1.0; their products are never formed or never stored).
 __global__ void __launch_bounds__(256) mx_tile_scales_kernel(const uint8_t* sf, int rows, int k, int stride,
                                                              uint8_t* out)
 {
-    const long long u = (long long)blockIdx.x * 256 + threadIdx.x;
-    const int groups = (k + 511) >> 9, blocks = k >> 5;
-    if (u >= (long long)rows * groups) return;
-    const int row = (int)(u % rows), kg = (int)(u / rows);
-    const uint8_t* src = sf + (size_t)row * stride + kg * 16;
-    uint32_t w[4] = {0, 0, 0, 0};
+    const size_t d = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (d >= mx_tiled_bytes(rows, k) / 4) return;
+    const int nblk = (rows + 63) >> 6, blocks = k >> 5;
+    const int jp = (int)(d & 1), g = (int)((d >> 1) & 3), r16 = (int)((d >> 3) & 15), pair = (int)((d >> 7) & 1);
+    const size_t rest = d >> 8;
+    const int blk = (int)(rest % nblk), kg = (int)(rest / nblk);
+    uint32_t w = 0;
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
+    for (int par = 0; par < 2; ++par)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int kblk = kg * 16 + s * 4 + g;
-            const uint32_t e = kblk < blocks ? src[s * 4 + g] : 127u;
-            w[g] |= e << (8 * s);
+        for (int s = 0; s < 2; ++s) {
+            const int row = blk * 64 + 32 * jp + 8 * (r16 >> 2) + 4 * par + (r16 & 3);
+            const int kblk = kg * 16 + pair * 8 + s * 4 + g;
+            const uint32_t e = (row < rows && kblk < blocks) ? sf[(size_t)row * stride + kblk] : 127u;
+            w |= e << (8 * (par * 2 + s));
         }
-    *(v4i*)(out + (size_t)u * 16) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    ((uint32_t*)out)[d] = w;
 }
 
-// 127 into the blocks of the last K group that lie past k (tiled layout), for producers that
-// write only the real blocks.
-__global__ void __launch_bounds__(256) mx_tiled_pad_kernel(uint8_t* scale, int rows, int k)
+// 127 everywhere (tiled layout), for producers that then write only the real (row, block) positions.
+__global__ void __launch_bounds__(256) mx_tiled_fill_kernel(uint32_t* scale, size_t dwords)
 {
-    const int blocks = k >> 5, total = ((k + 511) >> 9) * 16;
-    const int pad = total - blocks;
-    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)rows * pad) return;
-    const int row = (int)(idx % rows), kblk = blocks + (int)(idx / rows);
-    scale[mx_tiled_index(rows, row, kblk)] = 127;
+    const size_t d = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (d < dwords) scale[d] = 0x7f7f7f7fu;
 }
 
 }  // namespace a8w8

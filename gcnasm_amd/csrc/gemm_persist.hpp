@@ -43,6 +43,13 @@ constexpr int PERSIST_LDS_BYTES_MX = GEMM_LDS_BYTES_MX;
 #define A8W8_PERSIST_SCHED_BARRIER() (void)0
 #endif
 
+// scaled MFMA taking byte OA of scale_a and byte OB of scale_b (the selectors are immediates)
+template <int OA, int OB>
+A8W8_DEV v4f mfma_mx_sel(v8i a, v8i b, v4f c, int scale_a, int scale_b)
+{
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, OA, scale_a, OB, scale_b);
+}
+
 struct PersistParams {
     GemmParams g;
     int batch;        // work items = batch * tiles_m * tiles_n, walked with stride gridDim.x
@@ -59,6 +66,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     const int wave = wave_uniform(tid >> 6);
     const int wave_m = wave >> 1, wave_n = wave & 1;
     constexpr bool IS_MX = MODE == MODE_MX || MODE == MODE_MXT;
+    // tiled MX scales are laid out for A tiles whose rows are dealt like the B tiles' rows
+    constexpr bool PERM_A = MODE == MODE_MXT;
     const int r16 = lane & 15, g = lane >> 4;
     const int nk = p.k / BK;                       // >= 2 (checked by the host)
     const int tiles = p.tiles_m * p.tiles_n;
@@ -99,19 +108,17 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             voff_sf = min((is_b ? n0 : m0) + (wave & 3) * 64 + lane, rows - 1) * stride;
         }
         if constexpr (MODE == MODE_MXT) {
-            // tiled scales: the 16-byte units of 64 rows of a group are contiguous in memory, so one
-            // load instruction reads eight whole cache lines.  LDS slot (wave & 3) * 64 + lane takes
-            // tile row `slot` for A; for B the rows are dealt as the MFMA tiles read them (slot
-            // 16 j + r16 holds the row that lane r16 supplies to tile j).
+            // tiled scales: a 64-row block's exponents for four K steps are 1 KiB of contiguous memory
+            // in the order the lanes read them, so wave w copies block (w & 3) of the A tile (waves
+            // 0-3) or of the B tile (waves 4-7) with one load of eight whole cache lines.
             const bool is_b = wave >= 4;
             const int rows = is_b ? p.n : p.m;
             const uint8_t* base = is_b ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
                                        : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
-            rsrc_sf = make_rsrc(base, (uint32_t)rows * 16u * (uint32_t)((p.k + 511) >> 9));
-            const int slot = (wave & 3) * 64 + lane;
-            const int trow = is_b ? ((slot & ~31) | (((slot >> 2) & 3) << 3) | (((slot >> 4) & 1) << 2) | (slot & 3)) : slot;
-            voff_sf = min((is_b ? n0 : m0) + trow, rows - 1) * 16;
-            sf_group_stride = wave_uniform(rows * 16);
+            const int nblk = (rows + 63) >> 6;
+            rsrc_sf = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, p.k));   // blocks past the edge read 0
+            voff_sf = (((is_b ? n0 : m0) >> 6) + (wave & 3)) * 1024 + lane * 16;
+            sf_group_stride = wave_uniform(nblk * 1024);
         }
     };
     // one of the eight loads of a stage: 0..3 = A chunks, 4,5 = low B chunks, 6,7 = high B chunks.
@@ -150,14 +157,15 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     //     tile j, operand row 4g' + i  <-  row 32*(j/2) + 8g' + 4*(j%2) + i.
     // The swizzle key (row & 7) ^ (((row >> 3) & 3) << 1) keeps both read patterns free of LDS bank
     // conflicts (measured).  Only the tile's parity enters the key, the rest is an immediate offset.
+    const int lane_rg = r16 * 4 + g;
     auto swz_key = [](int row) __attribute__((always_inline)) { return ((row & 7) ^ (((row >> 3) & 3) << 1)) & 7; };
     int rd_a[2][2], rd_b[2][2];
 #pragma unroll
     for (int par = 0; par < 2; ++par)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const int row_a = 16 * par + r16;
             const int row_b = 8 * (r16 >> 2) + 4 * par + (r16 & 3);
+            const int row_a = PERM_A ? row_b : 16 * par + r16;
             rd_a[par][h] = (wave_m * WAVE_M + row_a) * BK + ((((g + 4 * h) ^ swz_key(row_a)) & 7) << 4);
             rd_b[par][h] = BM * BK + (wave_n * WAVE_N + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
         }
@@ -174,9 +182,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         return read_frag_at(stage, rd_b[j & 1], (j >> 1) * (32 * BK));
     };
     // natural MX scales: B tile t at + (t >> 1) * 512 + (t & 1) * 64; tiled: tile t at + t * 256, dword g
-    const int rd_sfa = GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16 + (MODE == MODE_MXT ? 4 * g : 0);
+    // tiled: 1 KiB per 64-row block = [pair of K steps][lane (r16, g)][8 bytes]
+    const int rd_sfa = MODE == MODE_MXT ? GEMM_LDS_BYTES + wave_m * 1024 + lane_rg * 8
+                                        : GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16;
     const int rd_sfb = MODE == MODE_MXT
-                           ? GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + r16) * 16 + 4 * g
+                           ? GEMM_LDS_BYTES + 4096 + wave_n * 2048 + lane_rg * 8
                            : GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + 8 * (r16 >> 2) + (r16 & 3)) * 16;
 
     int cur_item = blockIdx.x, cur_ks = 0;         // the step being multiplied
@@ -200,6 +210,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     // scales consumed by the MFMAs of a step (BLOCK: fp32 per row x per column block, MX: E8M0 bytes)
     float blk_s[TM], blk_s_next[TM];
     int mx_sa[TM], mx_sb[TN], mx_sa_next[TM], mx_sb_next[TN];
+    v2i mxt_a, mxt_a_next;      // tiled MX: dword t/2 serves tiles t, t^1 and both steps of a pair
+    v4i mxt_b, mxt_b_next;
     auto fetch_step_scales = [&](int batch, int mm0, int nn0, int kstep, int gbase) __attribute__((always_inline)) {
         (void)gbase;
         if constexpr (MODE == MODE_BLOCK) {
@@ -224,12 +236,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                 mx_sb_next[t] = *(const int*)(s + rd_sfb + (t >> 1) * 512 + (t & 1) * 64);
         }
         if constexpr (MODE == MODE_MXT) {
-            // the dword of (row, block position g) holds the exponents of the group's four K steps
-            const char* s = smem + ((gbase + (kstep >> 2)) & 1) * MX_GROUP_BYTES;
-#pragma unroll
-            for (int t = 0; t < TM; ++t) mx_sa_next[t] = *(const int*)(s + rd_sfa + t * 256);
-#pragma unroll
-            for (int t = 0; t < TN; ++t) mx_sb_next[t] = *(const int*)(s + rd_sfb + t * 256);
+            // called for the first step of a pair: the lane's eight bytes per 64-row block
+            const char* s = smem + ((gbase + (kstep >> 2)) & 1) * MX_GROUP_BYTES + ((kstep >> 1) & 1) * 512;
+            mxt_a_next = *(const v2i*)(s + rd_sfa);
+            const v2i lo = *(const v2i*)(s + rd_sfb), hi = *(const v2i*)(s + rd_sfb + 1024);
+            mxt_b_next = v4i{lo.x, lo.y, hi.x, hi.y};
         }
     };
     auto rotate_step_scales = [&]() __attribute__((always_inline)) {
@@ -244,11 +255,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             for (int t = 0; t < TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sb_next[t], 8 * g, 8);
         }
         if constexpr (MODE == MODE_MXT) {
-            const int sh = (cur_ks & 3) * 8;
-#pragma unroll
-            for (int t = 0; t < TM; ++t) mx_sa[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sa_next[t], sh, 8);
-#pragma unroll
-            for (int t = 0; t < TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sb_next[t], sh, 8);
+            mxt_a = mxt_a_next;
+            mxt_b = mxt_b_next;
         }
     };
 
@@ -256,14 +264,17 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     auto store_tile = [&]() __attribute__((always_inline)) {
         const float* sfa_f = (const float*)p.sfa + (long long)cur_batch * p.sfa_batch;
         const float* sfb_f = (const float*)p.sfb + (long long)cur_batch * p.sfb_batch;
-        const int cm_base = m0 + wave_m * WAVE_M + r16;
+        const int cm_base = m0 + wave_m * WAVE_M + (PERM_A ? 8 * (r16 >> 2) + (r16 & 3) : r16);
+        auto cm_of = [&](int i) __attribute__((always_inline)) {          // C row of MFMA tile i
+            return cm_base + (PERM_A ? 32 * (i >> 1) + 4 * (i & 1) : 16 * i);
+        };
         const int cn_base = n0 + wave_n * WAVE_N + 8 * g;      // + 32 * (tile pair): eight consecutive n
         float sa[TM];
         float ts = 1.f;
         if constexpr (MODE == MODE_TENSOR) ts = sfa_f[0] * sfb_f[0];
         if constexpr (MODE == MODE_ROWCOL) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) sa[i] = sfa_f[min(cm_base + 16 * i, p.m - 1)];
+            for (int i = 0; i < TM; ++i) sa[i] = sfa_f[min(cm_of(i), p.m - 1)];
         }
         char* c_base = (char*)p.c + (long long)cur_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
         const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 7) == 0 && (((uintptr_t)c_base) & 15) == 0)
@@ -293,7 +304,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             const int cn = cn_base + 32 * jp;
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                const int cm = cm_base + 16 * i;
+                const int cm = cm_of(i);
                 float v[8];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -373,7 +384,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         constexpr int P = decltype(parity)::value;
         Frags& cur = F[PREFETCH_FRAGS ? P : 0];
         Frags& nxt = F[PREFETCH_FRAGS ? P ^ 1 : 0];
-        rotate_step_scales();
+        if constexpr (MODE != MODE_MXT || P == 0) rotate_step_scales();
         if constexpr (!PREFETCH_FRAGS) {
 #pragma unroll
             for (int t = 0; t < TM; ++t) cur.a[t] = read_frag_a(P, t);
@@ -405,7 +416,15 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             A8W8_PERSIST_SCHED_BARRIER();
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                if constexpr (IS_MX) {
+                if constexpr (MODE == MODE_MXT) {
+                    // K steps come in pairs and tiles start on even steps, so the step inside the
+                    // pair is the LDS stage parity P
+                    const int sb = mxt_b[j >> 1], sa = mxt_a[i >> 1];
+                    acc[i][j] = (j & 1) ? ((i & 1) ? mfma_mx_sel<2 + P, 2 + P>(fb[j], cur.a[i], acc[i][j], sb, sa)
+                                                   : mfma_mx_sel<2 + P, P>(fb[j], cur.a[i], acc[i][j], sb, sa))
+                                        : ((i & 1) ? mfma_mx_sel<P, 2 + P>(fb[j], cur.a[i], acc[i][j], sb, sa)
+                                                   : mfma_mx_sel<P, P>(fb[j], cur.a[i], acc[i][j], sb, sa));
+                } else if constexpr (MODE == MODE_MX) {
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], cur.a[i], acc[i][j], 0, 0, 0,
                                                                                  mx_sb[j], 0, mx_sa[i]);
                 } else if constexpr (MODE == MODE_BLOCK) {
@@ -455,7 +474,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                     for (int t = 0; t < TM; ++t) nxt.a[t] = read_frag_a(P ^ 1, t);
                     nxt.b0 = read_frag_b(P ^ 1, 0);
                 }
-                if constexpr (IS_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
+                if constexpr (MODE == MODE_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
+                if constexpr (MODE == MODE_MXT && P == 1) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
             }
             if (j == 7) {
                 issue_one(P, ld_ks, 4);

@@ -64,6 +64,10 @@ def lib():
         L.orc_preshuffle_index.argtypes = [ctypes.c_int] * 3
         L.orc_preshuffle_b.argtypes = [_u8p, _u8p, ctypes.c_int, ctypes.c_int]
         L.orc_unshuffle_b.argtypes = [_u8p, _u8p, ctypes.c_int, ctypes.c_int]
+        L.orc_mx_tiled_bytes.restype = ctypes.c_size_t
+        L.orc_mx_tiled_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
+        L.orc_mx_tile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
+        L.orc_mx_untile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
         L.orc_flatmm_ref.argtypes = [_u8p, _u8p, _f32p, _f32p, _f32p] + [ctypes.c_int] * 5
         L.orc_count_abs_mismatch.restype = ctypes.c_long
         L.orc_count_abs_mismatch.argtypes = [_f32p, _f32p, ctypes.c_size_t, ctypes.c_float]
@@ -199,6 +203,26 @@ def unshuffle_b(bs, n, k):
     bs = _c(bs, np.uint8)
     out = np.empty((n, k), np.uint8)
     lib().orc_unshuffle_b(_p(bs, _u8p), _p(out, _u8p), n, k)
+    return out
+
+
+def mx_tiled_bytes(rows, k):
+    return lib().orc_mx_tiled_bytes(rows, k)
+
+
+def mx_tile_scales(sf):
+    """[rows, K/32] u8 -> flat u8 in the library's tiled MX scale layout."""
+    sf = _c(sf, np.uint8)
+    rows, kb = sf.shape
+    out = np.empty(mx_tiled_bytes(rows, kb * 32), np.uint8)
+    lib().orc_mx_tile_scales(_p(sf, _u8p), rows, kb * 32, kb, _p(out, _u8p))
+    return out
+
+
+def mx_untile_scales(tiled, rows, k):
+    tiled = _c(tiled, np.uint8)
+    out = np.zeros((rows, k // 32), np.uint8)
+    lib().orc_mx_untile_scales(_p(tiled, _u8p), rows, k, k // 32, _p(out, _u8p))
     return out
 
 

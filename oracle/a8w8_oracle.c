@@ -22,6 +22,10 @@
  *   orc_gemm_ref / orc_gemm_ref_mx   brute force in float64 on tiny shapes,
  *       exact-integer inputs, scale-mode reductions.
  *   orc_preshuffle_b       bijection + flatmm(A, shuffle(B)) == gemm(A, B).
+ *   orc_mx_tile_scales     a layout this library defines (the reference has no MXFP8
+ *       program): written as a walk over the layout's dimensions, i.e. the inverse of
+ *       the index formula the kernels use; bijection on full blocks, padding = 127,
+ *       and gemm(A, B, tile(sfa), tile(sfb)) == gemm(A, B, sfa, sfb).
  */
 #include <math.h>
 #include <stddef.h>
@@ -344,6 +348,50 @@ ORC_API void orc_unshuffle_b(const uint8_t* bs, uint8_t* out, int N, int K)
 {
     for (int n = 0; n < N; ++n)
         for (int k = 0; k < K; ++k) out[(size_t)n * K + k] = bs[orc_preshuffle_index(n, k, K)];
+}
+
+/* Tiled layout of MX E8M0 scales (defined by this library; no reference counterpart).
+ * Dimensions, outermost first, one byte per innermost element:
+ *     [K/512][ceil(rows/64)][pair of K steps: 2][r16: 16][g: 4][jp: 2][par: 2][s: 2]
+ * holding the exponent of row  64*blk + 32*jp + 8*(r16/4) + 4*par + r16%4  and of 32-wide
+ * K block  16*kg + 8*pair + 4*s + g.  Rows past `rows` and blocks past k/32 hold 127. */
+ORC_API size_t orc_mx_tiled_bytes(int rows, int k)
+{
+    return (size_t)((k + 511) / 512) * (size_t)((rows + 63) / 64) * 1024;
+}
+ORC_API void orc_mx_tile_scales(const uint8_t* sf, int rows, int k, int stride, uint8_t* out)
+{
+    const int groups = (k + 511) / 512, nblk = (rows + 63) / 64, blocks = k / 32;
+    uint8_t* o = out;
+    for (int kg = 0; kg < groups; ++kg)
+        for (int blk = 0; blk < nblk; ++blk)
+            for (int pair = 0; pair < 2; ++pair)
+                for (int r16 = 0; r16 < 16; ++r16)
+                    for (int g = 0; g < 4; ++g)
+                        for (int jp = 0; jp < 2; ++jp)
+                            for (int par = 0; par < 2; ++par)
+                                for (int st = 0; st < 2; ++st) {
+                                    const int row = 64 * blk + 32 * jp + 8 * (r16 / 4) + 4 * par + r16 % 4;
+                                    const int kblk = 16 * kg + 8 * pair + 4 * st + g;
+                                    *o++ = (row < rows && kblk < blocks) ? sf[(size_t)row * stride + kblk] : 127;
+                                }
+}
+ORC_API void orc_mx_untile_scales(const uint8_t* tiled, int rows, int k, int stride, uint8_t* sf)
+{
+    const int groups = (k + 511) / 512, nblk = (rows + 63) / 64, blocks = k / 32;
+    const uint8_t* o = tiled;
+    for (int kg = 0; kg < groups; ++kg)
+        for (int blk = 0; blk < nblk; ++blk)
+            for (int pair = 0; pair < 2; ++pair)
+                for (int r16 = 0; r16 < 16; ++r16)
+                    for (int g = 0; g < 4; ++g)
+                        for (int jp = 0; jp < 2; ++jp)
+                            for (int par = 0; par < 2; ++par)
+                                for (int st = 0; st < 2; ++st, ++o) {
+                                    const int row = 64 * blk + 32 * jp + 8 * (r16 / 4) + 4 * par + r16 % 4;
+                                    const int kblk = 16 * kg + 8 * pair + 4 * st + g;
+                                    if (row < rows && kblk < blocks) sf[(size_t)row * stride + kblk] = *o;
+                                }
 }
 
 /* flatmm oracle that consumes the SHUFFLED weights directly: gemm_ref's math

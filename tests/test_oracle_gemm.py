@@ -132,3 +132,31 @@ def test_generators_are_seeded_and_use_full_range(orc, gen):
     q = orc.decode(x[0])
     assert np.isfinite(q).all()
     assert np.abs(q).max() >= (224 if gen == "mx" else 448)   # amax maps to the top of E4M3
+
+
+def test_mx_tiled_layout_is_a_bijection_with_127_padding(orc):
+    """Full 64-row blocks and whole 512-wide K groups: tiling permutes the bytes (distinct values in,
+    the same multiset out, untile inverts it).  Ragged shapes: every byte no (row, block) owns is 127."""
+    rows, k = 128, 1024
+    sf = (np.arange(rows * (k // 32)) % 251).astype(np.uint8).reshape(rows, k // 32)
+    t = orc.mx_tile_scales(sf)
+    assert t.size == rows * (k // 32) == orc.mx_tiled_bytes(rows, k)
+    assert (np.sort(t) == np.sort(sf.ravel())).all()
+    assert (orc.mx_untile_scales(t, rows, k) == sf).all()
+    rows, k = 70, 384
+    sf = np.full((rows, k // 32), 5, np.uint8)
+    t = orc.mx_tile_scales(sf)
+    assert t.size == 2 * 1024 and (t == 5).sum() == rows * (k // 32) and (t == 127).sum() == t.size - rows * (k // 32)
+    assert (orc.mx_untile_scales(t, rows, k) == sf).all()
+
+
+def test_mx_tiled_layout_groups_what_one_lane_needs(orc):
+    """The eight bytes of (block, pair, r16, g) are two dwords of [tile parity][step]: byte (jp, par, s)
+    belongs to row 32 jp + 8 (r16/4) + 4 par + r16%4 of the block and to K block 8 pair + 4 s + g."""
+    rows, k = 64, 512
+    sf = np.zeros((rows, k // 32), np.uint8)
+    row, kblk = 32 * 1 + 8 * 2 + 4 * 1 + 3, 8 * 1 + 4 * 0 + 2      # jp=1, r16=11, par=1; pair=1, s=0, g=2
+    sf[row, kblk] = 200
+    t = orc.mx_tile_scales(sf)
+    pos = int(np.nonzero(t == 200)[0][0])
+    assert pos == ((1 * 64 + 11 * 4 + 2) * 8) + 1 * 4 + 1 * 2 + 0
