@@ -108,6 +108,8 @@ bool persist_ok(const a8w8_gemm_args* g)
 {
     // tiled MX scales come in pairs of K steps (one dword serves two steps)
     if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED && (g->k / BK) % 2 != 0) return false;
+    // the load offsets are formed with 24-bit multiplies
+    if (g->m >= (1 << 23) || g->n >= (1 << 23) || g->stride_a >= (1 << 23) || g->stride_b >= (1 << 23)) return false;
     return g->k >= 2 * BK &&
            (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 30);
 }

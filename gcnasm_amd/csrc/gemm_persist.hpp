@@ -31,8 +31,33 @@ constexpr int PERSIST_LDS_BYTES = GEMM_LDS_BYTES;
 constexpr int PERSIST_LDS_BYTES_MX = GEMM_LDS_BYTES_MX;
 
 #define A8W8_RAW_BARRIER() asm volatile("s_barrier" ::: "memory")
-#ifndef A8W8_PREFETCH_FRAGS
-#define A8W8_PREFETCH_FRAGS(mode) ((mode) == MODE_TENSOR)
+// How many of the next step's four A fragments (plus the first B fragment) are fetched from LDS in
+// the shadow of the current step's last MFMA group.  Bounded by the registers each mode has left:
+// a spill inside the K loop is reloaded behind a wait for every load in flight.
+#ifndef A8W8_NPF_ROWCOL
+#define A8W8_NPF_ROWCOL 2
+#endif
+#ifndef A8W8_NPF_MXT
+#define A8W8_NPF_MXT 2
+#endif
+#ifndef A8W8_NPF_MX
+#define A8W8_NPF_MX 1
+#endif
+#define A8W8_PREFETCH_A(mode)                                                                        \
+    ((mode) == MODE_TENSOR ? 4 : (mode) == MODE_ROWCOL ? A8W8_NPF_ROWCOL : (mode) == MODE_MXT ? A8W8_NPF_MXT \
+                                                     : (mode) == MODE_MX ? A8W8_NPF_MX : 0)
+#ifndef A8W8_PERSIST_BLK_LAG
+#define A8W8_PERSIST_BLK_LAG 4
+#endif
+#ifndef A8W8_BLK_SB
+#define A8W8_BLK_SB 1
+#endif
+#if A8W8_BLK_SB == 1
+#define A8W8_BLK_SCHED_BARRIER() __builtin_amdgcn_sched_barrier(0)
+#elif A8W8_BLK_SB == 2
+#define A8W8_BLK_SCHED_BARRIER() __builtin_amdgcn_sched_barrier(0x6)  /* VALU and SALU may cross */
+#else
+#define A8W8_BLK_SCHED_BARRIER() (void)0
 #endif
 #ifndef A8W8_PERSIST_SB
 #define A8W8_PERSIST_SB 0
@@ -78,13 +103,13 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     const int groups_per_tile = (nk + 3) >> 2;      // MX scale groups (4 K steps each) per tile
     int ld_gbase = 0, cur_gbase = 0;                // running group count: picks the scale buffer
     __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_sf;
-    int voff_a[4], voff_b[4], voff_sf = 0;
+    int ld_m0 = 0, ld_n0 = 0, voff_sf = 0;            // tile origin at the load position (wave-uniform)
     int sf_group_stride = 16;                       // bytes from one scale group of a row set to the next
     const int ld_row = wave * 8 + (lane >> 3);
     // lane i of a 1 KiB chunk lands on row (i>>3), slot (i&7) of the chunk's 8 rows; the slot holds
     // K-piece slot ^ key(row) with key(row) = (row & 7) ^ (((row >> 3) & 3) << 1), and bits 3-4 of the
     // tile row are (chunk & 3) = (wave & 3) for every chunk this wave fills
-    const int ld_piece = (lane & 7) ^ (((lane >> 3) ^ ((wave & 3) << 1)) & 7);
+    const int ld_piece16 = ((lane & 7) ^ (((lane >> 3) ^ ((wave & 3) << 1)) & 7)) * 16;
     auto point_loads_at = [&](int item) __attribute__((always_inline)) {
         item = min(item, pp.items - 1);            // past the end: keep loading valid data nobody reads
         const int batch = item / tiles;
@@ -93,11 +118,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         const int m0 = tm * BM, n0 = tn * BN;
         rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
         rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, (uint32_t)(p.n - 1) * p.ldb + p.k);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            voff_a[j] = min(m0 + ld_row + 64 * j, p.m - 1) * p.lda + ld_piece * 16;
-            voff_b[j] = min(n0 + ld_row + 64 * j, p.n - 1) * p.ldb + ld_piece * 16;
-        }
+        ld_m0 = m0;
+        ld_n0 = n0;
         if constexpr (MODE == MODE_MX) {
             const bool is_b = wave >= 4;           // waves 0-3 stage A-row scales, 4-7 B-row scales
             const int rows = is_b ? p.n : p.m;
@@ -127,11 +149,16 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     auto issue_one = [&](int stage, int kstep, int which) __attribute__((always_inline)) {
         A8W8_LDS char* s = (A8W8_LDS char*)smem + stage * STAGE_BYTES + wave * 1024;
         const int koff = kstep * BK;
+        // the lane's byte offset is recomputed for every load (three VALU operations) rather than
+        // kept in eight registers: the kernel has none to spare, and a spilled offset would be
+        // reloaded from scratch behind a wait for every load in flight
         if (which < 4) {
-            load_to_lds_16(rsrc_a, s + which * 8192, voff_a[which], koff);
+            const int voff = __mul24(min(ld_m0 + ld_row + 64 * which, p.m - 1), p.lda) + ld_piece16;
+            load_to_lds_16(rsrc_a, s + which * 8192, voff, koff);
         } else {
             const int j = which == 4 ? 0 : which == 5 ? 2 : which == 6 ? 1 : 3;
-            load_to_lds_16(rsrc_b, s + BM * BK + j * 8192, voff_b[j], koff);
+            const int voff = __mul24(min(ld_n0 + ld_row + 64 * j, p.n - 1), p.ldb) + ld_piece16;
+            load_to_lds_16(rsrc_b, s + BM * BK + j * 8192, voff, koff);
         }
     };
     auto issue_mx_group = [&](int group) __attribute__((always_inline)) {
@@ -159,27 +186,30 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     // conflicts (measured).  Only the tile's parity enters the key, the rest is an immediate offset.
     const int lane_rg = r16 * 4 + g;
     auto swz_key = [](int row) __attribute__((always_inline)) { return ((row & 7) ^ (((row >> 3) & 3) << 1)) & 7; };
-    int rd_a[2][2], rd_b[2][2];
+    // For the rows of tile parity 1 the key differs from parity 0's in bit 2 only, and so do the two
+    // K halves h of a fragment: slot(par, h) = slot(0, 0) ^ 4 (par ^ h).  Two address registers per
+    // operand (h = 0, 1 of parity 0) therefore serve all four combinations; parity 1 swaps them and
+    // adds its row offset as an immediate.
+    constexpr int A_PAR_BYTES = (PERM_A ? 4 : 16) * BK, B_PAR_BYTES = 4 * BK;
+    int rd_a[2], rd_b[2];
 #pragma unroll
-    for (int par = 0; par < 2; ++par)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int row_b = 8 * (r16 >> 2) + 4 * par + (r16 & 3);
-            const int row_a = PERM_A ? row_b : 16 * par + r16;
-            rd_a[par][h] = (wave_m * WAVE_M + row_a) * BK + ((((g + 4 * h) ^ swz_key(row_a)) & 7) << 4);
-            rd_b[par][h] = BM * BK + (wave_n * WAVE_N + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
-        }
-    auto read_frag_at = [&](int stage, const int (&base)[2], int byte_off) __attribute__((always_inline)) -> v8i {
+    for (int h = 0; h < 2; ++h) {
+        const int row_b = 8 * (r16 >> 2) + (r16 & 3);
+        const int row_a = PERM_A ? row_b : r16;
+        rd_a[h] = (wave_m * WAVE_M + row_a) * BK + ((((g + 4 * h) ^ swz_key(row_a)) & 7) << 4);
+        rd_b[h] = BM * BK + (wave_n * WAVE_N + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
+    }
+    auto read_frag_at = [&](int stage, const int (&base)[2], int par, int byte_off) __attribute__((always_inline)) -> v8i {
         const char* s = smem + stage * STAGE_BYTES + byte_off;
-        const v4i lo = *(const v4i*)(s + base[0]);
-        const v4i hi = *(const v4i*)(s + base[1]);
+        const v4i lo = *(const v4i*)(s + base[par]);
+        const v4i hi = *(const v4i*)(s + base[par ^ 1]);
         return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     };
     auto read_frag_a = [&](int stage, int t) __attribute__((always_inline)) -> v8i {
-        return read_frag_at(stage, rd_a[t & 1], (t >> 1) * (32 * BK));
+        return read_frag_at(stage, rd_a, t & 1, (t >> 1) * (32 * BK) + (t & 1) * A_PAR_BYTES);
     };
     auto read_frag_b = [&](int stage, int j) __attribute__((always_inline)) -> v8i {
-        return read_frag_at(stage, rd_b[j & 1], (j >> 1) * (32 * BK));
+        return read_frag_at(stage, rd_b, j & 1, (j >> 1) * (32 * BK) + (j & 1) * B_PAR_BYTES);
     };
     // natural MX scales: B tile t at + (t >> 1) * 512 + (t & 1) * 64; tiled: tile t at + t * 256, dword g
     // tiled: 1 KiB per 64-row block = [pair of K steps][lane (r16, g)][8 bytes]
@@ -215,14 +245,19 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     auto fetch_step_scales = [&](int batch, int mm0, int nn0, int kstep, int gbase) __attribute__((always_inline)) {
         (void)gbase;
         if constexpr (MODE == MODE_BLOCK) {
+            // A-row scales through a buffer descriptor: 32-bit lane offsets instead of 64-bit pointers
             const float* sfa_f = (const float*)p.sfa + (long long)batch * p.sfa_batch;
             const float* sfb_f = (const float*)p.sfb + (long long)batch * p.sfb_batch;
+            const __amdgpu_buffer_rsrc_t rs =
+                make_rsrc(sfa_f, (uint32_t)((nk - 1) * p.stride_sfa + p.m) * 4u);
             const int nb = min(nn0 + wave_n * WAVE_N, p.n - 1) >> 7;
             const float sb = sfb_f[(long long)nb * p.stride_sfb + kstep];
+            const int row0 = mm0 + wave_m * WAVE_M + r16;
 #pragma unroll
             for (int t = 0; t < TM; ++t)
-                blk_s_next[t] =
-                    sfa_f[(long long)kstep * p.stride_sfa + min(mm0 + wave_m * WAVE_M + r16 + 16 * t, p.m - 1)] * sb;
+                blk_s_next[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                              rs, min(row0 + 16 * t, p.m - 1) * 4,
+                                                              kstep * p.stride_sfa * 4, 0)) * sb;
         }
         if constexpr (MODE == MODE_MX) {
             // one dword per (row, K step) holds the four block exponents; lane group g extracts
@@ -345,7 +380,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     // The next step's A fragments and first B fragment are fetched in the shadow of the last MFMA
     // group; the block-scale mode has no registers to spare for that second set and reads them
     // when the step begins.
-    constexpr bool PREFETCH_FRAGS = A8W8_PREFETCH_FRAGS(MODE);
+    constexpr int NPF = A8W8_PREFETCH_A(MODE);
+    constexpr bool PREFETCH_FRAGS = NPF > 0;
     struct Frags {
         v8i a[TM];
         v8i b0;
@@ -371,7 +407,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     if constexpr (IS_MX) fetch_step_scales(cur_batch, m0, n0, 0, 0);
     if constexpr (PREFETCH_FRAGS) {
 #pragma unroll
-        for (int t = 0; t < TM; ++t) F[0].a[t] = read_frag_a(0, t);
+        for (int t = 0; t < NPF; ++t) F[0].a[t] = read_frag_a(0, t);
         F[0].b0 = read_frag_b(0, 0);
     }
     zero_acc();
@@ -385,11 +421,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         Frags& cur = F[PREFETCH_FRAGS ? P : 0];
         Frags& nxt = F[PREFETCH_FRAGS ? P ^ 1 : 0];
         if constexpr (MODE != MODE_MXT || P == 0) rotate_step_scales();
-        if constexpr (!PREFETCH_FRAGS) {
 #pragma unroll
-            for (int t = 0; t < TM; ++t) cur.a[t] = read_frag_a(P, t);
-            cur.b0 = read_frag_b(P, 0);
-        }
+        for (int t = NPF; t < TM; ++t) cur.a[t] = read_frag_a(P, t);
+        if constexpr (!PREFETCH_FRAGS) cur.b0 = read_frag_b(P, 0);
         // where the next step lives (it may be the first step of this workgroup's next tile)
         const bool last_of_tile = cur_ks + 1 == nk;
         int nx_batch = cur_batch, nx_m0 = m0, nx_n0 = n0, nx_gbase = cur_gbase;
@@ -407,7 +441,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         v8i fb[TN];
         fb[0] = cur.b0;
         // block scales: acc += part * scale trails the MFMA that made `part` by BLK_LAG tiles
-        constexpr int BLK_LAG = 4;
+        constexpr int BLK_LAG = A8W8_PERSIST_BLK_LAG;
         v4f part[BLK_LAG + 1];
         (void)part;
 #pragma unroll
@@ -431,12 +465,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                     const int t = j * TM + i;
                     part[t % (BLK_LAG + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                         fb[j], cur.a[i], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                    __builtin_amdgcn_sched_barrier(0);
+                    A8W8_BLK_SCHED_BARRIER();
                     if (t >= BLK_LAG) {
                         const int u = t - BLK_LAG;
                         acc[u % TM][u / TM] += part[u % (BLK_LAG + 1)] * blk_s[u % TM];
                     }
-                    __builtin_amdgcn_sched_barrier(0);
+                    A8W8_BLK_SCHED_BARRIER();
                     if (t == TM * TN - 1) {
 #pragma unroll
                         for (int u = TM * TN - BLK_LAG; u < TM * TN; ++u)
@@ -471,7 +505,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                 A8W8_RAW_BARRIER();                   // end: all of stage P is free
                 if constexpr (PREFETCH_FRAGS) {
 #pragma unroll
-                    for (int t = 0; t < TM; ++t) nxt.a[t] = read_frag_a(P ^ 1, t);
+                    for (int t = 0; t < NPF; ++t) nxt.a[t] = read_frag_a(P ^ 1, t);
                     nxt.b0 = read_frag_b(P ^ 1, 0);
                 }
                 if constexpr (MODE == MODE_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
