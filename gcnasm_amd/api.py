@@ -73,6 +73,8 @@ def lib():
         L.a8w8_quantize.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_int,
                                     ctypes.c_int, vp]
         L.a8w8_mx_tile_scales.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp]
+        L.a8w8_mx_tile_scales_ab.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_int, ctypes.c_int, vp,
+                                             ctypes.c_int, vp]
         L.a8w8_mx_tiled_bytes.restype = ctypes.c_size_t
         L.a8w8_mx_tiled_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
         L.a8w8_status_string.restype = ctypes.c_char_p
@@ -249,6 +251,18 @@ def mx_tile_scales(sf, out=None):
     _check(lib().a8w8_mx_tile_scales(sf.data_ptr(), rows, kb * 32, sf.stride(0), out.data_ptr(), _stream()),
            "a8w8_mx_tile_scales")
     return out
+
+
+def mx_tile_scales_ab(sfa, sfb):
+    """Both scale arrays of a GEMM ([M, K/32] and [N, K/32] u8) -> MX_TILED, one launch."""
+    import torch
+    m, kb = sfa.shape
+    n = sfb.shape[0]
+    ta = torch.empty(mx_tiled_bytes(m, kb * 32), dtype=torch.uint8, device=sfa.device)
+    tb = torch.empty(mx_tiled_bytes(n, kb * 32), dtype=torch.uint8, device=sfb.device)
+    _check(lib().a8w8_mx_tile_scales_ab(sfa.data_ptr(), m, sfa.stride(0), ta.data_ptr(), sfb.data_ptr(), n,
+                                        sfb.stride(0), tb.data_ptr(), kb * 32, _stream()), "a8w8_mx_tile_scales_ab")
+    return ta, tb
 
 
 def kernel_name(g):

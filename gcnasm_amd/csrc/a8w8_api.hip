@@ -397,9 +397,24 @@ int a8w8_mx_tile_scales(const uint8_t* sf, int rows, int k, int stride, uint8_t*
     if (stride < k / 32) return A8W8_ERR_BAD_STRIDE;
     if (!aligned16(out)) return A8W8_ERR_MISALIGNED;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-    const size_t dwords = mx_tiled_bytes(rows, k) / 4;
-    hipLaunchKernelGGL(mx_tile_scales_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)hip_stream, sf, rows, k, stride, out);
+    const size_t units = mx_tiled_bytes(rows, k) >> 10;
+    hipLaunchKernelGGL(mx_tile_scales_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0,
+                       (hipStream_t)hip_stream, sf, rows, stride, out, (const uint8_t*)nullptr, 0, 0, (uint8_t*)nullptr, k);
+    return launch_status();
+}
+
+int a8w8_mx_tile_scales_ab(const uint8_t* sfa, int m, int stride_sfa, uint8_t* out_a, const uint8_t* sfb, int n,
+                           int stride_sfb, uint8_t* out_b, int k, void* hip_stream)
+{
+    if (!sfa || !out_a || !sfb || !out_b) return A8W8_ERR_NULL_POINTER;
+    if (m <= 0 || n <= 0 || k <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
+    if (stride_sfa < k / 32 || stride_sfb < k / 32) return A8W8_ERR_BAD_STRIDE;
+    if (!aligned16(out_a) || !aligned16(out_b)) return A8W8_ERR_MISALIGNED;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    const size_t units0 = mx_tiled_bytes(m, k) >> 10, units1 = mx_tiled_bytes(n, k) >> 10;
+    hipLaunchKernelGGL(mx_tile_scales_kernel, dim3((unsigned)((units0 + units1 + 3) / 4)), dim3(256), 0,
+                       (hipStream_t)hip_stream, sfa, m, stride_sfa, out_a, sfb, n, stride_sfb, out_b, k);
     return launch_status();
 }
 

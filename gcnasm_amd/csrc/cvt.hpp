@@ -222,26 +222,64 @@ __global__ void __launch_bounds__(256) quant_mx_kernel(const float* src, int row
 // One thread per output dword: two tiles x two K steps of one (64-row block, r16, g, jp).
 // Consecutive threads write consecutive dwords.  Rows past `rows` and blocks past k get 127
 // (scale 1.0; their products are never formed or never stored).
-__global__ void __launch_bounds__(256) mx_tile_scales_kernel(const uint8_t* sf, int rows, int k, int stride,
-                                                             uint8_t* out)
+// One launch for one or two scale arrays (the A-side and the B-side scales of a GEMM).  A group of
+// 64 threads handles one 1 KiB unit (64 rows x 16 K blocks): thread r copies the 16 bytes of row r
+// into LDS, then thread t gathers and writes bytes 16t..16t+15 of the unit.  256 threads = 4 units.
+__global__ void __launch_bounds__(256) mx_tile_scales_kernel(const uint8_t* sf0, int rows0, int stride0, uint8_t* out0,
+                                                             const uint8_t* sf1, int rows1, int stride1, uint8_t* out1,
+                                                             int k)
 {
-    const size_t d = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (d >= mx_tiled_bytes(rows, k) / 4) return;
-    const int nblk = (rows + 63) >> 6, blocks = k >> 5;
-    const int jp = (int)(d & 1), g = (int)((d >> 1) & 3), r16 = (int)((d >> 3) & 15), pair = (int)((d >> 7) & 1);
-    const size_t rest = d >> 8;
-    const int blk = (int)(rest % nblk), kg = (int)(rest / nblk);
-    uint32_t w = 0;
+    __shared__ uint8_t lds[4][64 * 16];
+    const int t = threadIdx.x & 63, sub = threadIdx.x >> 6;
+    size_t unit = (size_t)blockIdx.x * 4 + sub;
+    const size_t units0 = mx_tiled_bytes(rows0, k) >> 10;
+    const uint8_t* sf = sf0;
+    uint8_t* out = out0;
+    int rows = rows0, stride = stride0;
+    bool live = true;
+    if (unit >= units0) {
+        unit -= units0;
+        sf = sf1;
+        out = out1;
+        rows = rows1;
+        stride = stride1;
+        live = sf1 != nullptr && unit < (mx_tiled_bytes(rows1, k) >> 10);
+    }
+    const int blocks = k >> 5;
+    if (live) {
+        const int nblk = (rows + 63) >> 6;
+        const int blk = (int)(unit % nblk), kg = (int)(unit / nblk);
+        const int row = blk * 64 + t;
+        const uint8_t* src = sf + (size_t)row * stride + kg * 16;
+        const bool vec = row < rows && kg * 16 + 16 <= blocks && (((uintptr_t)src) & 3) == 0;
+        uint32_t w[4] = {0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu};
+        if (vec) {
 #pragma unroll
-    for (int par = 0; par < 2; ++par)
+            for (int q = 0; q < 4; ++q) w[q] = ((const uint32_t*)src)[q];
+        } else if (row < rows) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const int row = blk * 64 + 32 * jp + 8 * (r16 >> 2) + 4 * par + (r16 & 3);
-            const int kblk = kg * 16 + pair * 8 + s * 4 + g;
-            const uint32_t e = (row < rows && kblk < blocks) ? sf[(size_t)row * stride + kblk] : 127u;
-            w |= e << (8 * (par * 2 + s));
+            for (int q = 0; q < 4; ++q) {
+                uint32_t v = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v |= (uint32_t)(kg * 16 + 4 * q + e < blocks ? src[4 * q + e] : 127u) << (8 * e);
+                w[q] = v;
+            }
         }
-    ((uint32_t*)out)[d] = w;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ((uint32_t*)lds[sub])[t * 4 + q] = w[q];
+    }
+    __syncthreads();
+    if (live) {
+        const int pair = t >> 5, r16 = (t >> 1) & 15;
+        uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int st = e & 1, par = (e >> 1) & 1, jp = (e >> 2) & 1, g = (t & 1) * 2 + (e >> 3);
+            const int row = 32 * jp + 8 * (r16 >> 2) + 4 * par + (r16 & 3);
+            w[e >> 2] |= (uint32_t)lds[sub][row * 16 + pair * 8 + st * 4 + g] << (8 * (e & 3));
+        }
+        *(v4i*)(out + (unit << 10) + t * 16) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    }
 }
 
 // 127 everywhere (tiled layout), for producers that then write only the real (row, block) positions.

@@ -50,7 +50,7 @@ constexpr int PERSIST_LDS_BYTES_MX = GEMM_LDS_BYTES_MX;
 #define A8W8_PERSIST_BLK_LAG 4
 #endif
 #ifndef A8W8_BLK_SB
-#define A8W8_BLK_SB 1
+#define A8W8_BLK_SB 2
 #endif
 #if A8W8_BLK_SB == 1
 #define A8W8_BLK_SCHED_BARRIER() __builtin_amdgcn_sched_barrier(0)

@@ -146,6 +146,10 @@ A8W8_API int a8w8_quantize(const float* src_dev, int rows, int k, int ld, uint8_
  * scales can be produced in this layout directly by a8w8_quantize. */
 A8W8_API int a8w8_mx_tile_scales(const uint8_t* sf_dev, int rows, int k, int stride, uint8_t* out_dev,
                                  void* hip_stream);
+/* Both scale arrays of one GEMM in a single launch (sfa [m][k/32] -> out_a, sfb [n][k/32] -> out_b). */
+A8W8_API int a8w8_mx_tile_scales_ab(const uint8_t* sfa_dev, int m, int stride_sfa, uint8_t* out_a_dev,
+                                    const uint8_t* sfb_dev, int n, int stride_sfb, uint8_t* out_b_dev, int k,
+                                    void* hip_stream);
 A8W8_API size_t a8w8_mx_tiled_bytes(int rows, int k);
 
 A8W8_API const char* a8w8_status_string(int status);

@@ -34,6 +34,15 @@ def test_tile_scales_kernel_matches_oracle(orc, rows, k):
     assert (got == orc.mx_tile_scales(wide[:, : k // 32])).all()
 
 
+def test_both_arrays_in_one_launch(orc):
+    rng = np.random.Generator(np.random.Philox(99))
+    ea = rng.integers(0, 255, (130, 24), dtype=np.uint8)
+    eb = rng.integers(0, 255, (520, 24), dtype=np.uint8)
+    ta, tb = g.mx_tile_scales_ab(dev(ea), dev(eb))
+    assert (ta.cpu().numpy() == orc.mx_tile_scales(ea)).all()
+    assert (tb.cpu().numpy() == orc.mx_tile_scales(eb)).all()
+
+
 @pytest.mark.parametrize("rows,k", [(128, 512), (70, 384), (300, 1024)])
 def test_quantize_writes_the_tiled_layout(orc, rows, k):
     rng = np.random.Generator(np.random.Philox(41 + rows))
