@@ -146,7 +146,7 @@ __global__ void __launch_bounds__(256) quant_rowwise_kernel(const float* src, in
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
     __syncthreads();
     amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
-    const float s = __fdiv_rn(amax, 448.0f);
+    const float s = amax > 0.f ? __fdiv_rn(amax, 448.0f) : 1.0f;   // an all-zero group keeps scale 1
     if (threadIdx.x == 0) scale[row] = s;
     for (int i = threadIdx.x; i < k; i += 256) q[(long long)row * k + i] = quant_one(x[i], s);
 }
@@ -163,7 +163,7 @@ __global__ void __launch_bounds__(256) quant_1x128_kernel(const float* src, int 
     const float* x = src + (long long)row * ld + g * 128;
     const float v0 = x[lane], v1 = x[lane + 64];
     const float amax = wave_max(fmaxf(fabsf(v0), fabsf(v1)));
-    const float s = __fdiv_rn(amax, 448.0f);
+    const float s = amax > 0.f ? __fdiv_rn(amax, 448.0f) : 1.0f;   // an all-zero group keeps scale 1
     if (lane == 0) scale[(long long)g * rows + row] = s;
     uint8_t* o = q + (long long)row * k + g * 128;
     o[lane] = quant_one(v0, s);
@@ -182,7 +182,7 @@ __global__ void __launch_bounds__(256) quant_128x128_kernel(const float* src, in
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
     __syncthreads();
     amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
-    const float s = __fdiv_rn(amax, 448.0f);
+    const float s = amax > 0.f ? __fdiv_rn(amax, 448.0f) : 1.0f;   // an all-zero group keeps scale 1
     if (threadIdx.x == 0) scale[(long long)gr * gridDim.x + gk] = s;
     uint8_t* o = q + (long long)gr * 128 * k + gk * 128;
     for (int i = threadIdx.x; i < 128 * 128; i += 256)

@@ -68,6 +68,9 @@ def lib():
         L.orc_mx_tiled_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
         L.orc_mx_tile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
         L.orc_mx_untile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
+        L.orc_quant_rowwise.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p]
+        L.orc_quant_block.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p, ctypes.c_int]
+        L.orc_quant_mx.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _u8p]
         L.orc_flatmm_ref.argtypes = [_u8p, _u8p, _f32p, _f32p, _f32p] + [ctypes.c_int] * 5
         L.orc_count_abs_mismatch.restype = ctypes.c_long
         L.orc_count_abs_mismatch.argtypes = [_f32p, _f32p, ctypes.c_size_t, ctypes.c_float]
@@ -224,6 +227,25 @@ def mx_untile_scales(tiled, rows, k):
     out = np.zeros((rows, k // 32), np.uint8)
     lib().orc_mx_untile_scales(_p(tiled, _u8p), rows, k, k // 32, _p(out, _u8p))
     return out
+
+
+def quantize(x, mode, group_rows=1):
+    """fp32 [rows, k] -> (E4M3 bytes, scales in the layout gemm_ref reads for `mode`)."""
+    x = _c(x, np.float32)
+    rows, k = x.shape
+    q = np.empty((rows, k), np.uint8)
+    if mode == ROWCOL:
+        s = np.empty(rows, np.float32)
+        lib().orc_quant_rowwise(_p(x, _f32p), rows, k, k, _p(q, _u8p), _p(s, _f32p))
+    elif mode == BLOCK:
+        s = np.empty((k // 128, rows) if group_rows == 1 else (rows // 128, k // 128), np.float32)
+        lib().orc_quant_block(_p(x, _f32p), rows, k, k, _p(q, _u8p), _p(s, _f32p), group_rows)
+    elif mode == MX:
+        s = np.empty((rows, k // 32), np.uint8)
+        lib().orc_quant_mx(_p(x, _f32p), rows, k, k, _p(q, _u8p), _p(s, _u8p))
+    else:
+        raise ValueError(mode)
+    return q, s
 
 
 def flatmm_ref(a, bshuf, sfa, sfb, n):

@@ -22,6 +22,10 @@
  *   orc_gemm_ref / orc_gemm_ref_mx   brute force in float64 on tiny shapes,
  *       exact-integer inputs, scale-mode reductions.
  *   orc_preshuffle_b       bijection + flatmm(A, shuffle(B)) == gemm(A, B).
+ *   orc_quant_*            no reference code (its harness has no quantiser): the recipe of the
+ *       benchmark configurations, fixed by properties -- the group's largest element maps to
+ *       +-448 (row/block) or into (224, 448] (MX, never saturating), dequantisation error within
+ *       half an E4M3 ulp of every element, scale = amax/448 exactly, layouts as gemm_ref reads them.
  *   orc_mx_tile_scales     a layout this library defines (the reference has no MXFP8
  *       program): written as a walk over the layout's dimensions, i.e. the inverse of
  *       the index formula the kernels use; bijection on full blocks, padding = 127,
@@ -410,6 +414,66 @@ ORC_API void orc_flatmm_ref(const uint8_t* a, const uint8_t* bshuf, const float*
             c[(size_t)i * ldc + j] = sum;
         }
     }
+}
+
+/* ------------------------------------------------------------ quantisation front end
+ * The recipe the benchmark configurations state: scale = amax(group)/448, q = E4M3-OCP(x / scale)
+ * with round-to-nearest-even and saturation; group = a row (per token / per channel), a 1 x 128
+ * block (A-side block scales, stored [k/128][rows] as gemm_a8w8_blockscale_host.cc:78 indexes
+ * them) or a 128 x 128 block (B side, stored [rows/128][k/128], host.cc:79).  The reference has no
+ * quantiser (its harness casts uniform random floats, host.cc:32-44); an all-zero group keeps
+ * scale 1 so that it dequantises to zeros instead of 0/0. */
+static float group_scale(float amax) { return amax > 0.0f ? amax / 448.0f : 1.0f; }
+
+ORC_API void orc_quant_rowwise(const float* x, int rows, int k, int ld, uint8_t* q, float* scale)
+{
+    for (int r = 0; r < rows; ++r) {
+        float amax = 0.0f;
+        for (int p = 0; p < k; ++p) amax = fmaxf(amax, fabsf(x[(size_t)r * ld + p]));
+        const float s = group_scale(amax);
+        scale[r] = s;
+        for (int p = 0; p < k; ++p) q[(size_t)r * k + p] = orc_e4m3_ocp_encode(x[(size_t)r * ld + p] / s);
+    }
+}
+
+ORC_API void orc_quant_block(const float* x, int rows, int k, int ld, uint8_t* q, float* scale, int group_rows)
+{
+    const int gk = k / 128;
+    for (int r0 = 0; r0 < rows; r0 += group_rows)
+        for (int g = 0; g < gk; ++g) {
+            float amax = 0.0f;
+            for (int r = r0; r < r0 + group_rows; ++r)
+                for (int p = 0; p < 128; ++p) amax = fmaxf(amax, fabsf(x[(size_t)r * ld + g * 128 + p]));
+            const float s = group_scale(amax);
+            if (group_rows == 1) scale[(size_t)g * rows + r0] = s;
+            else scale[(size_t)(r0 / group_rows) * gk + g] = s;
+            for (int r = r0; r < r0 + group_rows; ++r)
+                for (int p = 0; p < 128; ++p)
+                    q[(size_t)r * k + g * 128 + p] = orc_e4m3_ocp_encode(x[(size_t)r * ld + g * 128 + p] / s);
+        }
+}
+
+/* MX: e = clamp(ceil(log2(amax/448)), -127, 127), byte e + 127, q = E4M3-OCP(x * 2^-e).  The ceiling
+ * means the largest element never saturates (|x| 2^-e <= 448).  ceil(log2 t) is taken exactly:
+ * the binary exponent of t, plus one unless t is a power of two. */
+ORC_API void orc_quant_mx(const float* x, int rows, int k, int ld, uint8_t* q, uint8_t* scale)
+{
+    for (int r = 0; r < rows; ++r)
+        for (int g = 0; g < k / 32; ++g) {
+            float amax = 0.0f;
+            for (int p = 0; p < 32; ++p) amax = fmaxf(amax, fabsf(x[(size_t)r * ld + g * 32 + p]));
+            const float t = amax / 448.0f;
+            int e = -127;
+            if (t > 0.0f) {
+                e = ilogbf(t);
+                if (t > ldexpf(1.0f, e)) ++e;
+                if (e < -127) e = -127;
+                if (e > 127) e = 127;
+            }
+            scale[(size_t)r * (k / 32) + g] = (uint8_t)(e + 127);
+            for (int p = 0; p < 32; ++p)
+                q[(size_t)r * k + g * 32 + p] = orc_e4m3_ocp_encode(ldexpf(x[(size_t)r * ld + g * 32 + p], -e));
+        }
 }
 
 /* valid_vector, gemm_a8w8_blockscale_host.cc:46-63: count of elements whose absolute
