@@ -242,22 +242,34 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     int mx_sa[TM], mx_sb[TN], mx_sa_next[TM], mx_sb_next[TN];
     v2i mxt_a, mxt_a_next;      // tiled MX: dword t/2 serves tiles t, t^1 and both steps of a pair
     v4i mxt_b, mxt_b_next;
+    __amdgpu_buffer_rsrc_t blk_rs;                  // block scales of the tile whose scales are being fetched
+    const float* blk_sfb_row = nullptr;
+    int blk_voff[TM] = {0, 0, 0, 0};
+    const int blk_sfa_step = p.stride_sfa * 4;
+    auto point_block_scales_at = [&](int batch, int mm0, int nn0) __attribute__((always_inline)) {
+        if constexpr (MODE == MODE_BLOCK) {
+            const float* sfa_f = (const float*)p.sfa + (long long)batch * p.sfa_batch;
+            const float* sfb_f = (const float*)p.sfb + (long long)batch * p.sfb_batch;
+            blk_rs = make_rsrc(sfa_f, (uint32_t)((nk - 1) * p.stride_sfa + p.m) * 4u);
+            const int nb = min(nn0 + wave_n * WAVE_N, p.n - 1) >> 7;
+            blk_sfb_row = sfb_f + (long long)nb * p.stride_sfb;
+            const int row0 = mm0 + wave_m * WAVE_M + r16;
+#pragma unroll
+            for (int t = 0; t < TM; ++t) blk_voff[t] = min(row0 + 16 * t, p.m - 1) * 4;
+        }
+    };
     auto fetch_step_scales = [&](int batch, int mm0, int nn0, int kstep, int gbase) __attribute__((always_inline)) {
         (void)gbase;
         if constexpr (MODE == MODE_BLOCK) {
-            // A-row scales through a buffer descriptor: 32-bit lane offsets instead of 64-bit pointers
-            const float* sfa_f = (const float*)p.sfa + (long long)batch * p.sfa_batch;
-            const float* sfb_f = (const float*)p.sfb + (long long)batch * p.sfb_batch;
-            const __amdgpu_buffer_rsrc_t rs =
-                make_rsrc(sfa_f, (uint32_t)((nk - 1) * p.stride_sfa + p.m) * 4u);
-            const int nb = min(nn0 + wave_n * WAVE_N, p.n - 1) >> 7;
-            const float sb = sfb_f[(long long)nb * p.stride_sfb + kstep];
-            const int row0 = mm0 + wave_m * WAVE_M + r16;
+            // A-row scales through a buffer descriptor (32-bit lane offsets instead of 64-bit pointers).
+            // Descriptor, B-scale row and lane offsets change only with the tile: they are set up by
+            // point_block_scales_at, so that a K step spends a handful of scalar instructions here.
+            (void)batch; (void)mm0; (void)nn0;
+            const float sb = blk_sfb_row[kstep];
 #pragma unroll
             for (int t = 0; t < TM; ++t)
                 blk_s_next[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                                              rs, min(row0 + 16 * t, p.m - 1) * 4,
-                                                              kstep * p.stride_sfa * 4, 0)) * sb;
+                                                              blk_rs, blk_voff[t], kstep * blk_sfa_step, 0)) * sb;
         }
         if constexpr (MODE == MODE_MX) {
             // one dword per (row, K step) holds the four block exponents; lane group g extracts
@@ -401,7 +413,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     advance_ld();
 #pragma unroll
     for (int w = 0; w < 8; ++w) issue_one(1, ld_ks, w);
-    if constexpr (MODE == MODE_BLOCK) fetch_step_scales(cur_batch, m0, n0, 0, 0);
+    if constexpr (MODE == MODE_BLOCK) {
+        point_block_scales_at(cur_batch, m0, n0);
+        fetch_step_scales(cur_batch, m0, n0, 0, 0);
+    }
     __builtin_amdgcn_s_waitcnt(0);
     A8W8_RAW_BARRIER();
     if constexpr (IS_MX) fetch_step_scales(cur_batch, m0, n0, 0, 0);
@@ -436,6 +451,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             nx_m0 = tm * BM;
             nx_n0 = tn * BN;
             nx_gbase = cur_gbase + groups_per_tile;
+            point_block_scales_at(nx_batch, nx_m0, nx_n0);   // the fetch at group 2 is for the next tile's step 0
         }
 
         v8i fb[TN];
