@@ -4,7 +4,9 @@
 //   gemm_a8w8_blockscale.exe -b 1 -m 4096 -n 4096 -k 4096 -v 1
 // finds the same command line and the same lines of output.  One source builds three programs:
 //   gemm_a8w8_blockscale.exe   1x128 / 128x128 block scales, fp32 C (the reference program)
-//   gemm_a8w8_8wave.exe        dense GEMM, --scale-mode tensor|rowcol|mx, bf16 C
+//   gemm_a8w8_8wave.exe        dense GEMM, --scale-mode tensor|rowcol|mx|mxt, bf16 C
+//                              (mxt: the row-major MX scales are re-ordered into the tiled layout
+//                              inside the timed loop, then the GEMM runs on the tiled scales)
 //   flatmm_a8w8.exe            skinny-M GEMM over pre-shuffled weights, bf16 C
 // This is test infrastructure: validation (-v 1) calls the CPU oracle, exactly as the
 // reference program calls its own gemm_ref (host.cc:260-281).
@@ -208,7 +210,7 @@ int main(int argc, char** argv)
     int mode = A8W8_SCALE_ROWCOL;
     if (HARNESS_KIND == 0 || scale_mode == "block") mode = A8W8_SCALE_BLOCK_1x128_128x128;
     else if (scale_mode == "tensor") mode = A8W8_SCALE_TENSOR;
-    else if (scale_mode == "mx") mode = A8W8_SCALE_MX_E8M0_1x32;
+    else if (scale_mode == "mx" || scale_mode == "mxt") mode = A8W8_SCALE_MX_E8M0_1x32;
     else if (scale_mode != "rowcol") { fprintf(stderr, "unknown --scale-mode %s\n", scale_mode.c_str()); return 1; }
     if (mode == A8W8_SCALE_BLOCK_1x128_128x128 && (N % 128 != 0 || K % 128 != 0)) {
         fprintf(stderr, "M/N/K must be multiples of GROUP_M/GROUP_N/GROUP_K (1,128,128) for scale factors.\n");
@@ -277,9 +279,27 @@ int main(int argc, char** argv)
     CHECK_HIP(hipMalloc(&dev_c, c_bytes));
     args.a = dev_a; args.b = dev_b_copies[0]; args.c = dev_c; args.sfa = dev_sfa; args.sfb = dev_sfb;
 
+    // mxt: tiled copies of the scales, rebuilt from the row-major arrays by every launch
+    const bool tiled = scale_mode == "mxt";
+    uint8_t *dev_ta = nullptr, *dev_tb = nullptr;
+    const size_t ta_bytes = tiled ? a8w8_mx_tiled_bytes(M, K) : 0, tb_bytes = tiled ? a8w8_mx_tiled_bytes(N, K) : 0;
+    if (tiled) {
+        CHECK_HIP(hipMalloc(&dev_ta, ta_bytes * batch));
+        CHECK_HIP(hipMalloc(&dev_tb, tb_bytes * batch));
+    }
     auto launch = [&](int i) {
         a8w8_gemm_args local = args;
         local.b = dev_b_copies[(size_t)i % dev_b_copies.size()];
+        if (tiled) {
+            for (int b = 0; b < batch; ++b)
+                CHECK_A8W8(a8w8_mx_tile_scales_ab((const uint8_t*)dev_sfa + (size_t)b * args.stride_sfa_batch, M, K / 32,
+                                                  dev_ta + b * ta_bytes,
+                                                  (const uint8_t*)dev_sfb + (size_t)b * args.stride_sfb_batch, N, K / 32,
+                                                  dev_tb + b * tb_bytes, K, nullptr));
+            local.scale_mode = A8W8_SCALE_MX_E8M0_TILED;
+            local.sfa = dev_ta; local.sfb = dev_tb;
+            local.stride_sfa_batch = (int)ta_bytes; local.stride_sfb_batch = (int)tb_bytes;
+        }
         if (HARNESS_KIND == 0) CHECK_A8W8(a8w8_gemm_blockscale(&local, nullptr));
         else if (HARNESS_KIND == 1) CHECK_A8W8(a8w8_gemm(&local, nullptr));
         else CHECK_A8W8(a8w8_flatmm(&local, nullptr));

@@ -42,7 +42,7 @@ def test_blockscale_program_default_problem_and_flags():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("mode", ["tensor", "rowcol", "mx"])
+@pytest.mark.parametrize("mode", ["tensor", "rowcol", "mx", "mxt"])
 def test_dense_program(mode):
     r = _run("gemm_a8w8_8wave.exe", "-m", "512", "-n", "768", "-k", "512", "-v", "1", "--scale-mode", mode)
     assert r.returncode == 0, r.stdout + r.stderr
