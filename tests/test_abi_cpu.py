@@ -84,6 +84,28 @@ def test_kernel_selection():
     assert g.kernel_name(a) == "gemm_a8w8_general"
 
 
+def test_tiled_mx_mode_selection_and_reorder_preconditions():
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED)) == "gemm_a8w8_persist"
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=384)) == "gemm_a8w8_general"      # odd number of K steps
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=128)) == "gemm_a8w8_general"
+    a = _ok_args(mode=g.MX_TILED, k=48)
+    assert g.lib().a8w8_gemm(ctypes.byref(a), None) == -3
+    a = _ok_args(mode=g.MX_TILED)
+    a.sfa = 0x4004                                                                      # tiled scales need 16-byte alignment
+    assert g.kernel_name(a) == "gemm_a8w8_general"
+    L = g.lib()
+    assert L.a8w8_mx_tiled_bytes(64, 512) == 1024 and L.a8w8_mx_tiled_bytes(65, 513) == 4096
+    assert L.a8w8_mx_tiled_bytes(0, 512) == 0
+    assert g.mx_tiled_bytes(8192, 8192) == 8192 * 256 == L.a8w8_mx_tiled_bytes(8192, 8192)
+    assert L.a8w8_mx_tile_scales(None, 64, 512, 16, 0x1000, None) == -1
+    assert L.a8w8_mx_tile_scales(0x1000, 0, 512, 16, 0x2000, None) == -2
+    assert L.a8w8_mx_tile_scales(0x1000, 64, 500, 16, 0x2000, None) == -3
+    assert L.a8w8_mx_tile_scales(0x1000, 64, 512, 8, 0x2000, None) == -4
+    assert L.a8w8_mx_tile_scales(0x1000, 64, 512, 16, 0x2004, None) == -5
+    assert L.a8w8_mx_tile_scales_ab(0x1000, 64, 16, 0x2000, None, 64, 16, 0x3000, 512, None) == -1
+    assert L.a8w8_mx_tile_scales_ab(0x1000, 64, 16, 0x2000, 0x4000, 64, 8, 0x3000, 512, None) == -4
+
+
 def test_good_arguments_pass_validation_and_stop_at_the_device():
     import torch
     if torch.cuda.is_available():
