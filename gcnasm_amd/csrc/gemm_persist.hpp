@@ -59,6 +59,9 @@ constexpr int PERSIST_LDS_BYTES_MX = GEMM_LDS_BYTES_MX;
 #else
 #define A8W8_BLK_SCHED_BARRIER() (void)0
 #endif
+#ifndef A8W8_PERSIST_SG
+#define A8W8_PERSIST_SG 2
+#endif
 #ifndef A8W8_PERSIST_SB
 #define A8W8_PERSIST_SB 0
 #endif
@@ -498,6 +501,25 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                 }
             }
             A8W8_PERSIST_SCHED_BARRIER();
+#if A8W8_PERSIST_SG
+            if constexpr (MODE != MODE_BLOCK) {
+                // spread the two LDS reads of the next B fragment between this group's MFMAs
+                if (j + 1 < TN) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                } else if (A8W8_PERSIST_SG >= 2 && PREFETCH_FRAGS) {
+                    // the last group runs beside the next step's prefetched fragments
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, (2 * NPF + 2 + 3) / 4, 0);
+                    }
+                }
+            }
+#endif
 
             if (j == 0) issue_one(P ^ 1, ld_ks, 5);
             if (j == 1) issue_one(P ^ 1, ld_ks, 7);
