@@ -146,7 +146,9 @@ int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
     int dev = 0;
     (void)hipGetDevice(&dev);
     auto kern = gemm_a8w8_persist<MODE, CDT>;
-    constexpr int lds_bytes = (MODE == MODE_MX || MODE == MODE_MXT) ? PERSIST_LDS_BYTES_MX : PERSIST_LDS_BYTES;
+    constexpr int lds_bytes = (MODE == MODE_MX || MODE == MODE_MXT) ? PERSIST_LDS_BYTES_MX
+                              : MODE == MODE_ROWCOL                   ? PERSIST_LDS_BYTES_ROWCOL
+                                                                      : PERSIST_LDS_BYTES;
     if (!attr_set[dev & 63]) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
             return A8W8_ERR_LAUNCH;

@@ -29,6 +29,10 @@ namespace a8w8 {
 // LDS: two operand stages, then (MX only) two scale groups of 4 K steps.
 constexpr int PERSIST_LDS_BYTES = GEMM_LDS_BYTES;
 constexpr int PERSIST_LDS_BYTES_MX = GEMM_LDS_BYTES_MX;
+// row/col mode: two buffers of 256 A-row + 256 B-row fp32 scales (the tile being multiplied and the
+// one before it), filled by direct-to-LDS loads so that the epilogue waits on no global load
+constexpr int ROWCOL_SCALE_BYTES = (BM + BN) * 4;
+constexpr int PERSIST_LDS_BYTES_ROWCOL = GEMM_LDS_BYTES + 2 * ROWCOL_SCALE_BYTES;
 
 #define A8W8_RAW_BARRIER() asm volatile("s_barrier" ::: "memory")
 // How many of the next step's four A fragments (plus the first B fragment) are fetched from LDS in
@@ -169,6 +173,20 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             A8W8_LDS char* s =
                 (A8W8_LDS char*)smem + GEMM_LDS_BYTES + ((ld_gbase + group) & 1) * MX_GROUP_BYTES + wave * 1024;
             load_to_lds_16(rsrc_sf, s, voff_sf, group * sf_group_stride);
+        }
+    };
+    int tile_seq = 0;                               // tiles this workgroup has started: picks the scale buffer
+    auto issue_rowcol_scales = [&](int batch, int mm0, int nn0) __attribute__((always_inline)) {
+        if constexpr (MODE == MODE_ROWCOL) {
+            // thread t < 256 fetches sfa[m0 + t], the others sfb[n0 + t - 256] (row indices clamped)
+            const bool is_b = wave >= 4;
+            const int rows = is_b ? p.n : p.m;
+            const float* base = is_b ? (const float*)p.sfb + (long long)batch * p.sfb_batch
+                                     : (const float*)p.sfa + (long long)batch * p.sfa_batch;
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc(base, (uint32_t)rows * 4u);
+            const int voff = min((is_b ? nn0 : mm0) + (wave & 3) * 64 + lane, rows - 1) * 4;
+            A8W8_LDS char* s = (A8W8_LDS char*)smem + GEMM_LDS_BYTES + (tile_seq & 1) * ROWCOL_SCALE_BYTES + wave * 256;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, s, 4, voff, 0, 0, 0);
         }
     };
     auto advance_ld = [&]() __attribute__((always_inline)) {                      // the load position moves one K step
@@ -322,33 +340,24 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         float sa[TM];
         float ts = 1.f;
         if constexpr (MODE == MODE_TENSOR) ts = sfa_f[0] * sfb_f[0];
-        if constexpr (MODE == MODE_ROWCOL) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i) sa[i] = sfa_f[min(cm_of(i), p.m - 1)];
-        }
         char* c_base = (char*)p.c + (long long)cur_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
         const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 7) == 0 && (((uintptr_t)c_base) & 15) == 0)
                                             : ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 15) == 0);
-        // every scale is fetched before the first store: a wait for a load issued after a store would
-        // also wait for that store to be acknowledged (one counter, in issue order)
+        // row/col scales were staged in LDS when the tile began (issue_rowcol_scales): reading them
+        // waits on no global load, and a wait for a load issued after a store would also wait for
+        // that store to be acknowledged (one counter, in issue order)
         float sb[TN / 2][8];
         if constexpr (MODE == MODE_ROWCOL) {
-            const bool sfb_vec = (((uintptr_t)sfb_f) & 15) == 0;
+            const float* sc = (const float*)(smem + GEMM_LDS_BYTES + (tile_seq & 1) * ROWCOL_SCALE_BYTES);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) sa[i] = sc[cm_of(i) - m0];
 #pragma unroll
             for (int jp = 0; jp < TN / 2; ++jp) {
-                const int cn = cn_base + 32 * jp;
-                if (sfb_vec && cn + 7 < p.n) {
-                    const v4f lo = *(const v4f*)(sfb_f + cn), hi = *(const v4f*)(sfb_f + cn + 4);
+                const v4f lo = *(const v4f*)(sc + BM + (cn_base - n0) + 32 * jp), hi = *(const v4f*)(sc + BM + (cn_base - n0) + 32 * jp + 4);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) { sb[jp][e] = lo[e]; sb[jp][4 + e] = hi[e]; }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) sb[jp][e] = sfb_f[min(cn + e, p.n - 1)];
-                }
+                for (int e = 0; e < 4; ++e) { sb[jp][e] = lo[e]; sb[jp][4 + e] = hi[e]; }
             }
         }
-        // ... and waited for here, once, so that no wait ends up between the stores
-        if constexpr (MODE == MODE_ROWCOL) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
 #pragma unroll
         for (int jp = 0; jp < TN / 2; ++jp) {
             const int cn = cn_base + 32 * jp;
@@ -420,6 +429,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         point_block_scales_at(cur_batch, m0, n0);
         fetch_step_scales(cur_batch, m0, n0, 0, 0);
     }
+    issue_rowcol_scales(cur_batch, m0, n0);
     __builtin_amdgcn_s_waitcnt(0);
     A8W8_RAW_BARRIER();
     if constexpr (IS_MX) fetch_step_scales(cur_batch, m0, n0, 0, 0);
@@ -563,6 +573,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             m0 = nx_m0;
             n0 = nx_n0;
             cur_gbase = nx_gbase;
+            if constexpr (MODE == MODE_ROWCOL) ++tile_seq;
+            // the next tile's row/col scales: in flight from here, landed (and past a barrier) long
+            // before its epilogue; the end barrier's "all but the newest four loads" covers it
+            issue_rowcol_scales(cur_batch, m0, n0);
         } else {
             ++cur_ks;
         }

@@ -106,6 +106,25 @@ def test_tiled_mx_mode_selection_and_reorder_preconditions():
     assert L.a8w8_mx_tile_scales_ab(0x1000, 64, 16, 0x2000, 0x4000, 64, 8, 0x3000, 512, None) == -4
 
 
+def test_pipelined_kernels_use_no_scratch():
+    """The build keeps the compiler's per-kernel resource report.  A register spilled inside the K loop
+    of the persistent GEMM is reloaded behind a wait for every direct-to-LDS load in flight (the reload
+    and the loads share one in-order counter), which costs tens of percent: none may spill."""
+    path = os.path.join(ROOT, "gcnasm_amd", "libmi355a8w8.resources.txt")
+    if not os.path.exists(path):
+        pytest.skip("resource report not written by this build of the library")
+    text = open(path).read()
+    blocks = text.split("Function Name: ")[1:]
+    seen = 0
+    for b in blocks:
+        name = b.split()[0]
+        if "gemm_a8w8_persist" in name or "flatmm_a8w8" in name:
+            seen += 1
+            scratch = int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1))
+            assert scratch == 0, (name, scratch)
+    assert seen >= 10
+
+
 def test_good_arguments_pass_validation_and_stop_at_the_device():
     import torch
     if torch.cuda.is_available():
