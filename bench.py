@@ -64,14 +64,12 @@ def make_inputs(name, torch, g, seed):
         a, sfa = g.quantize(normal(m), g.BLOCK, 1)
         b, sfb = g.quantize(normal(n), g.BLOCK, 128)
         return dict(a=a, b=b, sfa=sfa, sfb=sfb, mode=g.BLOCK)
+    if mode == "tensor":
+        a, sfa = g.quantize(normal(m), g.TENSOR)
+        b, sfb = g.quantize(normal(n), g.TENSOR)
+        return dict(a=a, b=b, sfa=sfa, sfb=sfb, mode=g.TENSOR)
     a, sfa = g.quantize(normal(m), g.ROWCOL)
     b, sfb = g.quantize(normal(n), g.ROWCOL)
-    if mode == "tensor":
-        # one scale per tensor: requantise with the largest row scale
-        sa, sb = sfa.max().reshape(1), sfb.max().reshape(1)
-        a = g.cvt_f32_to_e4m3(g.cvt_e4m3_to_f32(a) * (sfa[:, None] / sa))
-        b = g.cvt_f32_to_e4m3(g.cvt_e4m3_to_f32(b) * (sfb[:, None] / sb))
-        return dict(a=a, b=b, sfa=sa.contiguous(), sfb=sb.contiguous(), mode=g.TENSOR)
     if mode == "flat":
         return dict(a=a, b=b, sfa=sfa, sfb=sfb, mode=g.ROWCOL, bshuf=g.preshuffle_b_device(b))
     return dict(a=a, b=b, sfa=sfa, sfb=sfb, mode=g.ROWCOL)

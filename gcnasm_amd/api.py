@@ -225,7 +225,9 @@ def quantize(x, scale_mode, group_rows=1):
     import torch
     rows, k = x.shape
     q = torch.empty((rows, k), dtype=torch.uint8, device=x.device)
-    if scale_mode == ROWCOL:
+    if scale_mode == TENSOR:
+        s = torch.empty(1, dtype=torch.float32, device=x.device)
+    elif scale_mode == ROWCOL:
         s = torch.empty(rows, dtype=torch.float32, device=x.device)
     elif scale_mode == BLOCK and group_rows == 1:
         s = torch.empty((k // 128, rows), dtype=torch.float32, device=x.device)

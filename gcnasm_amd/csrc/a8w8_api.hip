@@ -343,6 +343,16 @@ int a8w8_quantize(const float* src, int rows, int k, int ld, uint8_t* q, void* s
     if (ld < k) return A8W8_ERR_BAD_STRIDE;
     hipStream_t s = (hipStream_t)hip_stream;
     switch (scale_mode) {
+        case A8W8_SCALE_TENSOR: {
+            if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+            const long long total = (long long)rows * k;
+            const unsigned grid = (unsigned)(total / 256 + 1 < 4096 ? total / 256 + 1 : 4096);
+            hipLaunchKernelGGL(quant_tensor_clear_kernel, dim3(1), dim3(1), 0, s, (float*)scale);
+            hipLaunchKernelGGL(quant_tensor_amax_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, (float*)scale);
+            hipLaunchKernelGGL(quant_tensor_apply_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, q, (const float*)scale);
+            hipLaunchKernelGGL(quant_tensor_finish_kernel, dim3(1), dim3(1), 0, s, (float*)scale);
+            return launch_status();
+        }
         case A8W8_SCALE_ROWCOL:
             if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
             hipLaunchKernelGGL(quant_rowwise_kernel, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);

@@ -151,6 +151,40 @@ __global__ void __launch_bounds__(256) quant_rowwise_kernel(const float* src, in
     for (int i = threadIdx.x; i < k; i += 256) q[(long long)row * k + i] = quant_one(x[i], s);
 }
 
+// per-tensor scale = amax(all)/448 in three steps over the caller's one-float scale slot: clear it, fold
+// every workgroup's |x| maximum into it (non-negative floats order like their bit patterns), quantise with
+// amax/448, and finally turn the slot from amax into the scale.
+__global__ void quant_tensor_clear_kernel(float* scale) { *scale = 0.f; }
+__global__ void __launch_bounds__(256) quant_tensor_amax_kernel(const float* src, int rows, int k, int ld, float* scale)
+{
+    __shared__ float part[4];
+    const long long total = (long long)rows * k;
+    float amax = 0.f;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256)
+        amax = fmaxf(amax, fabsf(src[(i / k) * ld + i % k]));
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+        atomicMax((unsigned int*)scale, __float_as_uint(amax));
+    }
+}
+__global__ void __launch_bounds__(256) quant_tensor_apply_kernel(const float* src, int rows, int k, int ld, uint8_t* q,
+                                                                 const float* amax_slot)
+{
+    const long long total = (long long)rows * k;
+    const float amax = *amax_slot;
+    const float s = amax > 0.f ? __fdiv_rn(amax, 448.0f) : 1.0f;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256)
+        q[i] = quant_one(src[(i / k) * ld + i % k], s);
+}
+__global__ void quant_tensor_finish_kernel(float* scale)
+{
+    const float amax = *scale;
+    *scale = amax > 0.f ? __fdiv_rn(amax, 448.0f) : 1.0f;
+}
+
 // 1 x 128 blocks: one wave per (row, 128-group); scale stored [k/128][rows]
 __global__ void __launch_bounds__(256) quant_1x128_kernel(const float* src, int rows, int k, int ld, uint8_t* q,
                                                           float* scale)

@@ -135,8 +135,9 @@ A8W8_API size_t a8w8_cvt_e4m3_to_f32(const uint8_t* src_dev, float* dst_dev, siz
  *           group_rows = 128 -> scale[(r/128)*(k/128) + p/128] (the SFB layout)
  *   MX    : uint8 e = clamp(ceil(log2(amax32/448)), -127, 127) + 127 at scale[r*(k/32) + p/32]
  *   MX_TILED : the same bytes at their MX_TILED positions (a8w8_mx_tiled_bytes(rows, k) bytes)
- * TENSOR needs a grid-wide reduction first and is provided as ROWCOL followed by the
- * caller's own max; it returns A8W8_ERR_BAD_MODE here. */
+ *   TENSOR: scale[0] = amax(all)/448 (four small launches; the scale slot holds the running amax
+ *           in between, so it must not be read until the stream reaches the end of the call)
+ * An all-zero group keeps scale 1 (E8M0 byte 0 for MX). */
 A8W8_API int a8w8_quantize(const float* src_dev, int rows, int k, int ld, uint8_t* q_dev, void* scale_dev,
                            int scale_mode, int group_rows, void* hip_stream);
 

@@ -68,6 +68,7 @@ def lib():
         L.orc_mx_tiled_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
         L.orc_mx_tile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
         L.orc_mx_untile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
+        L.orc_quant_tensor.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p]
         L.orc_quant_rowwise.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p]
         L.orc_quant_block.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p, ctypes.c_int]
         L.orc_quant_mx.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _u8p]
@@ -234,7 +235,10 @@ def quantize(x, mode, group_rows=1):
     x = _c(x, np.float32)
     rows, k = x.shape
     q = np.empty((rows, k), np.uint8)
-    if mode == ROWCOL:
+    if mode == TENSOR:
+        s = np.empty(1, np.float32)
+        lib().orc_quant_tensor(_p(x, _f32p), rows, k, k, _p(q, _u8p), _p(s, _f32p))
+    elif mode == ROWCOL:
         s = np.empty(rows, np.float32)
         lib().orc_quant_rowwise(_p(x, _f32p), rows, k, k, _p(q, _u8p), _p(s, _f32p))
     elif mode == BLOCK:

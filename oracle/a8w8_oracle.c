@@ -436,6 +436,17 @@ ORC_API void orc_quant_rowwise(const float* x, int rows, int k, int ld, uint8_t*
     }
 }
 
+ORC_API void orc_quant_tensor(const float* x, int rows, int k, int ld, uint8_t* q, float* scale)
+{
+    float amax = 0.0f;
+    for (int r = 0; r < rows; ++r)
+        for (int p = 0; p < k; ++p) amax = fmaxf(amax, fabsf(x[(size_t)r * ld + p]));
+    const float s = group_scale(amax);
+    scale[0] = s;
+    for (int r = 0; r < rows; ++r)
+        for (int p = 0; p < k; ++p) q[(size_t)r * k + p] = orc_e4m3_ocp_encode(x[(size_t)r * ld + p] / s);
+}
+
 ORC_API void orc_quant_block(const float* x, int rows, int k, int ld, uint8_t* q, float* scale, int group_rows)
 {
     const int gk = k / 128;

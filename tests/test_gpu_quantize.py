@@ -25,6 +25,18 @@ def _run(x, mode, group_rows=1):
     return q.cpu().numpy(), s.cpu().numpy()
 
 
+@pytest.mark.parametrize("rows,k", [(1, 32), (37, 96), (300, 1024), (2048, 4096)])
+def test_per_tensor(orc, rows, k):
+    x = _x(rows, k, 5 + rows, wide=False)
+    q, s = _run(x, g.TENSOR)
+    qr, sr = orc.quantize(x, orc.TENSOR)
+    assert s.shape == (1,) and s.view(np.uint32)[0] == sr.view(np.uint32)[0]
+    assert (q == qr).all()
+    z = np.zeros((4, 64), np.float32)
+    q, s = _run(z, g.TENSOR)
+    assert s[0] == 1 and (q == 0).all()
+
+
 @pytest.mark.parametrize("rows,k", [(1, 32), (37, 96), (256, 512), (130, 7168)])
 def test_rowwise(orc, rows, k):
     x = _x(rows, k, 10 + rows)
@@ -87,7 +99,7 @@ def test_quantize_then_gemm_matches_oracle_pipeline(orc):
     """The bytes and scales a8w8_quantize writes feed a8w8_gemm directly, in every mode."""
     m, n, k = 256, 256, 512
     a, b = _x(m, k, 91, wide=False), _x(n, k, 92, wide=False)
-    for mode, ga, gb in ((g.ROWCOL, 1, 1), (g.BLOCK, 1, 128), (g.MX, 1, 1), (g.MX_TILED, 1, 1)):
+    for mode, ga, gb in ((g.TENSOR, 1, 1), (g.ROWCOL, 1, 1), (g.BLOCK, 1, 128), (g.MX, 1, 1), (g.MX_TILED, 1, 1)):
         qa, sa = g.quantize(dev(a), mode, ga)
         qb, sb = g.quantize(dev(b), mode, gb)
         c = g.gemm(qa, qb, sa, sb, mode, c_dtype=g.FP32).cpu().numpy()

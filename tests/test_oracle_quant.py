@@ -29,6 +29,18 @@ def test_rowwise_properties(orc):
     assert (np.sign(d) * np.sign(x) >= 0).all()
 
 
+def test_per_tensor_properties(orc):
+    x = _x(37, 256, 11)
+    q, s = orc.quantize(x, orc.TENSOR)
+    assert s.shape == (1,) and s[0] == np.abs(x).max() / np.float32(448)
+    d = orc.decode(q)
+    assert np.abs(d).max() == 448
+    assert (np.abs(d - x / s[0]) <= _half_step(x / s[0]) * 1.0001).all()
+    qr, sr = orc.quantize(x[:1], orc.ROWCOL)
+    qt, st = orc.quantize(x[:1], orc.TENSOR)                 # one row: both recipes coincide
+    assert (qr == qt).all() and sr[0] == st[0]
+
+
 def test_block_properties_and_layouts(orc):
     x = _x(256, 384, 2)
     q1, s1 = orc.quantize(x, orc.BLOCK, 1)
@@ -69,7 +81,7 @@ def test_mx_never_saturates_and_is_tight(orc):
 
 def test_all_zero_groups_stay_zero(orc):
     x = np.zeros((128, 256), np.float32)
-    for mode, gr in ((orc.ROWCOL, 1), (orc.BLOCK, 1), (orc.BLOCK, 128), (orc.MX, 1)):
+    for mode, gr in ((orc.TENSOR, 1), (orc.ROWCOL, 1), (orc.BLOCK, 1), (orc.BLOCK, 128), (orc.MX, 1)):
         q, s = orc.quantize(x, mode, gr)
         assert (q == 0).all()
         assert (s == (0 if mode == orc.MX else 1)).all()
@@ -79,7 +91,7 @@ def test_quantised_gemm_tracks_the_fp32_product(orc):
     """End to end: quantise, run the oracle GEMM on bytes + scales, compare with the fp32 matmul."""
     a, b = _x(64, 256, 4), _x(128, 256, 5)
     want = a.astype(np.float64) @ b.astype(np.float64).T
-    for mode, ga, gb in ((orc.ROWCOL, 1, 1), (orc.BLOCK, 1, 128), (orc.MX, 1, 1)):
+    for mode, ga, gb in ((orc.TENSOR, 1, 1), (orc.ROWCOL, 1, 1), (orc.BLOCK, 1, 128), (orc.MX, 1, 1)):
         qa, sa = orc.quantize(a, mode, ga)
         qb, sb = orc.quantize(b, mode, gb)
         got = orc.gemm_ref(qa, qb, sa, sb, mode)
