@@ -23,6 +23,13 @@ class A8W8Error(RuntimeError):
         super().__init__(f"{where}: {status_string(status)} (status {status})")
 
 
+class WeightHeader(ctypes.Structure):
+    _fields_ = [("magic", ctypes.c_char * 8), ("version", ctypes.c_uint32), ("n", ctypes.c_uint32), ("k", ctypes.c_uint32),
+                ("b_preshuffled", ctypes.c_uint32), ("scale_mode", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
+                ("b_bytes", ctypes.c_uint64), ("scale_bytes", ctypes.c_uint64), ("checksum", ctypes.c_uint64),
+                ("reserved2", ctypes.c_uint64)]
+
+
 class GemmArgs(ctypes.Structure):
     _fields_ = [
         ("a", ctypes.c_void_p), ("b", ctypes.c_void_p), ("c", ctypes.c_void_p),
@@ -77,6 +84,11 @@ def lib():
                                              ctypes.c_int, vp]
         L.a8w8_mx_tiled_bytes.restype = ctypes.c_size_t
         L.a8w8_mx_tiled_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
+        L.a8w8_weight_scale_bytes.restype = ctypes.c_size_t
+        L.a8w8_weight_scale_bytes.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        L.a8w8_weights_save.argtypes = [ctypes.c_char_p, vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        L.a8w8_weights_info.argtypes = [ctypes.c_char_p, ctypes.POINTER(WeightHeader)]
+        L.a8w8_weights_load.argtypes = [ctypes.c_char_p, vp, ctypes.c_size_t, vp, ctypes.c_size_t]
         L.a8w8_status_string.restype = ctypes.c_char_p
         L.a8w8_status_string.argtypes = [ctypes.c_int]
         L.a8w8_kernel_name.restype = ctypes.c_char_p
@@ -265,6 +277,28 @@ def mx_tile_scales_ab(sfa, sfb):
     _check(lib().a8w8_mx_tile_scales_ab(sfa.data_ptr(), m, sfa.stride(0), ta.data_ptr(), sfb.data_ptr(), n,
                                         sfb.stride(0), tb.data_ptr(), kb * 32, _stream()), "a8w8_mx_tile_scales_ab")
     return ta, tb
+
+
+def save_weights(path, b_np, scale_np, n, k, scale_mode, b_preshuffled=False):
+    """Write quantised weights (numpy uint8, row-major [n, k] or pre-shuffled flat) and their scales to a file."""
+    import numpy as np
+    b_np = np.ascontiguousarray(b_np, dtype=np.uint8)
+    scale_np = np.ascontiguousarray(scale_np)
+    assert b_np.size == n * k and scale_np.nbytes == lib().a8w8_weight_scale_bytes(n, k, scale_mode)
+    _check(lib().a8w8_weights_save(os.fsencode(path), b_np.ctypes.data, scale_np.ctypes.data, n, k, int(b_preshuffled),
+                                   scale_mode), "a8w8_weights_save")
+
+
+def load_weights(path):
+    """-> (header, weights uint8 array, scales array: float32, or uint8 for the MX modes)."""
+    import numpy as np
+    h = WeightHeader()
+    _check(lib().a8w8_weights_info(os.fsencode(path), ctypes.byref(h)), "a8w8_weights_info")
+    b = np.empty(h.b_bytes, np.uint8)
+    raw = np.empty(h.scale_bytes, np.uint8)
+    _check(lib().a8w8_weights_load(os.fsencode(path), b.ctypes.data, b.nbytes, raw.ctypes.data, raw.nbytes), "a8w8_weights_load")
+    scales = raw if h.scale_mode in (MX, MX_TILED) else raw.view(np.float32)
+    return h, (b if h.b_preshuffled else b.reshape(h.n, h.k)), scales
 
 
 def kernel_name(g):

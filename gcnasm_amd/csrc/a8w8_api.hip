@@ -2,6 +2,7 @@
 #include "../../include/mi355_a8w8.h"
 
 #include <hip/hip_runtime.h>
+#include <stdio.h>
 #include <string.h>
 
 #include "cvt.hpp"
@@ -436,6 +437,94 @@ size_t a8w8_mx_tiled_bytes(int rows, int k)
     return mx_tiled_bytes(rows, k);
 }
 
+// ------------------------------------------------------------ weight files (host only)
+namespace {
+const char kWeightMagic[8] = {'A', '8', 'W', '8', 'W', 'G', 'T', 0};
+
+uint64_t fnv1a64(const void* data, size_t n, uint64_t h)
+{
+    const uint8_t* p = (const uint8_t*)data;
+    for (size_t i = 0; i < n; ++i) { h ^= p[i]; h *= 1099511628211ull; }
+    return h;
+}
+
+int check_header(const a8w8_weight_header& h)
+{
+    if (memcmp(h.magic, kWeightMagic, 8) != 0 || h.version != 1) return A8W8_ERR_BAD_FILE;
+    if (h.n == 0 || h.k == 0 || h.n > (1u << 30) || h.k > (1u << 30)) return A8W8_ERR_BAD_FILE;
+    if (h.b_bytes != (uint64_t)h.n * h.k) return A8W8_ERR_BAD_FILE;
+    if (h.scale_bytes == 0 || h.scale_bytes != a8w8_weight_scale_bytes((int)h.n, (int)h.k, (int)h.scale_mode))
+        return A8W8_ERR_BAD_FILE;
+    return A8W8_OK;
+}
+}  // namespace
+
+size_t a8w8_weight_scale_bytes(int n, int k, int scale_mode)
+{
+    if (n <= 0 || k <= 0) return 0;
+    switch (scale_mode) {
+        case A8W8_SCALE_TENSOR: return 4;
+        case A8W8_SCALE_ROWCOL: return (size_t)n * 4;
+        case A8W8_SCALE_BLOCK_1x128_128x128: return (n % 128 || k % 128) ? 0 : (size_t)(n / 128) * (k / 128) * 4;
+        case A8W8_SCALE_MX_E8M0_1x32: return k % 32 ? 0 : (size_t)n * (k / 32);
+        case A8W8_SCALE_MX_E8M0_TILED: return k % 32 ? 0 : mx_tiled_bytes(n, k);
+        default: return 0;
+    }
+}
+
+int a8w8_weights_save(const char* path, const void* b_host, const void* scale_host, int n, int k, int b_preshuffled,
+                      int scale_mode)
+{
+    if (!path || !b_host || !scale_host) return A8W8_ERR_NULL_POINTER;
+    if (n <= 0 || k <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (b_preshuffled && (n % 16 != 0 || k % 64 != 0)) return A8W8_ERR_BAD_GROUP;
+    const size_t sbytes = a8w8_weight_scale_bytes(n, k, scale_mode);
+    if (sbytes == 0) return scale_mode < 0 || scale_mode > A8W8_SCALE_MX_E8M0_TILED ? A8W8_ERR_BAD_MODE : A8W8_ERR_BAD_GROUP;
+    a8w8_weight_header h;
+    memset(&h, 0, sizeof h);
+    memcpy(h.magic, kWeightMagic, 8);
+    h.version = 1;
+    h.n = (uint32_t)n; h.k = (uint32_t)k;
+    h.b_preshuffled = b_preshuffled ? 1 : 0;
+    h.scale_mode = (uint32_t)scale_mode;
+    h.b_bytes = (uint64_t)n * k;
+    h.scale_bytes = sbytes;
+    h.checksum = fnv1a64(scale_host, sbytes, fnv1a64(b_host, (size_t)h.b_bytes, 14695981039346656037ull));
+    FILE* f = fopen(path, "wb");
+    if (!f) return A8W8_ERR_IO;
+    const bool ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(b_host, 1, (size_t)h.b_bytes, f) == h.b_bytes &&
+                    fwrite(scale_host, 1, sbytes, f) == sbytes;
+    return (fclose(f) == 0 && ok) ? A8W8_OK : A8W8_ERR_IO;
+}
+
+int a8w8_weights_info(const char* path, a8w8_weight_header* out)
+{
+    if (!path || !out) return A8W8_ERR_NULL_POINTER;
+    FILE* f = fopen(path, "rb");
+    if (!f) return A8W8_ERR_IO;
+    const size_t got = fread(out, 1, sizeof *out, f);
+    fclose(f);
+    if (got != sizeof *out) return A8W8_ERR_BAD_FILE;
+    return check_header(*out);
+}
+
+int a8w8_weights_load(const char* path, void* b_host, size_t b_capacity, void* scale_host, size_t scale_capacity)
+{
+    if (!path || !b_host || !scale_host) return A8W8_ERR_NULL_POINTER;
+    FILE* f = fopen(path, "rb");
+    if (!f) return A8W8_ERR_IO;
+    a8w8_weight_header h;
+    int st = fread(&h, 1, sizeof h, f) == sizeof h ? check_header(h) : A8W8_ERR_BAD_FILE;
+    if (st == A8W8_OK && (h.b_bytes > b_capacity || h.scale_bytes > scale_capacity)) st = A8W8_ERR_BAD_STRIDE;
+    if (st == A8W8_OK && (fread(b_host, 1, (size_t)h.b_bytes, f) != h.b_bytes ||
+                          fread(scale_host, 1, (size_t)h.scale_bytes, f) != h.scale_bytes))
+        st = A8W8_ERR_BAD_FILE;
+    fclose(f);
+    if (st != A8W8_OK) return st;
+    const uint64_t sum = fnv1a64(scale_host, (size_t)h.scale_bytes, fnv1a64(b_host, (size_t)h.b_bytes, 14695981039346656037ull));
+    return sum == h.checksum ? A8W8_OK : A8W8_ERR_BAD_FILE;
+}
+
 const char* a8w8_status_string(int status)
 {
     switch (status) {
@@ -449,6 +538,8 @@ const char* a8w8_status_string(int status)
         case A8W8_ERR_TOO_LARGE: return "matrix too large for 32-bit offsets";
         case A8W8_ERR_LAUNCH: return "kernel launch failed";
         case A8W8_ERR_NO_DEVICE: return "current device is not gfx950";
+        case A8W8_ERR_IO: return "weight file could not be opened, read or written";
+        case A8W8_ERR_BAD_FILE: return "not a weight file of this version, truncated, or checksum mismatch";
         default: return "unknown status";
     }
 }

@@ -34,7 +34,10 @@ typedef enum {
                                      the entry point does not implement                    */
     A8W8_ERR_TOO_LARGE = -7,      /* an offset would not fit the 32-bit addressing in use   */
     A8W8_ERR_LAUNCH = -8,         /* hipGetLastError() reported a failed launch             */
-    A8W8_ERR_NO_DEVICE = -9       /* no gfx950 device is current                            */
+    A8W8_ERR_NO_DEVICE = -9,      /* no gfx950 device is current                            */
+    A8W8_ERR_IO = -10,            /* a weight file could not be opened, read or written     */
+    A8W8_ERR_BAD_FILE = -11       /* not a weight file of this version, truncated, or its
+                                     checksum does not match                                */
 } a8w8_status;
 
 /* How the dequantisation scales are laid out.  All fp32 unless stated.
@@ -152,6 +155,33 @@ A8W8_API int a8w8_mx_tile_scales_ab(const uint8_t* sfa_dev, int m, int stride_sf
                                     const uint8_t* sfb_dev, int n, int stride_sfb, uint8_t* out_b_dev, int k,
                                     void* hip_stream);
 A8W8_API size_t a8w8_mx_tiled_bytes(int rows, int k);
+
+/* Pre-processed weights on disk (host memory in, host memory out): the quantised B matrix, row-major
+ * or in the a8w8_preshuffle_b layout, plus its scales in the layout a8w8_gemm / a8w8_flatmm read for
+ * `scale_mode`, behind a 64-byte header, so that quantisation, shuffling and scale tiling are paid
+ * once.  The reference keeps no such cache (its harness regenerates random weights per run).
+ * File: header, n*k weight bytes, scale bytes (TENSOR 4; ROWCOL 4n; BLOCK 4*(n/128)*(k/128);
+ * MX n*k/32; MX_TILED a8w8_mx_tiled_bytes(n, k)); `checksum` is FNV-1a-64 over both payloads. */
+typedef struct {
+    char magic[8];          /* "A8W8WGT" and a NUL                                  */
+    uint32_t version;       /* 1                                                     */
+    uint32_t n, k;
+    uint32_t b_preshuffled; /* 0 row-major [n][k], 1 a8w8_preshuffle_b layout        */
+    uint32_t scale_mode;    /* a8w8_scale_mode of the stored scales                  */
+    uint32_t reserved;
+    uint64_t b_bytes, scale_bytes;
+    uint64_t checksum;
+    uint64_t reserved2;
+} a8w8_weight_header;
+
+A8W8_API size_t a8w8_weight_scale_bytes(int n, int k, int scale_mode);
+A8W8_API int a8w8_weights_save(const char* path, const void* b_host, const void* scale_host, int n, int k,
+                               int b_preshuffled, int scale_mode);
+/* Reads and checks the header only. */
+A8W8_API int a8w8_weights_info(const char* path, a8w8_weight_header* out);
+/* Reads both payloads into buffers of at least header.b_bytes / header.scale_bytes and verifies the checksum. */
+A8W8_API int a8w8_weights_load(const char* path, void* b_host, size_t b_capacity, void* scale_host,
+                               size_t scale_capacity);
 
 A8W8_API const char* a8w8_status_string(int status);
 
