@@ -69,6 +69,7 @@ def lib():
         vp = ctypes.c_void_p
         L.a8w8_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a8w8_gemm_blockscale.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.a16w16_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a8w8_flatmm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a8w8_preshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
         L.a8w8_unshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
@@ -169,6 +170,13 @@ def gemm(a, b, sfa, sfb, scale_mode, c=None, c_dtype=BF16):
     """C = dequant(A) @ dequant(B)^T through a8w8_gemm.  a [.., M, K] u8, b [.., N, K] u8 on the GPU."""
     g, c = _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, 0)
     _check(lib().a8w8_gemm(ctypes.byref(g), _stream()), "a8w8_gemm")
+    return c
+
+
+def gemm_a16w16(a, b, c=None, c_dtype=BF16):
+    """C = A @ B^T for bf16 a [.., M, K] and b [.., N, K] (torch.bfloat16 on the GPU) through a16w16_gemm."""
+    g, c = _args_from_tensors(a, b, a, b, TENSOR, c, c_dtype, 0)
+    _check(lib().a16w16_gemm(ctypes.byref(g), _stream()), "a16w16_gemm")
     return c
 
 

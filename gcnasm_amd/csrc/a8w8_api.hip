@@ -243,6 +243,45 @@ int a8w8_gemm(const a8w8_gemm_args* g, void* hip_stream)
     return persist_ok(g) ? dispatch_persist(g, p, s) : dispatch_tiled(g, p, s);
 }
 
+int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
+{
+    if (!g) return A8W8_ERR_NULL_POINTER;
+    if (!g->a || !g->b || !g->c) return A8W8_ERR_NULL_POINTER;
+    if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
+    if (g->b_preshuffled) return A8W8_ERR_BAD_MODE;
+    if (g->stride_c < g->n || g->stride_a < g->k || g->stride_b < g->k) return A8W8_ERR_BAD_STRIDE;
+    if (g->batch > 1 && (g->stride_a_batch < 0 || g->stride_b_batch < 0 || g->stride_c_batch < 0)) return A8W8_ERR_BAD_STRIDE;
+    const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) * 2;
+    const long long b_span = ((long long)(g->n - 1) * g->stride_b + g->k) * 2;
+    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    hipStream_t s = (hipStream_t)hip_stream;
+    // the tiled kernel reads bf16 rows as byte rows of 2k columns
+    a8w8_gemm_args bytes = *g;
+    bytes.k = g->k * 2;
+    bytes.stride_a = g->stride_a * 2; bytes.stride_b = g->stride_b * 2;
+    bytes.stride_a_batch = g->stride_a_batch * 2; bytes.stride_b_batch = g->stride_b_batch * 2;
+    bytes.scale_mode = A8W8_SCALE_TENSOR;
+    const bool fits = (long long)g->stride_a_batch * 2 < (1ll << 31) && (long long)g->stride_b_batch * 2 < (1ll << 31);
+    if (fits && tiled_ok(&bytes) && persist_ok(&bytes)) {
+        GemmParams p = make_params(&bytes);
+        p.sfa = p.sfb = nullptr;
+        return g->c_dtype == A8W8_C_BF16 ? launch_persist<MODE_BF16, C_BF16>(p, g->batch, s)
+                                         : launch_persist<MODE_BF16, C_FP32>(p, g->batch, s);
+    }
+    dim3 grid((unsigned)((g->n + 15) / 16), (unsigned)((g->m + 15) / 16), (unsigned)g->batch);
+    if (g->c_dtype == A8W8_C_BF16)
+        hipLaunchKernelGGL((gemm_a16w16_general<C_BF16>), grid, dim3(256), 0, s, (const unsigned short*)g->a,
+                           (const unsigned short*)g->b, g->c, g->m, g->n, g->k, g->stride_a, g->stride_b, g->stride_c,
+                           (long long)g->stride_a_batch, (long long)g->stride_b_batch, (long long)g->stride_c_batch);
+    else
+        hipLaunchKernelGGL((gemm_a16w16_general<C_FP32>), grid, dim3(256), 0, s, (const unsigned short*)g->a,
+                           (const unsigned short*)g->b, g->c, g->m, g->n, g->k, g->stride_a, g->stride_b, g->stride_c,
+                           (long long)g->stride_a_batch, (long long)g->stride_b_batch, (long long)g->stride_c_batch);
+    return launch_status();
+}
+
 int a8w8_gemm_blockscale(const a8w8_gemm_args* g, void* hip_stream)
 {
     if (!g) return A8W8_ERR_NULL_POINTER;

@@ -10,11 +10,13 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned short v4u16 __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 #define A8W8_DEV __device__ __forceinline__
 #define A8W8_LDS __attribute__((address_space(3)))
 
-enum : int { MODE_TENSOR = 0, MODE_ROWCOL = 1, MODE_BLOCK = 2, MODE_MX = 3, MODE_MXT = 4 };
+// MODE_BF16: A and B hold bf16 (the a16w16 sibling), no scales; the kernels see them as byte matrices of 2k columns
+enum : int { MODE_TENSOR = 0, MODE_ROWCOL = 1, MODE_BLOCK = 2, MODE_MX = 3, MODE_MXT = 4, MODE_BF16 = 5 };
 
 // Byte position of the E8M0 exponent of (row, 32-wide K block kblk) in the tiled MX scale layout
 //   [K/512][ceil(rows/64)][pair of K steps: 2][r16: 16][g: 4][jp: 2][par: 2][s: 2]       (1 byte each)

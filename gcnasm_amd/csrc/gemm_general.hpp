@@ -56,4 +56,28 @@ __global__ void __launch_bounds__(256) gemm_a8w8_general(GemmParams p)
     else ((float*)p.c)[ci] = sum;
 }
 
+// bf16 x bf16 -> fp32 accumulate, any shape: the order of operations of the reference CPU GEMM
+// (sequential K, product then add, no fused multiply-add).  a, b hold bf16 bit patterns.
+template <int CDT>
+__global__ void __launch_bounds__(256) gemm_a16w16_general(const unsigned short* a, const unsigned short* b, void* c, int m, int n,
+                                                           int k, int lda, int ldb, int ldc, long long a_batch, long long b_batch,
+                                                           long long c_batch)
+{
+#pragma clang fp contract(off)
+    const int j = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int i = blockIdx.y * 16 + (threadIdx.x >> 4);
+    const int batch = blockIdx.z;
+    if (i >= m || j >= n) return;
+    const unsigned short* ar = a + batch * a_batch + (long long)i * lda;
+    const unsigned short* br = b + batch * b_batch + (long long)j * ldb;
+    float sum = 0.f;
+    for (int p = 0; p < k; ++p) {
+        const float prod = __uint_as_float((unsigned)ar[p] << 16) * __uint_as_float((unsigned)br[p] << 16);
+        sum = sum + prod;
+    }
+    const long long ci = batch * c_batch + (long long)i * ldc + j;
+    if constexpr (CDT == C_BF16) ((unsigned short*)c)[ci] = bf16_bits(sum);
+    else ((float*)c)[ci] = sum;
+}
+
 }  // namespace a8w8

@@ -48,7 +48,7 @@ constexpr int PERSIST_LDS_BYTES_ROWCOL = GEMM_LDS_BYTES + 2 * ROWCOL_SCALE_BYTES
 #define A8W8_NPF_MX 1
 #endif
 #define A8W8_PREFETCH_A(mode)                                                                        \
-    ((mode) == MODE_TENSOR ? 4 : (mode) == MODE_ROWCOL ? A8W8_NPF_ROWCOL : (mode) == MODE_MXT ? A8W8_NPF_MXT \
+    ((mode) == MODE_TENSOR || (mode) == MODE_BF16 ? 4 : (mode) == MODE_ROWCOL ? A8W8_NPF_ROWCOL : (mode) == MODE_MXT ? A8W8_NPF_MXT \
                                                      : (mode) == MODE_MX ? A8W8_NPF_MX : 0)
 #ifndef A8W8_PERSIST_BLK_LAG
 #define A8W8_PERSIST_BLK_LAG 4
@@ -505,26 +505,44 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                         for (int u = TM * TN - BLK_LAG; u < TM * TN; ++u)
                             acc[u % TM][u / TM] += part[u % (BLK_LAG + 1)] * blk_s[u % TM];
                     }
+                } else if constexpr (MODE == MODE_BF16) {
+                    // a 128-byte row is 64 bf16: the fragment's two 16-byte halves feed one 16x16x32 MFMA each
+                    // (both operands split K the same way, so the order inside an instruction is immaterial).
+                    // First halves here, second halves after the loop: back-to-back MFMAs on one accumulator stall.
+                    const v4i blo = {fb[j][0], fb[j][1], fb[j][2], fb[j][3]};
+                    const v4i alo = {cur.a[i][0], cur.a[i][1], cur.a[i][2], cur.a[i][3]};
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, blo), __builtin_bit_cast(v8bf, alo),
+                                                                        acc[i][j], 0, 0, 0);
                 } else {
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], cur.a[i], acc[i][j], 0, 0, 0,
                                                                                  0, 0, 0);
+                }
+            }
+            if constexpr (MODE == MODE_BF16) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const v4i bhi = {fb[j][4], fb[j][5], fb[j][6], fb[j][7]};
+                    const v4i ahi = {cur.a[i][4], cur.a[i][5], cur.a[i][6], cur.a[i][7]};
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, bhi), __builtin_bit_cast(v8bf, ahi),
+                                                                        acc[i][j], 0, 0, 0);
                 }
             }
             A8W8_PERSIST_SCHED_BARRIER();
 #if A8W8_PERSIST_SG
             if constexpr (MODE != MODE_BLOCK) {
                 // spread the two LDS reads of the next B fragment between this group's MFMAs
+                constexpr int MPF = MODE == MODE_BF16 ? 2 : 1;      // MFMAs per operand fragment pair
                 if (j + 1 < TN) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, MPF, 0);
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, MPF, 0);
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 2 * MPF, 0);
                 } else if (A8W8_PERSIST_SG >= 2 && PREFETCH_FRAGS) {
                     // the last group runs beside the next step's prefetched fragments
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, MPF, 0);
                         __builtin_amdgcn_sched_group_barrier(0x100, (2 * NPF + 2 + 3) / 4, 0);
                     }
                 }

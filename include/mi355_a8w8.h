@@ -92,6 +92,13 @@ typedef struct {
  * the tiled kernels; other shapes run on a slower general kernel.  m, n edges are handled. */
 A8W8_API int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream);
 
+/* The bf16 sibling (gemm_a16w16_8wave, the program opus_gemm/rebuild.sh:3-13 builds; its source is
+ * absent from the reference): A [batch, m, k] and B [batch, n, k] hold bf16, C = A * B^T in bf16 or
+ * fp32, fp32 accumulation, no scales (sfa, sfb, stride_sf*, scale_mode are ignored).  Runs on the
+ * same pipelined kernel as a8w8_gemm with the 16x16x32 bf16 MFMA when k % 64 == 0, k >= 128 and rows
+ * are 16-byte aligned; other shapes take a general kernel that follows the CPU order of operations. */
+A8W8_API int a16w16_gemm(const a8w8_gemm_args* args, void* hip_stream);
+
 /* The block-scale entry point with exactly the reference's preconditions: scale_mode is
  * taken as BLOCK_1x128_128x128, n % 128 == 0 and k % 128 == 0 are required
  * (host.cc:179-187); c_dtype may be fp32 (the reference's output, common.h / host.cc:216)

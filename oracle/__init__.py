@@ -68,6 +68,7 @@ def lib():
         L.orc_mx_tiled_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
         L.orc_mx_tile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
         L.orc_mx_untile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
+        L.orc_gemm_bf16_ref.argtypes = [_u16p, _u16p, _f32p] + [ctypes.c_int] * 6
         L.orc_quant_tensor.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p]
         L.orc_quant_rowwise.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p]
         L.orc_quant_block.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p, ctypes.c_int]
@@ -228,6 +229,17 @@ def mx_untile_scales(tiled, rows, k):
     out = np.zeros((rows, k // 32), np.uint8)
     lib().orc_mx_untile_scales(_p(tiled, _u8p), rows, k, k // 32, _p(out, _u8p))
     return out
+
+
+def gemm_bf16_ref(a_bits, b_bits):
+    """fp32 C of the bf16 GEMM; a_bits [M, K], b_bits [N, K] uint16 bf16 patterns."""
+    a_bits = _c(a_bits, np.uint16)
+    b_bits = _c(b_bits, np.uint16)
+    m, k = a_bits.shape
+    n = b_bits.shape[0]
+    c = np.empty((m, n), np.float32)
+    lib().orc_gemm_bf16_ref(_p(a_bits, _u16p), _p(b_bits, _u16p), _p(c, _f32p), m, n, k, k, k, n)
+    return c
 
 
 def quantize(x, mode, group_rows=1):

@@ -22,6 +22,7 @@
  *   orc_gemm_ref / orc_gemm_ref_mx   brute force in float64 on tiny shapes,
  *       exact-integer inputs, scale-mode reductions.
  *   orc_preshuffle_b       bijection + flatmm(A, shuffle(B)) == gemm(A, B).
+ *   orc_gemm_bf16_ref      float64 matmul on small shapes, exact-integer inputs.
  *   orc_quant_*            no reference code (its harness has no quantiser): the recipe of the
  *       benchmark configurations, fixed by properties -- the group's largest element maps to
  *       +-448 (row/block) or into (224, 448] (MX, never saturating), dequantisation error within
@@ -414,6 +415,22 @@ ORC_API void orc_flatmm_ref(const uint8_t* a, const uint8_t* bshuf, const float*
             c[(size_t)i * ldc + j] = sum;
         }
     }
+}
+
+/* bf16 x bf16 GEMM of the a16w16 sibling (its source is absent; opus_gemm/rebuild.sh:3 names it): the same
+ * loop as gemm_ref, host.cc:66-90, without scales -- fp32 accumulation over K in order, C[i][j] =
+ * sum_k float(A[i][k]) * float(B[j][k]).  a, b hold bf16 bit patterns. */
+ORC_API void orc_gemm_bf16_ref(const uint16_t* a, const uint16_t* b, float* c, int m, int n, int k, int lda, int ldb,
+                               int ldc)
+{
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int i = 0; i < m; ++i)
+        for (int j = 0; j < n; ++j) {
+            float sum = 0.0f;
+            for (int p = 0; p < k; ++p)
+                sum += u2f((uint32_t)a[(size_t)i * lda + p] << 16) * u2f((uint32_t)b[(size_t)j * ldb + p] << 16);
+            c[(size_t)i * ldc + j] = sum;
+        }
 }
 
 /* ------------------------------------------------------------ quantisation front end

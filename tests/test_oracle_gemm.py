@@ -160,3 +160,18 @@ def test_mx_tiled_layout_groups_what_one_lane_needs(orc):
     t = orc.mx_tile_scales(sf)
     pos = int(np.nonzero(t == 200)[0][0])
     assert pos == ((1 * 64 + 11 * 4 + 2) * 8) + 1 * 4 + 1 * 2 + 0
+
+
+def test_bf16_gemm_oracle_against_float64_and_integers(orc):
+    rng = np.random.Generator(np.random.Philox(77))
+    a = rng.standard_normal((9, 40)).astype(np.float32)
+    b = rng.standard_normal((7, 40)).astype(np.float32)
+    ab, bb = orc.to_bf16_bits(a), orc.to_bf16_bits(b)
+    af, bf = orc.bf16_bits_to_f32(ab).astype(np.float64), orc.bf16_bits_to_f32(bb).astype(np.float64)
+    got = orc.gemm_bf16_ref(ab, bb)
+    assert np.abs(got - af @ bf.T).max() <= 1e-5 * (np.abs(af) @ np.abs(bf).T).max()
+    ai = rng.integers(-8, 9, (5, 64)).astype(np.float32)
+    bi = rng.integers(-8, 9, (6, 64)).astype(np.float32)
+    assert (orc.gemm_bf16_ref(orc.to_bf16_bits(ai), orc.to_bf16_bits(bi)) == ai @ bi.T).all()
+    # a transposed B would not pass: the oracle indexes B as [N, K]
+    assert got.shape == (9, 7)
