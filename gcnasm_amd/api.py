@@ -70,6 +70,7 @@ def lib():
         L.a8w8_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a8w8_gemm_blockscale.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a16w16_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.a16w16_flatmm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a8w8_flatmm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a8w8_preshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
         L.a8w8_unshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
@@ -177,6 +178,20 @@ def gemm_a16w16(a, b, c=None, c_dtype=BF16):
     """C = A @ B^T for bf16 a [.., M, K] and b [.., N, K] (torch.bfloat16 on the GPU) through a16w16_gemm."""
     g, c = _args_from_tensors(a, b, a, b, TENSOR, c, c_dtype, 0)
     _check(lib().a16w16_gemm(ctypes.byref(g), _stream()), "a16w16_gemm")
+    return c
+
+
+def preshuffle_b_bf16_device(b):
+    """bf16 weights [N, K] on the GPU -> the pre-shuffled byte layout a16w16_flatmm streams (flat uint8 tensor)."""
+    import torch
+    n, k = b.shape
+    return preshuffle_b_device(b.contiguous().view(torch.uint8).view(n, 2 * k))
+
+
+def flatmm_a16w16(a, b_shuffled, n, c=None, c_dtype=BF16):
+    """Skinny-M bf16 GEMM over weights from preshuffle_b_bf16_device."""
+    g, c = _args_from_tensors(a, b_shuffled, a, a, TENSOR, c, c_dtype, 1, n=n)
+    _check(lib().a16w16_flatmm(ctypes.byref(g), _stream()), "a16w16_flatmm")
     return c
 
 

@@ -282,6 +282,30 @@ int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
     return launch_status();
 }
 
+int a16w16_flatmm(const a8w8_gemm_args* g, void* hip_stream)
+{
+    if (!g) return A8W8_ERR_NULL_POINTER;
+    if (!g->a || !g->b || !g->c) return A8W8_ERR_NULL_POINTER;
+    if (!g->b_preshuffled) return A8W8_ERR_BAD_MODE;
+    if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0 || g->m > 64) return A8W8_ERR_BAD_SHAPE;
+    if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
+    if (g->n % 16 != 0 || g->k % 32 != 0) return A8W8_ERR_BAD_GROUP;
+    if (g->stride_c < g->n || g->stride_a < g->k) return A8W8_ERR_BAD_STRIDE;
+    if (!aligned16(g->a) || !aligned16(g->b) || g->stride_a % 8 != 0) return A8W8_ERR_MISALIGNED;
+    if (g->batch > 1 && (g->stride_a_batch % 8 != 0 || g->stride_b_batch % 8 != 0)) return A8W8_ERR_MISALIGNED;
+    if ((long long)g->n * g->k * 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    a8w8_gemm_args bytes = *g;      // bf16 rows as byte rows of 2k columns
+    bytes.k = g->k * 2;
+    bytes.stride_a = g->stride_a * 2; bytes.stride_b = g->k * 2;
+    bytes.stride_a_batch = g->stride_a_batch * 2; bytes.stride_b_batch = g->stride_b_batch * 2;
+    GemmParams p = make_params(&bytes);
+    p.sfa = p.sfb = nullptr;
+    hipStream_t s = (hipStream_t)hip_stream;
+    return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_BF16>(p, g->batch, s)
+                                     : launch_flat<C_FP32, MODE_BF16>(p, g->batch, s);
+}
+
 int a8w8_gemm_blockscale(const a8w8_gemm_args* g, void* hip_stream)
 {
     if (!g) return A8W8_ERR_NULL_POINTER;

@@ -44,7 +44,9 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     if (finisher) {
         const float* sfa = (const float*)p.sfa + (long long)batch * p.sfa_batch;
         const float* sfb = (const float*)p.sfb + (long long)batch * p.sfb_batch;
-        if constexpr (MODE == MODE_TENSOR) {
+        if constexpr (MODE == MODE_BF16) {
+            // bf16 operands carry no scales
+        } else if constexpr (MODE == MODE_TENSOR) {
             sa = sfa[0] * sfb[0];
         } else {
             sa = sfa[cm];
@@ -89,7 +91,15 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         for (int t = 0; t < NT; ++t) {
             const v8i fb = v8i{f.b[t][0].x, f.b[t][0].y, f.b[t][0].z, f.b[t][0].w,
                                f.b[t][1].x, f.b[t][1].y, f.b[t][1].z, f.b[t][1].w};
-            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[t], 0, 0, 0, 0, 0, 0);
+            if constexpr (MODE == MODE_BF16) {
+                // bf16 weights: a 1 KiB block is 16 rows x 32 bf16, one 16x16x32 MFMA operand
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, f.b[t][0]),
+                                                                 __builtin_bit_cast(v8bf, f.a[0]), acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, f.b[t][1]),
+                                                                 __builtin_bit_cast(v8bf, f.a[1]), acc[t], 0, 0, 0);
+            } else {
+                acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[t], 0, 0, 0, 0, 0, 0);
+            }
         }
     };
 

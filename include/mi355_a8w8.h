@@ -99,6 +99,11 @@ A8W8_API int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream);
  * are 16-byte aligned; other shapes take a general kernel that follows the CPU order of operations. */
 A8W8_API int a16w16_gemm(const a8w8_gemm_args* args, void* hip_stream);
 
+/* The bf16 flat GEMM (flatmm_a16w16_gfx950, opus_fmm/README.md:10,51-57; source absent): A [batch, m, k]
+ * bf16 with m <= 64, B bf16 pre-shuffled as a byte matrix -- a8w8_preshuffle_b[_device](b, out, n, 2*k) --
+ * n % 16 == 0, k % 32 == 0, no scales, bf16 or fp32 C.  Same streaming kernel as a8w8_flatmm. */
+A8W8_API int a16w16_flatmm(const a8w8_gemm_args* args, void* hip_stream);
+
 /* The block-scale entry point with exactly the reference's preconditions: scale_mode is
  * taken as BLOCK_1x128_128x128, n % 128 == 0 and k % 128 == 0 are required
  * (host.cc:179-187); c_dtype may be fp32 (the reference's output, common.h / host.cc:216)

@@ -75,3 +75,26 @@ def test_full_size_4096(orc):
     assert torch.equal(g.gemm_a16w16(a * 2, b).float(), 2 * c)
     perm = torch.randperm(m, generator=torch.Generator().manual_seed(3)).cuda()
     assert torch.equal(g.gemm_a16w16(a[perm].contiguous(), b), g.gemm_a16w16(a, b)[perm])
+
+
+@pytest.mark.parametrize("shape", [(16, 256, 512), (1, 64, 32), (33, 2048, 1024), (64, 128, 96)])
+def test_flat_gemm_over_preshuffled_bf16_weights(orc, shape):
+    m, n, k = shape
+    a, b = _rand(m, k, 61 + m), _rand(n, k, 62 + n)
+    bs = g.preshuffle_b_bf16_device(b)
+    # the device shuffle of the byte view is the oracle's shuffle of the same bytes
+    assert (bs.cpu().numpy() == orc.preshuffle_b(b.view(torch.uint8).view(n, 2 * k).cpu().numpy())).all()
+    ref = orc.gemm_bf16_ref(_bits(a), _bits(b))
+    c32 = g.flatmm_a16w16(a, bs, n, c_dtype=g.FP32).cpu().numpy()
+    np.testing.assert_allclose(c32, ref, rtol=1e-4, atol=1e-4 * max(np.abs(ref).max(), 1e-6))
+    c = g.flatmm_a16w16(a, bs, n).float().cpu().numpy()
+    assert (np.abs(c - ref) <= 1e-2 * np.abs(ref) + 1e-2).all()
+
+
+def test_flat_gemm_exact_integers_and_decode_shape(orc):
+    m, n, k = 16, 16384, 7168
+    gen = torch.Generator(device="cuda"); gen.manual_seed(8)
+    a = torch.randint(-4, 5, (m, k), generator=gen, device="cuda").to(torch.bfloat16)
+    b = torch.randint(-4, 5, (n, k), generator=gen, device="cuda").to(torch.bfloat16)
+    want = a.float() @ b.float().T
+    assert torch.equal(g.flatmm_a16w16(a, g.preshuffle_b_bf16_device(b), n, c_dtype=g.FP32), want)
