@@ -9,3 +9,4 @@ from .api import (  # noqa: F401
     cvt_f32_to_e4m3, flatmm, flatmm_a16w16, gemm, gemm_a16w16, gemm_blockscale, kernel_name, lib, library_path, load_weights, save_weights, mx_tile_scales, mx_tile_scales_ab, mx_tiled_bytes, preshuffle_b, preshuffle_b_bf16_device,
     preshuffle_b_device, quantize, raw_gemm_args, status_string, unshuffle_b,
 )
+from .ops import register as register_torch_ops  # noqa: E402,F401
