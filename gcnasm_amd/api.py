@@ -71,6 +71,8 @@ def lib():
         L.a8w8_gemm_blockscale.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a16w16_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a16w16_flatmm.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.a4w4_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.a4w4_quantize_mx.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_int, vp]
         L.a8w8_flatmm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a8w8_preshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
         L.a8w8_unshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
@@ -192,6 +194,27 @@ def flatmm_a16w16(a, b_shuffled, n, c=None, c_dtype=BF16):
     """Skinny-M bf16 GEMM over weights from preshuffle_b_bf16_device."""
     g, c = _args_from_tensors(a, b_shuffled, a, a, TENSOR, c, c_dtype, 1, n=n)
     _check(lib().a16w16_flatmm(ctypes.byref(g), _stream()), "a16w16_flatmm")
+    return c
+
+
+def quantize_mxfp4(x, tiled=False):
+    """fp32 [rows, K] -> (packed E2M1 bytes [rows, K/2], E8M0 scales row-major [rows, K/32] or tiled)."""
+    import torch
+    rows, k = x.shape
+    q = torch.empty((rows, k // 2), dtype=torch.uint8, device=x.device)
+    s = torch.empty(mx_tiled_bytes(rows, k) if tiled else (rows, k // 32), dtype=torch.uint8, device=x.device)
+    _check(lib().a4w4_quantize_mx(x.data_ptr(), rows, k, x.stride(0), q.data_ptr(), s.data_ptr(), int(tiled), _stream()),
+           "a4w4_quantize_mx")
+    return q, s
+
+
+def gemm_a4w4(a, b, sfa, sfb, scale_mode=MX_TILED, c=None, c_dtype=BF16):
+    """MXFP4 GEMM through a4w4_gemm: a [M, K/2], b [N, K/2] packed E2M1 (uint8 on the GPU)."""
+    m, n, k = a.shape[-2], b.shape[-2], a.shape[-1] * 2
+    c = _out(c, (m, n), c_dtype, a.device)
+    g = raw_gemm_args(a.data_ptr(), b.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, scale_mode, c_dtype,
+                      stride_a=a.stride(-2) * 2, stride_b=b.stride(-2) * 2, stride_c=c.stride(-2))
+    _check(lib().a4w4_gemm(ctypes.byref(g), _stream()), "a4w4_gemm")
     return c
 
 

@@ -147,7 +147,7 @@ int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
     int dev = 0;
     (void)hipGetDevice(&dev);
     auto kern = gemm_a8w8_persist<MODE, CDT>;
-    constexpr int lds_bytes = (MODE == MODE_MX || MODE == MODE_MXT) ? PERSIST_LDS_BYTES_MX
+    constexpr int lds_bytes = (MODE == MODE_MX || MODE == MODE_MXT || MODE == MODE_F4T) ? PERSIST_LDS_BYTES_MX
                               : MODE == MODE_ROWCOL                   ? PERSIST_LDS_BYTES_ROWCOL
                                                                       : PERSIST_LDS_BYTES;
     if (!attr_set[dev & 63]) {
@@ -279,6 +279,74 @@ int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
         hipLaunchKernelGGL((gemm_a16w16_general<C_FP32>), grid, dim3(256), 0, s, (const unsigned short*)g->a,
                            (const unsigned short*)g->b, g->c, g->m, g->n, g->k, g->stride_a, g->stride_b, g->stride_c,
                            (long long)g->stride_a_batch, (long long)g->stride_b_batch, (long long)g->stride_c_batch);
+    return launch_status();
+}
+
+int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream)
+{
+    if (!g) return A8W8_ERR_NULL_POINTER;
+    if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
+    if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (g->scale_mode != A8W8_SCALE_MX_E8M0_1x32 && g->scale_mode != A8W8_SCALE_MX_E8M0_TILED) return A8W8_ERR_BAD_MODE;
+    if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
+    if (g->b_preshuffled) return A8W8_ERR_BAD_MODE;
+    if (g->k % 32 != 0) return A8W8_ERR_BAD_GROUP;
+    if (g->stride_c < g->n || g->stride_a < g->k || g->stride_b < g->k) return A8W8_ERR_BAD_STRIDE;
+    if ((g->stride_a & 1) || (g->stride_b & 1)) return A8W8_ERR_MISALIGNED;      // rows start on a byte
+    const bool tiled = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;
+    if (!tiled && (g->stride_sfa < g->k / 32 || g->stride_sfb < g->k / 32)) return A8W8_ERR_BAD_STRIDE;
+    if (g->batch > 1 && ((g->stride_a_batch & 1) || (g->stride_b_batch & 1))) return A8W8_ERR_MISALIGNED;
+    if (g->batch > 1 && (g->stride_a_batch < 0 || g->stride_b_batch < 0 || g->stride_c_batch < 0 ||
+                         g->stride_sfa_batch < 0 || g->stride_sfb_batch < 0))
+        return A8W8_ERR_BAD_STRIDE;
+    const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) / 2;
+    const long long b_span = ((long long)(g->n - 1) * g->stride_b + g->k) / 2;
+    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    hipStream_t s = (hipStream_t)hip_stream;
+    // the tiled kernel reads packed rows as byte rows of k/2 columns
+    a8w8_gemm_args bytes = *g;
+    bytes.k = g->k / 2;
+    bytes.stride_a = g->stride_a / 2; bytes.stride_b = g->stride_b / 2;
+    bytes.stride_a_batch = g->stride_a_batch / 2; bytes.stride_b_batch = g->stride_b_batch / 2;
+    bytes.scale_mode = A8W8_SCALE_MX_E8M0_TILED;
+    if (tiled && g->k % 256 == 0 && tiled_ok(&bytes) && persist_ok(&bytes)) {
+        const GemmParams p = make_params(&bytes);
+        return g->c_dtype == A8W8_C_BF16 ? launch_persist<MODE_F4T, C_BF16>(p, g->batch, s)
+                                         : launch_persist<MODE_F4T, C_FP32>(p, g->batch, s);
+    }
+    dim3 grid((unsigned)((g->n + 15) / 16), (unsigned)((g->m + 15) / 16), (unsigned)g->batch);
+#define A4W4_GENERAL(CDT, TILED)                                                                                        \
+    hipLaunchKernelGGL((gemm_a4w4_general<CDT, TILED>), grid, dim3(256), 0, s, (const uint8_t*)g->a, (const uint8_t*)g->b, \
+                       (const uint8_t*)g->sfa, (const uint8_t*)g->sfb, g->c, g->m, g->n, g->k, g->stride_a / 2,            \
+                       g->stride_b / 2, g->stride_c, g->stride_sfa, g->stride_sfb, (long long)g->stride_a_batch / 2,       \
+                       (long long)g->stride_b_batch / 2, (long long)g->stride_c_batch, (long long)g->stride_sfa_batch,     \
+                       (long long)g->stride_sfb_batch)
+    if (g->c_dtype == A8W8_C_BF16) { if (tiled) A4W4_GENERAL(C_BF16, true); else A4W4_GENERAL(C_BF16, false); }
+    else { if (tiled) A4W4_GENERAL(C_FP32, true); else A4W4_GENERAL(C_FP32, false); }
+#undef A4W4_GENERAL
+    return launch_status();
+}
+
+int a4w4_quantize_mx(const float* src, int rows, int k, int ld, uint8_t* q, uint8_t* scale, int tiled, void* hip_stream)
+{
+    if (!src || !q || !scale) return A8W8_ERR_NULL_POINTER;
+    if (rows <= 0 || k <= 0) return A8W8_ERR_BAD_SHAPE;
+    if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
+    if (ld < k) return A8W8_ERR_BAD_STRIDE;
+    if (tiled && ((uintptr_t)scale & 3)) return A8W8_ERR_MISALIGNED;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    hipStream_t s = (hipStream_t)hip_stream;
+    const long long threads = (long long)rows * k;
+    if (tiled) {
+        if (rows % 64 != 0 || k % 512 != 0) {
+            const size_t dwords = mx_tiled_bytes(rows, k) / 4;
+            hipLaunchKernelGGL(mx_tiled_fill_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0, s, (uint32_t*)scale, dwords);
+        }
+        hipLaunchKernelGGL(quant_mxfp4_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+    } else {
+        hipLaunchKernelGGL(quant_mxfp4_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+    }
     return launch_status();
 }
 

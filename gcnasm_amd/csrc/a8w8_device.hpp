@@ -16,7 +16,9 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 #define A8W8_LDS __attribute__((address_space(3)))
 
 // MODE_BF16: A and B hold bf16 (the a16w16 sibling), no scales; the kernels see them as byte matrices of 2k columns
-enum : int { MODE_TENSOR = 0, MODE_ROWCOL = 1, MODE_BLOCK = 2, MODE_MX = 3, MODE_MXT = 4, MODE_BF16 = 5 };
+// MODE_F4 / MODE_F4T: A and B hold packed E2M1 (MXFP4: two elements per byte, even K in the low nibble) with
+// row-major / tiled E8M0 scales; the kernels see byte matrices of k/2 columns
+enum : int { MODE_TENSOR = 0, MODE_ROWCOL = 1, MODE_BLOCK = 2, MODE_MX = 3, MODE_MXT = 4, MODE_BF16 = 5, MODE_F4 = 6, MODE_F4T = 7 };
 
 // Byte position of the E8M0 exponent of (row, 32-wide K block kblk) in the tiled MX scale layout
 //   [K/512][ceil(rows/64)][pair of K steps: 2][r16: 16][g: 4][jp: 2][par: 2][s: 2]       (1 byte each)

@@ -256,6 +256,42 @@ __global__ void __launch_bounds__(256) quant_mx_kernel(const float* src, int row
 // One thread per output dword: two tiles x two K steps of one (64-row block, r16, g, jp).
 // Consecutive threads write consecutive dwords.  Rows past `rows` and blocks past k get 127
 // (scale 1.0; their products are never formed or never stored).
+// MXFP4: one E8M0 exponent per 32 K-elements, e = ceil(log2(amax/6)) clamped to [-127, 127]; elements
+// become E2M1 (round to nearest, ties to the even mantissa bit, saturating at 6), two per byte with
+// the even K index in the low nibble.  32 lanes per block; even lanes write the byte.
+A8W8_DEV unsigned e2m1_encode(float x)
+{
+    const float a = fabsf(x);
+    const unsigned code = (a > 0.25f) + (a >= 0.75f) + (a > 1.25f) + (a >= 1.75f) + (a > 2.5f) + (a >= 3.5f) + (a > 5.0f);
+    return ((__float_as_uint(x) >> 31) << 3) | (a != a ? 7u : code);
+}
+template <bool TILED>
+__global__ void __launch_bounds__(256) quant_mxfp4_kernel(const float* src, int rows, int k, int ld, uint8_t* q,
+                                                          uint8_t* scale)
+{
+    const int blocks = k >> 5;
+    const long long idx = ((long long)blockIdx.x * 256 + threadIdx.x) >> 5;
+    if (idx >= (long long)rows * blocks) return;
+    const int row = (int)(idx / blocks), g = (int)(idx % blocks);
+    const int l = threadIdx.x & 31;
+    const float v = src[(long long)row * ld + g * 32 + l];
+    float amax = fabsf(v);
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float t = __fdiv_rn(amax, 6.0f);
+    int e = -127;
+    if (t > 0.f) {
+        int ex;
+        const float f = frexpf(t, &ex);          // t = f * 2^ex, f in [0.5, 1)
+        e = (f == 0.5f) ? ex - 1 : ex;
+        e = max(-127, min(127, e));
+    }
+    if (l == 0) scale[TILED ? mx_tiled_index(rows, row, g) : (size_t)row * blocks + g] = (uint8_t)(e + 127);
+    const unsigned code = e2m1_encode(ldexpf(v, -e));
+    const unsigned hi = __shfl_down(code, 1, 64);
+    if ((l & 1) == 0) q[(long long)row * (k >> 1) + ((g * 32 + l) >> 1)] = (uint8_t)(code | (hi << 4));
+}
+
 // One launch for one or two scale arrays (the A-side and the B-side scales of a GEMM).  A group of
 // 64 threads handles one 1 KiB unit (64 rows x 16 K blocks): thread r copies the 16 bytes of row r
 // into LDS, then thread t gathers and writes bytes 16t..16t+15 of the unit.  256 threads = 4 units.

@@ -80,4 +80,47 @@ __global__ void __launch_bounds__(256) gemm_a16w16_general(const unsigned short*
     else ((float*)c)[ci] = sum;
 }
 
+A8W8_DEV float e2m1_to_f32(unsigned nibble)
+{
+    // +-{0, 0.5, 1, 1.5, 2, 3, 4, 6}: exponent field 0 is the subnormal pair {0, 0.5}
+    const unsigned e = (nibble >> 1) & 3, m = nibble & 1;
+    const float v = e == 0 ? 0.5f * (float)m : __builtin_ldexpf(1.0f + 0.5f * (float)m, (int)e - 1);
+    return (nibble & 8) ? -v : v;
+}
+
+// MXFP4 x MXFP4 -> fp32 accumulate, any shape: packed E2M1 operands [rows][k/2] (even K in the low nibble),
+// E8M0 scales row-major [rows][k/32] or tiled; the oracle's order of operations (product, times scale, add).
+template <int CDT, bool TILED>
+__global__ void __launch_bounds__(256) gemm_a4w4_general(const uint8_t* a, const uint8_t* b, const uint8_t* sfa, const uint8_t* sfb,
+                                                         void* c, int m, int n, int k, int lda_bytes, int ldb_bytes, int ldc,
+                                                         int stride_sfa, int stride_sfb, long long a_batch, long long b_batch,
+                                                         long long c_batch, long long sfa_batch, long long sfb_batch)
+{
+#pragma clang fp contract(off)
+    const int j = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int i = blockIdx.y * 16 + (threadIdx.x >> 4);
+    const int batch = blockIdx.z;
+    if (i >= m || j >= n) return;
+    const uint8_t* ar = a + batch * a_batch + (long long)i * lda_bytes;
+    const uint8_t* br = b + batch * b_batch + (long long)j * ldb_bytes;
+    const uint8_t* ea = sfa + batch * sfa_batch;
+    const uint8_t* eb = sfb + batch * sfb_batch;
+    float sum = 0.f;
+    for (int g = 0; g < k / 32; ++g) {
+        const uint8_t xa = TILED ? ea[mx_tiled_index(m, i, g)] : ea[(long long)i * stride_sfa + g];
+        const uint8_t xb = TILED ? eb[mx_tiled_index(n, j, g)] : eb[(long long)j * stride_sfb + g];
+        const float scale = e8m0_pair_scale(xa, xb);
+        for (int p = g * 32; p < g * 32 + 32; ++p) {
+            const float av = e2m1_to_f32((ar[p >> 1] >> ((p & 1) * 4)) & 15u);
+            const float bv = e2m1_to_f32((br[p >> 1] >> ((p & 1) * 4)) & 15u);
+            const float prod = av * bv;
+            const float term = prod * scale;
+            sum = sum + term;
+        }
+    }
+    const long long ci = batch * c_batch + (long long)i * ldc + j;
+    if constexpr (CDT == C_BF16) ((unsigned short*)c)[ci] = bf16_bits(sum);
+    else ((float*)c)[ci] = sum;
+}
+
 }  // namespace a8w8

@@ -48,7 +48,7 @@ constexpr int PERSIST_LDS_BYTES_ROWCOL = GEMM_LDS_BYTES + 2 * ROWCOL_SCALE_BYTES
 #define A8W8_NPF_MX 1
 #endif
 #define A8W8_PREFETCH_A(mode)                                                                        \
-    ((mode) == MODE_TENSOR || (mode) == MODE_BF16 ? 4 : (mode) == MODE_ROWCOL ? A8W8_NPF_ROWCOL : (mode) == MODE_MXT ? A8W8_NPF_MXT \
+    ((mode) == MODE_TENSOR || (mode) == MODE_BF16 ? 4 : (mode) == MODE_ROWCOL ? A8W8_NPF_ROWCOL : (mode) == MODE_MXT || (mode) == MODE_F4T ? A8W8_NPF_MXT \
                                                      : (mode) == MODE_MX ? A8W8_NPF_MX : 0)
 #ifndef A8W8_PERSIST_BLK_LAG
 #define A8W8_PERSIST_BLK_LAG 4
@@ -82,6 +82,13 @@ A8W8_DEV v4f mfma_mx_sel(v8i a, v8i b, v4f c, int scale_a, int scale_b)
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, OA, scale_a, OB, scale_b);
 }
 
+// the same for packed E2M1 operands (format 4 for A and B; only the low four operand registers are read)
+template <int OA, int OB>
+A8W8_DEV v4f mfma_f4_sel(v8i a, v8i b, v4f c, int scale_a, int scale_b)
+{
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 4, 4, OA, scale_a, OB, scale_b);
+}
+
 struct PersistParams {
     GemmParams g;
     int batch;        // work items = batch * tiles_m * tiles_n, walked with stride gridDim.x
@@ -97,9 +104,15 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     const int lane = tid & 63;
     const int wave = wave_uniform(tid >> 6);
     const int wave_m = wave >> 1, wave_n = wave & 1;
-    constexpr bool IS_MX = MODE == MODE_MX || MODE == MODE_MXT;
+    // MODE_F4T (packed E2M1 operands): a 128-byte K step holds 256 elements = eight scale blocks = one
+    // "pair of K steps" of the tiled scale layout, so the tiled-MX plumbing serves it with two steps
+    // per scale group, a scale fetch every step, and two 16x16x128 FP4 MFMAs per fragment pair.
+    constexpr bool TILED_SF = MODE == MODE_MXT || MODE == MODE_F4T;
+    constexpr bool IS_MX = MODE == MODE_MX || TILED_SF;
+    constexpr int GROUP_SHIFT = MODE == MODE_F4T ? 1 : 2;          // log2(K steps per scale group)
+    constexpr int GROUP_MASK = (1 << GROUP_SHIFT) - 1;
     // tiled MX scales are laid out for A tiles whose rows are dealt like the B tiles' rows
-    constexpr bool PERM_A = MODE == MODE_MXT;
+    constexpr bool PERM_A = TILED_SF;
     const int r16 = lane & 15, g = lane >> 4;
     const int nk = p.k / BK;                       // >= 2 (checked by the host)
     const int tiles = p.tiles_m * p.tiles_n;
@@ -107,7 +120,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     // ---------------------------------------------------------------- load side state
     // position of the stage whose loads are being issued: (item, k step), two steps ahead
     int ld_item = blockIdx.x, ld_ks = 0;
-    const int groups_per_tile = (nk + 3) >> 2;      // MX scale groups (4 K steps each) per tile
+    const int groups_per_tile = (nk + GROUP_MASK) >> GROUP_SHIFT;   // MX scale groups per tile
     int ld_gbase = 0, cur_gbase = 0;                // running group count: picks the scale buffer
     __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_sf;
     int ld_m0 = 0, ld_n0 = 0, voff_sf = 0;            // tile origin at the load position (wave-uniform)
@@ -136,7 +149,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             rsrc_sf = make_rsrc(base, (uint32_t)(rows - 1) * stride + (uint32_t)(p.k >> 5));
             voff_sf = min((is_b ? n0 : m0) + (wave & 3) * 64 + lane, rows - 1) * stride;
         }
-        if constexpr (MODE == MODE_MXT) {
+        if constexpr (TILED_SF) {
             // tiled scales: a 64-row block's exponents for four K steps are 1 KiB of contiguous memory
             // in the order the lanes read them, so wave w copies block (w & 3) of the A tile (waves
             // 0-3) or of the B tile (waves 4-7) with one load of eight whole cache lines.
@@ -145,7 +158,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             const uint8_t* base = is_b ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
                                        : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
             const int nblk = (rows + 63) >> 6;
-            rsrc_sf = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, p.k));   // blocks past the edge read 0
+            const int k_elems = MODE == MODE_F4T ? 2 * p.k : p.k;
+            rsrc_sf = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, k_elems));   // blocks past the edge read 0
             voff_sf = (((is_b ? n0 : m0) >> 6) + (wave & 3)) * 1024 + lane * 16;
             sf_group_stride = wave_uniform(nblk * 1024);
         }
@@ -234,9 +248,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     };
     // natural MX scales: B tile t at + (t >> 1) * 512 + (t & 1) * 64; tiled: tile t at + t * 256, dword g
     // tiled: 1 KiB per 64-row block = [pair of K steps][lane (r16, g)][8 bytes]
-    const int rd_sfa = MODE == MODE_MXT ? GEMM_LDS_BYTES + wave_m * 1024 + lane_rg * 8
+    const int rd_sfa = TILED_SF ? GEMM_LDS_BYTES + wave_m * 1024 + lane_rg * 8
                                         : GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16;
-    const int rd_sfb = MODE == MODE_MXT
+    const int rd_sfb = TILED_SF
                            ? GEMM_LDS_BYTES + 4096 + wave_n * 2048 + lane_rg * 8
                            : GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + 8 * (r16 >> 2) + (r16 & 3)) * 16;
 
@@ -303,9 +317,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             for (int t = 0; t < TN; ++t)
                 mx_sb_next[t] = *(const int*)(s + rd_sfb + (t >> 1) * 512 + (t & 1) * 64);
         }
-        if constexpr (MODE == MODE_MXT) {
-            // called for the first step of a pair: the lane's eight bytes per 64-row block
-            const char* s = smem + ((gbase + (kstep >> 2)) & 1) * MX_GROUP_BYTES + ((kstep >> 1) & 1) * 512;
+        if constexpr (TILED_SF) {
+            // called for the first step of a pair (FP4: for every step, which is a pair by itself): the
+            // lane's eight bytes per 64-row block
+            const int pair = MODE == MODE_F4T ? (kstep & 1) : ((kstep >> 1) & 1);
+            const char* s = smem + ((gbase + (kstep >> GROUP_SHIFT)) & 1) * MX_GROUP_BYTES + pair * 512;
             mxt_a_next = *(const v2i*)(s + rd_sfa);
             const v2i lo = *(const v2i*)(s + rd_sfb), hi = *(const v2i*)(s + rd_sfb + 1024);
             mxt_b_next = v4i{lo.x, lo.y, hi.x, hi.y};
@@ -322,7 +338,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
 #pragma unroll
             for (int t = 0; t < TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sb_next[t], 8 * g, 8);
         }
-        if constexpr (MODE == MODE_MXT) {
+        if constexpr (TILED_SF) {
             mxt_a = mxt_a_next;
             mxt_b = mxt_b_next;
         }
@@ -448,7 +464,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         constexpr int P = decltype(parity)::value;
         Frags& cur = F[PREFETCH_FRAGS ? P : 0];
         Frags& nxt = F[PREFETCH_FRAGS ? P ^ 1 : 0];
-        if constexpr (MODE != MODE_MXT || P == 0) rotate_step_scales();
+        if constexpr (MODE != MODE_MXT || P == 0) rotate_step_scales();   // tiled MXFP8: one dword serves two steps
 #pragma unroll
         for (int t = NPF; t < TM; ++t) cur.a[t] = read_frag_a(P, t);
         if constexpr (!PREFETCH_FRAGS) cur.b0 = read_frag_b(P, 0);
@@ -479,7 +495,15 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             A8W8_PERSIST_SCHED_BARRIER();
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                if constexpr (MODE == MODE_MXT) {
+                if constexpr (MODE == MODE_F4T) {
+                    // first halves of the fragments here (op_sel byte 2*(tile parity)), second halves after
+                    // the loop: format 4 = E2M1 for both operands, the upper four operand registers unused
+                    const int sb = mxt_b[j >> 1], sa = mxt_a[i >> 1];
+                    const v8i fb4 = {fb[j][0], fb[j][1], fb[j][2], fb[j][3], 0, 0, 0, 0};
+                    const v8i fa4 = {cur.a[i][0], cur.a[i][1], cur.a[i][2], cur.a[i][3], 0, 0, 0, 0};
+                    acc[i][j] = (j & 1) ? ((i & 1) ? mfma_f4_sel<2, 2>(fb4, fa4, acc[i][j], sb, sa) : mfma_f4_sel<2, 0>(fb4, fa4, acc[i][j], sb, sa))
+                                        : ((i & 1) ? mfma_f4_sel<0, 2>(fb4, fa4, acc[i][j], sb, sa) : mfma_f4_sel<0, 0>(fb4, fa4, acc[i][j], sb, sa));
+                } else if constexpr (MODE == MODE_MXT) {
                     // K steps come in pairs and tiles start on even steps, so the step inside the
                     // pair is the LDS stage parity P
                     const int sb = mxt_b[j >> 1], sa = mxt_a[i >> 1];
@@ -518,6 +542,16 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                                                                                  0, 0, 0);
                 }
             }
+            if constexpr (MODE == MODE_F4T) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const int sb = mxt_b[j >> 1], sa = mxt_a[i >> 1];
+                    const v8i fb4 = {fb[j][4], fb[j][5], fb[j][6], fb[j][7], 0, 0, 0, 0};
+                    const v8i fa4 = {cur.a[i][4], cur.a[i][5], cur.a[i][6], cur.a[i][7], 0, 0, 0, 0};
+                    acc[i][j] = (j & 1) ? ((i & 1) ? mfma_f4_sel<3, 3>(fb4, fa4, acc[i][j], sb, sa) : mfma_f4_sel<3, 1>(fb4, fa4, acc[i][j], sb, sa))
+                                        : ((i & 1) ? mfma_f4_sel<1, 3>(fb4, fa4, acc[i][j], sb, sa) : mfma_f4_sel<1, 1>(fb4, fa4, acc[i][j], sb, sa));
+                }
+            }
             if constexpr (MODE == MODE_BF16) {
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
@@ -531,7 +565,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
 #if A8W8_PERSIST_SG
             if constexpr (MODE != MODE_BLOCK) {
                 // spread the two LDS reads of the next B fragment between this group's MFMAs
-                constexpr int MPF = MODE == MODE_BF16 ? 2 : 1;      // MFMAs per operand fragment pair
+                constexpr int MPF = (MODE == MODE_BF16 || MODE == MODE_F4T) ? 2 : 1;      // MFMAs per operand fragment pair
                 if (j + 1 < TN) {
                     __builtin_amdgcn_sched_group_barrier(0x008, MPF, 0);
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -554,7 +588,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             if (j == 2) {
                 advance_ld();
                 if constexpr (IS_MX) {
-                    if ((ld_ks & 3) == 0) issue_mx_group(ld_ks >> 2);   // scales of steps ld_ks .. ld_ks+3
+                    if ((ld_ks & GROUP_MASK) == 0) issue_mx_group(ld_ks >> GROUP_SHIFT);   // scales of the group starting at ld_ks
                 }
                 if constexpr (MODE == MODE_BLOCK) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, 0);
             }
@@ -576,6 +610,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                 }
                 if constexpr (MODE == MODE_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
                 if constexpr (MODE == MODE_MXT && P == 1) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
+                if constexpr (MODE == MODE_F4T) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
             }
             if (j == 7) {
                 issue_one(P, ld_ks, 4);

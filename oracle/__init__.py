@@ -68,6 +68,12 @@ def lib():
         L.orc_mx_tiled_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
         L.orc_mx_tile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
         L.orc_mx_untile_scales.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p]
+        L.orc_e2m1_decode.restype = ctypes.c_float
+        L.orc_e2m1_decode.argtypes = [ctypes.c_uint8]
+        L.orc_e2m1_encode.restype = ctypes.c_uint8
+        L.orc_e2m1_encode.argtypes = [ctypes.c_float]
+        L.orc_gemm_ref_mxfp4.argtypes = [_u8p, _u8p, _u8p, _u8p, _f32p] + [ctypes.c_int] * 5
+        L.orc_quant_mxfp4.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _u8p]
         L.orc_gemm_bf16_ref.argtypes = [_u16p, _u16p, _f32p] + [ctypes.c_int] * 6
         L.orc_quant_tensor.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p]
         L.orc_quant_rowwise.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _u8p, _f32p]
@@ -229,6 +235,34 @@ def mx_untile_scales(tiled, rows, k):
     out = np.zeros((rows, k // 32), np.uint8)
     lib().orc_mx_untile_scales(_p(tiled, _u8p), rows, k, k // 32, _p(out, _u8p))
     return out
+
+
+def e2m1_decode_packed(q):
+    """[rows, K/2] packed E2M1 bytes -> fp32 [rows, K] (even K in the low nibble)."""
+    q = _c(q, np.uint8)
+    table = np.array([lib().orc_e2m1_decode(c) for c in range(16)], np.float32)
+    out = np.empty(q.shape[:-1] + (q.shape[-1] * 2,), np.float32)
+    out[..., 0::2] = table[q & 15]
+    out[..., 1::2] = table[q >> 4]
+    return out
+
+
+def gemm_ref_mxfp4(a, b, ea, eb, rows=None):
+    a, b, ea, eb = _c(a, np.uint8), _c(b, np.uint8), _c(ea, np.uint8), _c(eb, np.uint8)
+    m, n, k = a.shape[0], b.shape[0], a.shape[1] * 2
+    r0, r1 = rows if rows is not None else (0, m)
+    c = np.zeros((m, n), np.float32)
+    lib().orc_gemm_ref_mxfp4(_p(a, _u8p), _p(b, _u8p), _p(ea, _u8p), _p(eb, _u8p), _p(c, _f32p), m, n, k, r0, r1)
+    return c[r0:r1]
+
+
+def quantize_mxfp4(x):
+    x = _c(x, np.float32)
+    rows, k = x.shape
+    q = np.empty((rows, k // 2), np.uint8)
+    s = np.empty((rows, k // 32), np.uint8)
+    lib().orc_quant_mxfp4(_p(x, _f32p), rows, k, k, _p(q, _u8p), _p(s, _u8p))
+    return q, s
 
 
 def gemm_bf16_ref(a_bits, b_bits):

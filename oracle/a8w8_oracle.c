@@ -23,6 +23,9 @@
  *       exact-integer inputs, scale-mode reductions.
  *   orc_preshuffle_b       bijection + flatmm(A, shuffle(B)) == gemm(A, B).
  *   orc_gemm_bf16_ref      float64 matmul on small shapes, exact-integer inputs.
+ *   orc_e2m1_* / orc_gemm_ref_mxfp4 / orc_quant_mxfp4   the OCP MX value table (16 codes, checked one by
+ *       one), nearest-even against a brute force over the table, float64 matmul of the decoded
+ *       operands, the quantiser's properties (largest element in (3, 6], error within half a step).
  *   orc_quant_*            no reference code (its harness has no quantiser): the recipe of the
  *       benchmark configurations, fixed by properties -- the group's largest element maps to
  *       +-448 (row/block) or into (224, 448] (MX, never saturating), dequantisation error within
@@ -294,6 +297,78 @@ ORC_API void orc_gemm_ref_mx(const uint8_t* a, const uint8_t* b, const uint8_t* 
             c[(size_t)i * ldc + j] = sum;
         }
     }
+}
+
+/* ------------------------------------------------------------ MXFP4 (OCP MX, E2M1 elements)
+ * The reference stops at naming the instruction's FP4 format (wmma_opus_rdna4/opus/opus.hpp:1854-1855);
+ * arithmetic per the OCP Microscaling spec v1.0: E2M1 = sign, 2 exponent bits (bias 1), 1 mantissa bit,
+ * values +-{0, 0.5, 1, 1.5, 2, 3, 4, 6}, no NaN / infinity; two elements per byte, the even K index in
+ * the low nibble; one E8M0 scale per 32 elements. */
+static const float e2m1_values[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+ORC_API float orc_e2m1_decode(uint8_t nibble)
+{
+    const float v = e2m1_values[nibble & 7];
+    return (nibble & 8) ? -v : v;
+}
+/* round to nearest, ties to the value with an even mantissa bit, saturating at +-6 */
+ORC_API uint8_t orc_e2m1_encode(float x)
+{
+    const uint8_t sign = signbit(x) ? 8 : 0;
+    const float a = fabsf(x);
+    if (!(a == a)) return (uint8_t)(sign | 7);              /* NaN has no code: saturate */
+    int best = 0;
+    for (int c = 1; c < 8; ++c) {
+        const float d0 = fabsf(a - e2m1_values[best]), d1 = fabsf(a - e2m1_values[c]);
+        if (d1 < d0 || (d1 == d0 && (c & 1) == 0)) best = c;
+    }
+    return (uint8_t)(sign | best);
+}
+static inline float fp4_at(const uint8_t* row, int p) { return orc_e2m1_decode((uint8_t)((row[p >> 1] >> ((p & 1) * 4)) & 15)); }
+
+/* C = A * B^T for packed E2M1 A [m][k/2], B [n][k/2] and E8M0 scales [rows][k/32]: gemm_ref's loop
+ * (host.cc:66-90) with group_k = 32 and scale = 2^(ea-127) * 2^(eb-127). */
+ORC_API void orc_gemm_ref_mxfp4(const uint8_t* a, const uint8_t* b, const uint8_t* ea, const uint8_t* eb, float* c,
+                                int m, int n, int k, int row_begin, int row_end)
+{
+    (void)m;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int i = row_begin; i < row_end; ++i)
+        for (int j = 0; j < n; ++j) {
+            const uint8_t* a_row = a + (size_t)i * (k / 2);
+            const uint8_t* b_row = b + (size_t)j * (k / 2);
+            float sum = 0.0f;
+            for (int g = 0; g < k / 32; ++g) {
+                const uint8_t xa = ea[(size_t)i * (k / 32) + g], xb = eb[(size_t)j * (k / 32) + g];
+                const float scale = (xa == 255 || xb == 255) ? u2f(0x7fc00000u) : ldexpf(1.0f, (int)xa + (int)xb - 254);
+                for (int p = g * 32; p < g * 32 + 32; ++p) sum += fp4_at(a_row, p) * fp4_at(b_row, p) * scale;
+            }
+            c[(size_t)i * n + j] = sum;
+        }
+}
+
+/* MXFP4 quantiser: e = clamp(ceil(log2(amax/6)), -127, 127), byte e + 127, q = E2M1(x * 2^-e): the
+ * ceiling keeps the largest element at or below 6. */
+ORC_API void orc_quant_mxfp4(const float* x, int rows, int k, int ld, uint8_t* q, uint8_t* scale)
+{
+    for (int r = 0; r < rows; ++r)
+        for (int g = 0; g < k / 32; ++g) {
+            float amax = 0.0f;
+            for (int p = 0; p < 32; ++p) amax = fmaxf(amax, fabsf(x[(size_t)r * ld + g * 32 + p]));
+            const float t = amax / 6.0f;
+            int e = -127;
+            if (t > 0.0f) {
+                e = ilogbf(t);
+                if (t > ldexpf(1.0f, e)) ++e;
+                if (e < -127) e = -127;
+                if (e > 127) e = 127;
+            }
+            scale[(size_t)r * (k / 32) + g] = (uint8_t)(e + 127);
+            for (int p = 0; p < 32; p += 2) {
+                const uint8_t lo = orc_e2m1_encode(ldexpf(x[(size_t)r * ld + g * 32 + p], -e));
+                const uint8_t hi = orc_e2m1_encode(ldexpf(x[(size_t)r * ld + g * 32 + p + 1], -e));
+                q[(size_t)r * (k / 2) + (g * 32 + p) / 2] = (uint8_t)(lo | (hi << 4));
+            }
+        }
 }
 
 /* Selected (i,j) probes of either GEMM, for spot checks at sizes where a slab is too slow.

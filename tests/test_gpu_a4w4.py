@@ -1,0 +1,101 @@
+"""MXFP4 (packed E2M1 + E8M0) on the GPU against the oracle: quantiser bit for bit, GEMM exact on the
+general kernel and on integer inputs, |C - Cref| <= 1e-2*|Cref| + 1e-2 on the pipelined kernel (with the
+same allowance for cancellation-dominated outputs as the MXFP8 tests: under 0.1%, each within 1e-4 of
+sum|a||b|s of the float64 value)."""
+import numpy as np
+import pytest
+import torch
+
+import gcnasm_amd as g
+from gpu_util import MFMA_ACC_ERR, dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _x(rows, k, seed):
+    rng = np.random.Generator(np.random.Philox(seed))
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    return x * np.exp2(rng.integers(-4, 5, (rows, k // 32))).repeat(32, axis=1).astype(np.float32)
+
+
+def _exact(orc, qa, qb, ea, eb):
+    A = orc.e2m1_decode_packed(qa).astype(np.float64) * np.exp2(ea.astype(np.float64) - 127).repeat(32, axis=1)
+    B = orc.e2m1_decode_packed(qb).astype(np.float64) * np.exp2(eb.astype(np.float64) - 127).repeat(32, axis=1)
+    return A @ B.T, np.abs(A) @ np.abs(B).T
+
+
+@pytest.mark.parametrize("rows,k", [(1, 32), (37, 96), (256, 1024), (70, 7168)])
+def test_quantiser_matches_oracle(orc, rows, k):
+    x = _x(rows, k, 3 + rows)
+    x[0, :32] = [6 * 2.0 ** -3] + [0] * 31                    # exactly a power of two times 6
+    q, s = g.quantize_mxfp4(dev(x))
+    qr, sr = orc.quantize_mxfp4(x)
+    assert (s.cpu().numpy() == sr).all() and (q.cpu().numpy() == qr).all()
+    qt, st = g.quantize_mxfp4(dev(x), tiled=True)
+    assert torch.equal(qt, q) and (st.cpu().numpy() == orc.mx_tile_scales(sr)).all()
+
+
+@pytest.mark.parametrize("shape", [(37, 53, 96), (64, 64, 256), (70, 40, 384)])
+def test_general_kernel_is_bit_exact(orc, shape):
+    m, n, k = shape
+    qa, ea = orc.quantize_mxfp4(_x(m, k, 11))
+    qb, eb = orc.quantize_mxfp4(_x(n, k, 12))
+    ref = orc.gemm_ref_mxfp4(qa, qb, ea, eb)
+    got = g.gemm_a4w4(dev(qa), dev(qb), dev(ea), dev(eb), g.MX, c_dtype=g.FP32).cpu().numpy()
+    assert (got == ref).all()
+    ta, tb = g.mx_tile_scales(dev(ea)), g.mx_tile_scales(dev(eb))
+    got = g.gemm_a4w4(dev(qa), dev(qb), ta, tb, g.MX_TILED, c_dtype=g.FP32).cpu().numpy()
+    assert (got == ref).all()
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 512), (512, 256, 2048), (130, 270, 1024), (300, 520, 768)])
+def test_pipelined_kernel(orc, shape):
+    m, n, k = shape
+    qa, ea = orc.quantize_mxfp4(_x(m, k, 21 + m))
+    qb, eb = orc.quantize_mxfp4(_x(n, k, 22 + n))
+    ref = orc.gemm_ref_mxfp4(qa, qb, ea, eb)
+    exact, mag = _exact(orc, qa, qb, ea, eb)
+    ta, tb = g.mx_tile_scales(dev(ea)), g.mx_tile_scales(dev(eb))
+    c32 = g.gemm_a4w4(dev(qa), dev(qb), ta, tb, c_dtype=g.FP32).cpu().numpy()
+    assert (np.abs(c32 - exact) <= MFMA_ACC_ERR * mag + 1e-30).all()
+    c = g.gemm_a4w4(dev(qa), dev(qb), ta, tb).float().cpu().numpy()
+    miss = ~(np.abs(c - ref) <= 1e-2 * np.abs(ref) + 1e-2)
+    assert miss.mean() <= 1e-3
+    assert (np.abs(c - exact)[miss] <= MFMA_ACC_ERR * mag[miss] + 2.0 ** -8 * np.abs(exact)[miss]).all()
+
+
+def test_scale_bytes_reach_the_right_lane_and_half(orc):
+    """Distinct powers of two per (row, 32-block) on exactly representable operands: any mix-up of row,
+    block, fragment half or op_sel byte changes the exact result."""
+    m, n, k = 256, 512, 1024
+    rng = np.random.Generator(np.random.Philox(9))
+    qa = rng.integers(0, 256, (m, k // 2), dtype=np.uint8)
+    qb = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    ea = (125 + (np.arange(m)[:, None] * 3 + np.arange(k // 32)[None, :]) % 4).astype(np.uint8)
+    eb = (126 + (np.arange(n)[:, None] * 5 + np.arange(k // 32)[None, :] * 2) % 3).astype(np.uint8)
+    exact, _ = _exact(orc, qa, qb, ea, eb)                     # sums of multiples of 2^-6 below 2^17: exact in fp32
+    got = g.gemm_a4w4(dev(qa), dev(qb), g.mx_tile_scales(dev(ea)), g.mx_tile_scales(dev(eb)), c_dtype=g.FP32).cpu().numpy()
+    assert (got == exact).all()
+
+
+def test_full_size_8192(orc):
+    m = n = k = 8192
+    gen = torch.Generator(device="cuda"); gen.manual_seed(7)
+    xa = torch.randn((m, k), generator=gen, device="cuda")
+    xb = torch.randn((n, k), generator=gen, device="cuda")
+    qa, ta = g.quantize_mxfp4(xa, tiled=True)
+    qb, tb = g.quantize_mxfp4(xb, tiled=True)
+    _, ea = g.quantize_mxfp4(xa[:8].contiguous())
+    _, eb = g.quantize_mxfp4(xb)
+    del xa, xb
+    c = g.gemm_a4w4(qa, qb, ta, tb)
+    ref = orc.gemm_ref_mxfp4(qa[:8].cpu().numpy(), qb.cpu().numpy(), ea.cpu().numpy(), eb.cpu().numpy())
+    got = c[:8].float().cpu().numpy()
+    assert (np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-2).mean() >= 0.999
+    np.testing.assert_allclose(got, ref, rtol=2e-2, atol=2e-2 * np.abs(ref).max())
+    # permuting the rows of A (with their scales) permutes the rows of C bit for bit
+    perm = torch.randperm(m, generator=torch.Generator().manual_seed(3)).cuda()
+    qa_p = qa[perm].contiguous()
+    e_np = orc.mx_untile_scales(ta.cpu().numpy(), m, k)          # row-major scales of A, to permute and re-tile
+    tp = g.mx_tile_scales(dev(e_np[perm.cpu().numpy()]))
+    assert torch.equal(g.gemm_a4w4(qa_p, qb, tp, tb), c[perm])
