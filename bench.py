@@ -28,6 +28,7 @@ METRIC = "FP8 GEMM TFLOPS & % gfx950 FP8 MFMA peak; HBM GB/s for M=16 flatmm"
 PEAK_FP8_TFLOPS = 5000.0      # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E, published
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA, published
+PEAK_FP4_TFLOPS = 10100.0     # MI355X dense FP4 MFMA, published
 # Bytes that crossed the L2 <-> fabric boundary per launch, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 117 MB device copy calibrates; profiles/).
 MEASURED_TRAFFIC = {"mxfp8_8192": 1.03e9, "flatmm_16x16384x7168": 1.190e8}
@@ -41,6 +42,8 @@ WORKLOADS = {
     "flatmm_16x16384x7168": ("flat", 16, 16384, 7168, 118145088),
     # the bf16 sibling (a16w16_gemm), priced against the dense bf16 peak
     "a16w16_4096": ("bf16", 4096, 4096, 4096, 100663296),
+    # MXFP4 (a4w4_gemm, tiled scales), priced against the dense FP4 peak
+    "mxfp4_8192": ("f4", 8192, 8192, 8192, 205520896),
 }
 
 
@@ -54,6 +57,10 @@ def make_inputs(name, torch, g, seed):
     def normal(rows):
         return torch.randn((rows, k), generator=gen, device="cuda", dtype=torch.float32)
 
+    if mode == "f4":
+        a, sfa = g.quantize_mxfp4(normal(m), tiled=True)
+        b, sfb = g.quantize_mxfp4(normal(n), tiled=True)
+        return dict(a=a, b=b, sfa=sfa, sfb=sfb, mode=g.MX_TILED)
     if mode == "bf16":
         a = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
         b = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
@@ -157,7 +164,7 @@ def run_workload(name, torch, g, steps, warmup, seed, headline=True):
         gemm_args = args_for(inp["b"], 0)
         gemm_ref_ = ctypes.byref(gemm_args)
 
-        entry = L.a16w16_gemm if mode == "bf16" else L.a8w8_gemm
+        entry = L.a16w16_gemm if mode == "bf16" else L.a4w4_gemm if mode == "f4" else L.a8w8_gemm
 
         def fn_direct(i):
             if entry(gemm_ref_, stream) != 0:
@@ -191,11 +198,14 @@ def run_workload(name, torch, g, steps, warmup, seed, headline=True):
                        ms_row_major_scales_one_launch=ms_direct, tflops_row_major_scales_one_launch=flops / ms_direct / 1e9,
                        step="a8w8_mx_tile_scales_ab(sfa, sfb) + a8w8_gemm(MX_TILED)")
         else:
-            res["kernel"] = "gemm_a8w8_persist<bf16>" if mode == "bf16" else g.kernel_name(gemm_args)
+            res["kernel"] = ("gemm_a8w8_persist<bf16>" if mode == "bf16" else "gemm_a8w8_persist<mxfp4>" if mode == "f4"
+                             else g.kernel_name(gemm_args))
             ms, wall = timer(torch, fn, steps, warmup)
         res.update(ms_per_launch=ms, wall_ms_per_launch=wall, tflops=flops / ms / 1e9, gbs=abytes / ms / 1e6)
         if mode == "bf16":
             res["frac_bf16_peak"] = flops / ms / 1e9 / PEAK_BF16_TFLOPS
+        elif mode == "f4":
+            res["frac_fp4_peak"] = flops / ms / 1e9 / PEAK_FP4_TFLOPS
         else:
             res["frac_fp8_peak"] = flops / ms / 1e9 / PEAK_FP8_TFLOPS
     fn(0)
@@ -238,7 +248,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="mxfp8_8192", choices=sorted(w for w in WORKLOADS if WORKLOADS[w][0] != "bf16"))
+    ap.add_argument("--workload", default="mxfp8_8192", choices=sorted(w for w in WORKLOADS if WORKLOADS[w][0] not in ("bf16", "f4")))
     ap.add_argument("--seed", type=int, default=0xA8A80004)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="time only the selected workload")
