@@ -10,6 +10,7 @@
 #include "gemm_general.hpp"
 #include "gemm_persist.hpp"
 #include "gemm_tile.hpp"
+#include "gemm_wide.hpp"
 
 using namespace a8w8;
 
@@ -115,6 +116,14 @@ bool persist_ok(const a8w8_gemm_args* g)
            (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 30);
 }
 
+// The four-wave kernel walks K in pairs of steps and has the per-tensor, row/col and tiled-MX scale modes.
+bool wide_ok(const a8w8_gemm_args* g)
+{
+    if (g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_ROWCOL && g->scale_mode != A8W8_SCALE_MX_E8M0_TILED)
+        return false;
+    return persist_ok(g) && (g->k / BK) % 2 == 0;
+}
+
 template <int MODE, int CDT>
 int launch_general(const GemmParams& p, int batch, hipStream_t stream);
 
@@ -165,6 +174,34 @@ int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
     return launch_status();
 }
 
+// Four-wave persistent kernel (one wave per SIMD, 128 x 128 per wave).
+template <int MODE, int CDT>
+int launch_wide(const GemmParams& p, int batch, hipStream_t stream)
+{
+    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT) {
+        static bool attr_set[64];
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        auto kern = gemm_a8w8_wide<MODE, CDT>;
+        constexpr int lds_bytes = wide_lds_bytes(MODE);
+        if (!attr_set[dev & 63]) {
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+                return A8W8_ERR_LAUNCH;
+            attr_set[dev & 63] = true;
+        }
+        PersistParams pp;
+        pp.g = p;
+        pp.batch = batch;
+        pp.items = batch * p.tiles_m * p.tiles_n;
+        const int cus = g_num_cus[dev & 63] > 0 ? g_num_cus[dev & 63] : 256;
+        dim3 grid((unsigned)(pp.items < cus ? pp.items : cus), 1, 1);
+        hipLaunchKernelGGL(kern, grid, dim3(WIDE_THREADS), lds_bytes, stream, pp);
+        return launch_status();
+    } else {
+        return launch_persist<MODE, CDT>(p, batch, stream);
+    }
+}
+
 template <int MODE, int CDT>
 int launch_general(const GemmParams& p, int batch, hipStream_t stream)
 {
@@ -196,6 +233,10 @@ int dispatch_tiled(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
 int dispatch_persist(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
 {
     A8W8_DISPATCH(launch_persist, g->scale_mode, g->c_dtype, p, g->batch, s)
+}
+int dispatch_wide(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
+{
+    A8W8_DISPATCH(launch_wide, g->scale_mode, g->c_dtype, p, g->batch, s)
 }
 int dispatch_general(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
 {
@@ -240,6 +281,7 @@ int a8w8_gemm(const a8w8_gemm_args* g, void* hip_stream)
     const GemmParams p = make_params(g);
     hipStream_t s = (hipStream_t)hip_stream;
     if (!tiled_ok(g)) return dispatch_general(g, p, s);
+    if (wide_ok(g)) return dispatch_wide(g, p, s);
     return persist_ok(g) ? dispatch_persist(g, p, s) : dispatch_tiled(g, p, s);
 }
 
@@ -681,6 +723,7 @@ const char* a8w8_kernel_name(const a8w8_gemm_args* g)
     if (g->b_preshuffled) return validate_flat(g) == A8W8_OK ? "flatmm_a8w8" : nullptr;
     if (validate_common(g) != A8W8_OK) return nullptr;
     if (!tiled_ok(g)) return "gemm_a8w8_general";
+    if (wide_ok(g)) return "gemm_a8w8_wide";
     if (persist_ok(g)) return "gemm_a8w8_persist";
     return g->scale_mode == A8W8_SCALE_MX_E8M0_TILED ? "gemm_a8w8_general" : "gemm_a8w8_tile256";
 }

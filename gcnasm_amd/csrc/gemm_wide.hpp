@@ -1,0 +1,440 @@
+// Persistent dense A8W8 GEMM for gfx950 with four waves per workgroup and both operand fragment
+// sets resident in registers.
+//
+// Tile 256 x 256 x 128, 4 waves (2 along M x 2 along N), wave tile 128 x 128 = 8 x 8 MFMA tiles of
+// 16 x 16 x 128: 256 accumulator registers per lane and 16 operand fragments (128 registers).  Each
+// fragment is read from LDS once per K step, so a step moves 128 KiB out of LDS instead of the 192 KiB
+// of the eight-wave 64 x 128 layout; with one wave per SIMD nothing else hides an LDS wait, so the
+// schedule below never has one:
+//
+//  * A K step is four quadrants of 16 MFMAs: (aL,bL) (aL,bH) (aH,bH) (aH,bL) on even steps and
+//    (aL,bH) (aL,bL) (aH,bL) (aH,bH) on odd ones, where aL/aH are the fragments of the wave's A rows
+//    0-63 / 64-127 and bL/bH the same for B.  Consecutive quadrants share one set, so exactly one
+//    set of four fragments dies per quadrant; it is re-read (8 ds_read_b128, for the same step or the
+//    next one) while the quadrant after its death runs and is first used one quadrant later.
+//  * Seen from LDS, a quadrant reads one quarter of a stage (16 KiB: 64 + 64 rows of one operand, the
+//    same for all four waves).  Two barriers per step ("mid" after the second quadrant, "end" after
+//    the fourth) hand the two quarters read since the last barrier back to the loads, and each
+//    quadrant issues one quarter (four 1 KiB direct-to-LDS loads per wave) of the step after next.
+//    Every byte has 1.5 K steps to arrive.
+//  * Loads complete in issue order: "all but the newest 16" at a barrier is "the two quarters the
+//    next two quadrants read have landed".
+#pragma once
+#include <utility>
+
+#include "gemm_persist.hpp"
+
+namespace a8w8 {
+
+constexpr int WIDE_THREADS = 256;
+constexpr int WIDE_T = 8;                            // 8 x 8 MFMA tiles per wave
+constexpr int wide_lds_bytes(int mode)
+{
+    return GEMM_LDS_BYTES + (mode == MODE_MXT ? 2 * MX_GROUP_BYTES : mode == MODE_ROWCOL ? 2 * ROWCOL_SCALE_BYTES : 0);
+}
+
+// Scaled MFMA on accumulator registers, in place: c += (a . b) with byte OA of sa and byte OB of sb
+// as the E8M0 scales of the lane's 32-element K block (the selectors are instruction modifiers).
+A8W8_DEV void mfma_mx_asm(v4f& c, const v8i& a, const v8i& b, int sa, int sb, int oa, int ob)
+{
+#define A8W8_MX_CASE(OA, OB, ALO, AHI, BLO, BHI)                                                               \
+    case OA * 4 + OB:                                                                                            \
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[" #ALO "," #BLO         \
+                     ",0] op_sel_hi:[" #AHI "," #BHI ",0]"                                                      \
+                     : "+a"(c)                                                                                   \
+                     : "v"(a), "v"(b), "v"(sa), "v"(sb));                                                      \
+        break;
+    switch (oa * 4 + ob) {
+        A8W8_MX_CASE(0, 0, 0, 0, 0, 0) A8W8_MX_CASE(0, 1, 0, 0, 1, 0) A8W8_MX_CASE(0, 2, 0, 0, 0, 1) A8W8_MX_CASE(0, 3, 0, 0, 1, 1)
+        A8W8_MX_CASE(1, 0, 1, 0, 0, 0) A8W8_MX_CASE(1, 1, 1, 0, 1, 0) A8W8_MX_CASE(1, 2, 1, 0, 0, 1) A8W8_MX_CASE(1, 3, 1, 0, 1, 1)
+        A8W8_MX_CASE(2, 0, 0, 1, 0, 0) A8W8_MX_CASE(2, 1, 0, 1, 1, 0) A8W8_MX_CASE(2, 2, 0, 1, 0, 1) A8W8_MX_CASE(2, 3, 0, 1, 1, 1)
+        A8W8_MX_CASE(3, 0, 1, 1, 0, 0) A8W8_MX_CASE(3, 1, 1, 1, 1, 0) A8W8_MX_CASE(3, 2, 1, 1, 0, 1) A8W8_MX_CASE(3, 3, 1, 1, 1, 1)
+    }
+#undef A8W8_MX_CASE
+}
+
+template <int MODE, int CDT>
+__global__ void __launch_bounds__(WIDE_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
+gemm_a8w8_wide(PersistParams pp)
+{
+    static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT, "scale modes of the four-wave kernel");
+    constexpr bool IS_MXT = MODE == MODE_MXT;
+    // tiled MX scales are laid out for A tiles whose rows are dealt like the B tiles' rows
+    constexpr bool PERM_A = IS_MXT;
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const GemmParams& p = pp.g;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = wave_uniform(tid >> 6);
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int nk = p.k / BK;                       // >= 2 (checked by the host)
+    const int tiles = p.tiles_m * p.tiles_n;
+
+    // ---------------------------------------------------------------- load side
+    int ld_item = blockIdx.x, ld_ks = 0;           // the step whose quarters are being issued
+    __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b;
+    const int ld_row = wave * 8 + (lane >> 3);
+    // lane i of a 1 KiB load lands on row (i >> 3), slot (i & 7) of 8 consecutive tile rows; the slot
+    // holds K piece slot ^ key(row), key(row) = (row & 7) ^ (((row >> 3) & 3) << 1), and bits 3-4 of
+    // the tile row equal the wave number for every load this wave issues
+    const int ld_piece16 = ((lane & 7) ^ (((lane >> 3) ^ (wave << 1)) & 7)) * 16;
+    // Lane offsets of the sixteen loads of a step: they change only with the tile, and this kernel
+    // has registers to keep them, so a load costs one scalar add (its LDS address) and itself.
+    int ld_voff[16];
+    auto point_loads_at = [&](int item) __attribute__((always_inline)) {
+        item = min(item, pp.items - 1);            // past the end: keep loading valid data nobody reads
+        const int batch = item / tiles;
+        int tm, tn;
+        tile_of_block(item - batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+        rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
+        rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, (uint32_t)(p.n - 1) * p.ldb + p.k);
+#pragma unroll
+        for (int qt = 0; qt < 4; ++qt)
+#pragma unroll
+            for (int l = 0; l < 4; ++l) {
+                const int row = 128 * (l >> 1) + 64 * (qt & 1) + 32 * (l & 1) + ld_row;
+                ld_voff[qt * 4 + l] = qt < 2 ? __mul24(min(tm * BM + row, p.m - 1), p.lda) + ld_piece16
+                                             : __mul24(min(tn * BN + row, p.n - 1), p.ldb) + ld_piece16;
+            }
+    };
+    // Load l (0..3) of quarter qt (0 aL, 1 aH, 2 bL, 3 bH) of the step at the load position.  A quarter
+    // is tile rows [64h, 64h + 64) and [128 + 64h, 192 + 64h) of one operand (h = qt & 1): the L or H
+    // rows of both wave rows (A) or wave columns (B).  Wave w fills rows 8w.. and 32 + 8w.. of each.
+    int wave_lds = wave * 1024;
+    auto issue_one = [&](int stage, int qt, int l) __attribute__((always_inline)) {
+        const int row0 = 128 * (l >> 1) + 64 * (qt & 1) + 32 * (l & 1);
+        A8W8_LDS char* s = (A8W8_LDS char*)smem + (stage * STAGE_BYTES + (qt >= 2 ? BM * BK : 0) + row0 * BK) + wave_lds;
+        load_to_lds_16(qt < 2 ? rsrc_a : rsrc_b, s, ld_voff[qt * 4 + l], ld_ks * BK);
+    };
+    auto advance_ld = [&]() __attribute__((always_inline)) {
+        if (++ld_ks == nk) {
+            ld_ks = 0;
+            ld_item += gridDim.x;
+            point_loads_at(ld_item);
+        }
+    };
+
+    // Tiled MX scales: the exponents of a 64-row block for four K steps are 1 KiB of contiguous memory
+    // in the order the lanes read them ([pair of steps][lane (r16, g)][8 bytes]).  Wave w copies block w
+    // of the A tile and block w of the B tile of one scale group (four K steps) into LDS buffer `buf`.
+    auto issue_mx_group = [&](int item, int group, int buf) __attribute__((always_inline)) {
+        if constexpr (IS_MXT) {
+            item = min(item, pp.items - 1);
+            const int batch = item / tiles;
+            int tm, tn;
+            tile_of_block(item - batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+#pragma unroll
+            for (int side = 0; side < 2; ++side) {
+                const int rows = side ? p.n : p.m;
+                const uint8_t* base = side ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
+                                           : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
+                const int nblk = (rows + 63) >> 6;
+                const __amdgpu_buffer_rsrc_t rs = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, p.k));   // blocks past the edge read 0
+                const int voff = ((side ? tn * (BN / 64) : tm * (BM / 64)) + wave) * 1024 + lane * 16;
+                A8W8_LDS char* s = (A8W8_LDS char*)smem + GEMM_LDS_BYTES + buf * MX_GROUP_BYTES + side * 4096 + wave_lds;
+                load_to_lds_16(rs, s, voff, group * (nblk * 1024));
+            }
+        }
+    };
+    // Row/col scales of a tile: thread t fetches sfa[m0 + t] and sfb[n0 + t] (indices clamped) into LDS
+    // buffer `buf`, so that the epilogue waits on no global load.
+    auto issue_rowcol_scales = [&](int batch, int mm0, int nn0, int buf) __attribute__((always_inline)) {
+        if constexpr (MODE == MODE_ROWCOL) {
+#pragma unroll
+            for (int side = 0; side < 2; ++side) {
+                const int rows = side ? p.n : p.m;
+                const float* base = side ? (const float*)p.sfb + (long long)batch * p.sfb_batch
+                                         : (const float*)p.sfa + (long long)batch * p.sfa_batch;
+                const __amdgpu_buffer_rsrc_t rs = make_rsrc(base, (uint32_t)rows * 4u);
+                const int voff = min((side ? nn0 : mm0) + tid, rows - 1) * 4;
+                A8W8_LDS char* s = (A8W8_LDS char*)smem + GEMM_LDS_BYTES + buf * ROWCOL_SCALE_BYTES + side * (BM * 4) + wave * 256;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, s, 4, voff, 0, 0, 0);
+            }
+        }
+    };
+
+    // ---------------------------------------------------------------- compute side
+    // LDS rows as in the eight-wave kernel.  A: MFMA tile t, operand row r16 <- wave row 16t + r16.
+    // B: tile j, operand row 4g' + i <- wave row 32 (j/2) + 8g' + 4 (j%2) + i, so that a lane ends up
+    // with eight consecutive n.  For tile parity 1 the swizzle key differs from parity 0's in bit 2
+    // only, as do the two K halves h of a fragment: two address registers per operand serve all four.
+    auto swz_key = [](int row) __attribute__((always_inline)) { return ((row & 7) ^ (((row >> 3) & 3) << 1)) & 7; };
+    constexpr int A_PAR_BYTES = (PERM_A ? 4 : 16) * BK, B_PAR_BYTES = 4 * BK;
+    int rd_a[2], rd_b[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int row_b = 8 * (r16 >> 2) + (r16 & 3);
+        const int row_a = PERM_A ? row_b : r16;
+        rd_a[h] = (wave_m * 128 + row_a) * BK + ((((g + 4 * h) ^ swz_key(row_a)) & 7) << 4);
+        rd_b[h] = BM * BK + (wave_n * 128 + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
+    }
+    auto read_frag_at = [&](int stage, const int (&base)[2], int par, int byte_off) __attribute__((always_inline)) -> v8i {
+        const char* s = smem + stage * STAGE_BYTES + byte_off;
+        const v4i lo = *(const v4i*)(s + base[par]);
+        const v4i hi = *(const v4i*)(s + base[par ^ 1]);
+        return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    };
+    auto read_frag_a = [&](int stage, int t) __attribute__((always_inline)) -> v8i {
+        return read_frag_at(stage, rd_a, t & 1, (t >> 1) * (32 * BK) + (t & 1) * A_PAR_BYTES);
+    };
+    auto read_frag_b = [&](int stage, int j) __attribute__((always_inline)) -> v8i {
+        return read_frag_at(stage, rd_b, j & 1, (j >> 1) * (32 * BK) + (j & 1) * B_PAR_BYTES);
+    };
+
+    // MX scales in registers: per 64-row block of the wave's A rows (and B rows) one dword per tile
+    // pair, whose byte 2 (tile parity) + (step parity) belongs to the MFMA; they serve two K steps.
+    const int lane_rg = r16 * 4 + g;
+    const int rd_sfa = GEMM_LDS_BYTES + wave_m * 2048 + lane_rg * 8;
+    const int rd_sfb = GEMM_LDS_BYTES + 4096 + wave_n * 2048 + lane_rg * 8;
+    v2i sc_a[2], sc_b[2], sc_a_next[2], sc_b_next[2];
+    int sc_rd_off = 0;                              // LDS offset (buffer, pair) of the scales to fetch next
+    const int groups_per_tile = (nk + 3) >> 2;
+    int cur_gbase = 0;                              // running group count: picks the scale buffer
+
+    int cur_item = blockIdx.x;                     // the tile being multiplied
+    int cur_batch = 0, m0 = 0, n0 = 0;
+    auto point_compute_at = [&](int item) __attribute__((always_inline)) {
+        item = min(item, pp.items - 1);
+        cur_batch = item / tiles;
+        int tm, tn;
+        tile_of_block(item - cur_batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+        m0 = tm * BM;
+        n0 = tn * BN;
+    };
+
+    v4f acc[WIDE_T][WIDE_T];
+    auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < WIDE_T; ++i)
+#pragma unroll
+            for (int j = 0; j < WIDE_T; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    };
+
+    // ---------------------------------------------------------------- epilogue of one tile
+    int tile_seq = 0;                               // tiles this workgroup has started: picks the row/col scale buffer
+    auto store_tile = [&]() __attribute__((always_inline)) {
+        const float* sfa_f = (const float*)p.sfa + (long long)cur_batch * p.sfa_batch;
+        const float* sfb_f = (const float*)p.sfb + (long long)cur_batch * p.sfb_batch;
+        const int cm_base = m0 + wave_m * 128 + (PERM_A ? 8 * (r16 >> 2) + (r16 & 3) : r16);
+        auto cm_of = [&](int i) __attribute__((always_inline)) {          // C row of MFMA tile i
+            return cm_base + (PERM_A ? 32 * (i >> 1) + 4 * (i & 1) : 16 * i);
+        };
+        const int cn_base = n0 + wave_n * 128 + 8 * g;         // + 32 * (tile pair): eight consecutive n
+        float ts = 1.f;
+        if constexpr (MODE == MODE_TENSOR) ts = sfa_f[0] * sfb_f[0];
+        char* c_base = (char*)p.c + (long long)cur_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
+        const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 7) == 0 && (((uintptr_t)c_base) & 15) == 0)
+                                            : ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 15) == 0);
+        // row/col scales were staged in LDS when the tile began
+        const float* sc = (const float*)(smem + GEMM_LDS_BYTES + (tile_seq & 1) * ROWCOL_SCALE_BYTES);
+        float sa[WIDE_T];
+        if constexpr (MODE == MODE_ROWCOL) {
+#pragma unroll
+            for (int i = 0; i < WIDE_T; ++i) sa[i] = sc[cm_of(i) - m0];
+        }
+#pragma unroll
+        for (int jp = 0; jp < WIDE_T / 2; ++jp) {
+            const int cn = cn_base + 32 * jp;
+            float sb[8];
+            if constexpr (MODE == MODE_ROWCOL) {
+                const v4f lo = *(const v4f*)(sc + BM + (cn - n0)), hi = *(const v4f*)(sc + BM + (cn - n0) + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { sb[e] = lo[e]; sb[4 + e] = hi[e]; }
+            }
+#pragma unroll
+            for (int i = 0; i < WIDE_T; ++i) {
+                const int cm = cm_of(i);
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    v[e] = acc[i][2 * jp + (e >> 2)][e & 3];
+                    if constexpr (MODE == MODE_TENSOR) v[e] *= ts;
+                    if constexpr (MODE == MODE_ROWCOL) v[e] *= sb[e] * sa[i];
+                }
+                if (cm >= p.m) continue;
+                if constexpr (CDT == C_BF16) {
+                    unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
+                    if (vec_ok && cn + 7 < p.n) {
+                        v4i w;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+                        A8W8_STORE_C((v4i*)dst, w);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (cn + e < p.n) dst[e] = bf16_bits(v[e]);
+                    }
+                } else {
+                    float* dst = (float*)c_base + (long long)cm * p.ldc + cn;
+                    if (vec_ok && cn + 7 < p.n) {
+                        A8W8_STORE_C((v4f*)dst, (v4f{v[0], v[1], v[2], v[3]}));
+                        A8W8_STORE_C((v4f*)(dst + 4), (v4f{v[4], v[5], v[6], v[7]}));
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (cn + e < p.n) dst[e] = v[e];
+                    }
+                }
+            }
+        }
+    };
+
+    // ---------------------------------------------------------------- prologue
+    const int my_items = (pp.items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    if (my_items == 0) return;
+    point_loads_at(ld_item);
+    point_compute_at(cur_item);
+    issue_mx_group(cur_item, 0, 0);
+    // steps 0 and 1 in full
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+        for (int qt = 0; qt < 4; ++qt)
+#pragma unroll
+            for (int l = 0; l < 4; ++l) issue_one(st, qt, l);
+        advance_ld();
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    A8W8_RAW_BARRIER();
+    v8i fa[WIDE_T], fb[WIDE_T];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        fa[t] = read_frag_a(0, t);
+        fb[t] = read_frag_b(0, t);
+    }
+    if constexpr (IS_MXT) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            sc_a[u] = *(const v2i*)(smem + rd_sfa + u * 1024);
+            sc_b[u] = *(const v2i*)(smem + rd_sfb + u * 1024);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    A8W8_RAW_BARRIER();                              // the quarters just read may be overwritten from here on
+
+    // ---------------------------------------------------------------- one quadrant
+    // MFMAs of fa[IA..IA+3] x fb[JB..JB+3]; fragment set REF (0 aL, 1 aH, 2 bL, 3 bH) is re-read from
+    // stage RS; quarter LQ of the step at the load position is issued into stage LS.
+    auto quad = [&](auto IA, auto JB, auto REF, auto RS, auto LQ, auto LS, auto AOUTER, auto SPAR, auto SCREAD) __attribute__((always_inline)) {
+        constexpr bool a_outer = decltype(AOUTER)::value != 0;
+        constexpr int sp = decltype(SPAR)::value;            // the step's parity: scale byte inside a pair
+        constexpr bool SCR = decltype(SCREAD)::value != 0;   // this quadrant also fetches the next pair's scales
+        constexpr int ia = decltype(IA)::value, jb = decltype(JB)::value, ref = decltype(REF)::value;
+        constexpr int rs = decltype(RS)::value, lq = decltype(LQ)::value, ls = decltype(LS)::value;
+        // The MFMAs are written as assembly statements: the accumulators stay in the accumulator
+        // registers and are updated in place, and the statements keep their order, so the source
+        // order below is the schedule: two MFMAs, one LDS read; a load after every fourth MFMA.
+        v4i half[8];
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const int j = jb + (a_outer ? (t & 3) : (t >> 2)), i = ia + (a_outer ? (t >> 2) : (t & 3));
+            if constexpr (IS_MXT) {
+                mfma_mx_asm(acc[i][j], fb[j], fa[i], sc_b[j >> 2][(j >> 1) & 1], sc_a[i >> 2][(i >> 1) & 1], 2 * (j & 1) + sp, 2 * (i & 1) + sp);
+            } else {
+                asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fb[j]), "v"(fa[i]));
+            }
+            if (t & 1) {
+                const int r = t >> 1, f = (ref & 1) * 4 + (r >> 1), h = r & 1;     // half h of fragment f
+                const int par = f & 1;
+                const int* base = ref < 2 ? rd_a : rd_b;
+                const int off = (f >> 1) * (32 * BK) + par * (ref < 2 ? A_PAR_BYTES : B_PAR_BYTES);
+                half[r] = *(const v4i*)(smem + rs * STAGE_BYTES + off + base[par ^ h]);
+            }
+            if ((t & 3) == 2) issue_one(ls, lq, t >> 2);
+            if constexpr (IS_MXT && SCR) {
+                // the next pair of steps' scales, one 8-byte read after every fourth MFMA
+                if ((t & 3) == 0) {
+                    const int u = t >> 2;
+                    const v2i v = *(const v2i*)(smem + sc_rd_off + (u < 2 ? rd_sfa : rd_sfb) + (u & 1) * 1024);
+                    if (u < 2) sc_a_next[u] = v;
+                    else sc_b_next[u - 2] = v;
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const v4i lo = half[2 * t], hi = half[2 * t + 1];
+            const v8i v = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            if constexpr (ref < 2) fa[(ref & 1) * 4 + t] = v;
+            else fb[(ref & 1) * 4 + t] = v;
+        }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    using I4 = std::integral_constant<int, 4>;
+    auto handover = [&]() __attribute__((always_inline)) {
+        // every LDS read issued so far is complete, and all loads but the newest 16 have landed
+        __builtin_amdgcn_s_waitcnt(0x4070);
+        A8W8_RAW_BARRIER();
+    };
+
+    auto step = [&](auto parity) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity)::value;
+        // keeps the 32 LDS addresses of the loads from being computed once and parked in registers
+        asm volatile("" : "+s"(wave_lds));
+        using SP = std::integral_constant<int, P>;
+        using SN = std::integral_constant<int, P ^ 1>;
+        if constexpr (P == 0) {
+            quad(I0{}, I0{}, I3{}, SP{}, I0{}, SP{}, I0{}, SP{}, I0{});      // aL x bL | read bH of this step | load aL
+            quad(I0{}, I4{}, I1{}, SP{}, I2{}, SP{}, I0{}, SP{}, I0{});      // aL x bH | read aH of this step | load bL
+            handover();
+            quad(I4{}, I4{}, I0{}, SN{}, I3{}, SP{}, I1{}, SP{}, I0{});      // aH x bH | read aL of the next step | load bH
+            quad(I4{}, I0{}, I3{}, SN{}, I1{}, SP{}, I0{}, SP{}, I0{});      // aH x bL | read bH of the next step | load aH
+        } else {
+            quad(I0{}, I4{}, I2{}, SP{}, I0{}, SP{}, I0{}, SP{}, I0{});      // aL x bH | read bL of this step | load aL
+            quad(I0{}, I0{}, I1{}, SP{}, I3{}, SP{}, I0{}, SP{}, I0{});      // aL x bL | read aH of this step | load bH
+            handover();
+            quad(I4{}, I0{}, I0{}, SN{}, I2{}, SP{}, I1{}, SP{}, I0{});      // aH x bL | read aL of the next step | load bL
+            quad(I4{}, I4{}, I2{}, SN{}, I1{}, SP{}, I0{}, SP{}, I1{});      // aH x bH | read bL of the next step | load aH
+        }
+        advance_ld();
+        if constexpr (IS_MXT && P == 1) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                sc_a[u] = sc_a_next[u];
+                sc_b[u] = sc_b_next[u];
+            }
+        }
+        handover();
+    };
+
+    // The K loop of a tile is an even number of steps (checked by the host), so every tile starts on
+    // an even step; loads and fragment reads run on across the tile boundary.
+    for (int it = 0; it < my_items; ++it) {
+        zero_acc();
+        issue_rowcol_scales(cur_batch, m0, n0, tile_seq & 1);
+        asm volatile("s_nop 7" ::: "memory");           // accumulator writes -> first MFMA
+        for (int ks = 0; ks < nk; ks += 2) {
+            if constexpr (IS_MXT) {
+                // at the first step of a scale group: fetch the next group (of this tile or the first of
+                // the next tile) into the other buffer; its first pair is read three steps from here
+                if ((ks & 2) == 0) {
+                    const int g1 = (ks >> 2) + 1;
+                    if (g1 < groups_per_tile) issue_mx_group(cur_item, g1, (cur_gbase + g1) & 1);
+                    else issue_mx_group(cur_item + (int)gridDim.x, 0, (cur_gbase + groups_per_tile) & 1);
+                }
+                // where the pair after this one lives
+                const int npair = (ks >> 1) + 1;
+                const int nbuf = ks + 2 < nk ? (cur_gbase + (npair >> 1)) & 1 : (cur_gbase + groups_per_tile) & 1;
+                sc_rd_off = nbuf * MX_GROUP_BYTES + (ks + 2 < nk ? (npair & 1) * 512 : 0);
+            }
+            step(std::integral_constant<int, 0>{});
+            step(std::integral_constant<int, 1>{});
+        }
+        cur_gbase += groups_per_tile;
+        // the compiler does not see the MFMAs: keep the required distance between the last of them
+        // and the first read of an accumulator
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        store_tile();
+        ++tile_seq;
+        cur_item += gridDim.x;
+        point_compute_at(cur_item);
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // no direct-to-LDS load may outlive the workgroup's LDS allocation
+}
+
+}  // namespace a8w8

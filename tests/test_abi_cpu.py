@@ -76,7 +76,10 @@ def test_flatmm_preconditions():
 def test_kernel_selection():
     assert g.kernel_name(_ok_args()) == "gemm_a8w8_persist"
     assert g.kernel_name(_ok_args(mode=g.MX)) == "gemm_a8w8_persist"
-    assert g.kernel_name(_ok_args(mode=g.ROWCOL)) == "gemm_a8w8_persist"
+    # per-tensor, row/col and tiled-MX scales with an even number of K steps: the four-wave kernel
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL)) == "gemm_a8w8_wide"
+    assert g.kernel_name(_ok_args(mode=g.TENSOR, k=1024)) == "gemm_a8w8_wide"
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=384)) == "gemm_a8w8_persist"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=128)) == "gemm_a8w8_tile256"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=200)) == "gemm_a8w8_general"
     a = _ok_args(mode=g.ROWCOL)
@@ -85,7 +88,7 @@ def test_kernel_selection():
 
 
 def test_tiled_mx_mode_selection_and_reorder_preconditions():
-    assert g.kernel_name(_ok_args(mode=g.MX_TILED)) == "gemm_a8w8_persist"
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED)) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=384)) == "gemm_a8w8_general"      # odd number of K steps
     assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=128)) == "gemm_a8w8_general"
     a = _ok_args(mode=g.MX_TILED, k=48)

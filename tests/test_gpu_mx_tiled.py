@@ -58,7 +58,7 @@ def test_gemm_with_tiled_scales(orc, shape):
     m, n, k = shape
     a, b, ea, eb = datagen.mx(m, n, k, seed=1500 + m + k)
     args = g.raw_gemm_args(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, m, n, k, g.MX_TILED)
-    assert g.kernel_name(args) == "gemm_a8w8_persist"
+    assert g.kernel_name(args) == "gemm_a8w8_wide"
     want = orc.gemm_ref(a, b, ea, eb, orc.MX)
     exact, mag = exact64(orc, a, b, ea, eb, g.MX)
     assert_close(_tiled_gemm(a, b, ea, eb), want, f"mx tiled {shape}", exact=exact, mag=mag)
