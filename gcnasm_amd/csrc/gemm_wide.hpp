@@ -33,24 +33,47 @@ constexpr int wide_lds_bytes(int mode)
     return GEMM_LDS_BYTES + (mode == MODE_MXT ? 2 * MX_GROUP_BYTES : mode == MODE_ROWCOL ? 2 * ROWCOL_SCALE_BYTES : 0);
 }
 
-// Scaled MFMA on accumulator registers, in place: c += (a . b) with byte OA of sa and byte OB of sb
-// as the E8M0 scales of the lane's 32-element K block (the selectors are instruction modifiers).
-A8W8_DEV void mfma_mx_asm(v4f& c, const v8i& a, const v8i& b, int sa, int sb, int oa, int ob)
+// The 64 accumulator tiles of a wave live in accumulator registers a[0:255], tile (i, j) in
+// a[4 (8i + j) : +3].  They are named in assembly statements only and never appear as variables: the
+// compiler allocates nothing there (its own registers stay below 256, which the build checks), so no
+// copy, spill or re-materialisation can come between two MFMAs of one tile.  The statements keep
+// their order; the compiler does not see the MFMAs' latency, so the code that reads an accumulator
+// makes sure that enough instructions separate it from the last MFMA into that tile.
+template <int N, class F, int... I>
+A8W8_DEV void static_for_impl(F&& f, std::integer_sequence<int, I...>)
 {
-#define A8W8_MX_CASE(OA, OB, ALO, AHI, BLO, BHI)                                                               \
-    case OA * 4 + OB:                                                                                            \
-        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[" #ALO "," #BLO         \
-                     ",0] op_sel_hi:[" #AHI "," #BHI ",0]"                                                      \
-                     : "+a"(c)                                                                                   \
-                     : "v"(a), "v"(b), "v"(sa), "v"(sb));                                                      \
-        break;
-    switch (oa * 4 + ob) {
-        A8W8_MX_CASE(0, 0, 0, 0, 0, 0) A8W8_MX_CASE(0, 1, 0, 0, 1, 0) A8W8_MX_CASE(0, 2, 0, 0, 0, 1) A8W8_MX_CASE(0, 3, 0, 0, 1, 1)
-        A8W8_MX_CASE(1, 0, 1, 0, 0, 0) A8W8_MX_CASE(1, 1, 1, 0, 1, 0) A8W8_MX_CASE(1, 2, 1, 0, 0, 1) A8W8_MX_CASE(1, 3, 1, 0, 1, 1)
-        A8W8_MX_CASE(2, 0, 0, 1, 0, 0) A8W8_MX_CASE(2, 1, 0, 1, 1, 0) A8W8_MX_CASE(2, 2, 0, 1, 0, 1) A8W8_MX_CASE(2, 3, 0, 1, 1, 1)
-        A8W8_MX_CASE(3, 0, 1, 1, 0, 0) A8W8_MX_CASE(3, 1, 1, 1, 1, 0) A8W8_MX_CASE(3, 2, 1, 1, 0, 1) A8W8_MX_CASE(3, 3, 1, 1, 1, 1)
-    }
-#undef A8W8_MX_CASE
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+A8W8_DEV void static_for(F&& f)
+{
+    static_for_impl<N>(f, std::make_integer_sequence<int, N>{});
+}
+
+// tile LO/4 += a . b, or = a . b when ZC (the tile's first K step)
+template <int LO, bool ZC>
+A8W8_DEV void mfma_acc(const v8i& a, const v8i& b)
+{
+    if constexpr (ZC) asm volatile("v_mfma_f32_16x16x128_f8f6f4 a[%2:%3], %0, %1, 0" ::"v"(a), "v"(b), "n"(LO), "n"(LO + 3));
+    else asm volatile("v_mfma_f32_16x16x128_f8f6f4 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(a), "v"(b), "n"(LO), "n"(LO + 3));
+}
+// the same with E8M0 block scales: byte OA of sa scales a's K block of the lane, byte OB of sb b's
+template <int LO, bool ZC, int OA, int OB>
+A8W8_DEV void mfma_acc_mx(const v8i& a, const v8i& b, int sa, int sb)
+{
+    if constexpr (ZC)
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, 0, %2, %3 op_sel:[%6,%7,0] op_sel_hi:[%8,%9,0]" ::"v"(a),
+                     "v"(b), "v"(sa), "v"(sb), "n"(LO), "n"(LO + 3), "n"(OA & 1), "n"(OB & 1), "n"(OA >> 1), "n"(OB >> 1));
+    else
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel:[%6,%7,0] op_sel_hi:[%8,%9,0]" ::"v"(a),
+                     "v"(b), "v"(sa), "v"(sb), "n"(LO), "n"(LO + 3), "n"(OA & 1), "n"(OB & 1), "n"(OA >> 1), "n"(OB >> 1));
+}
+template <int IDX>
+A8W8_DEV float acc_read()
+{
+    float x;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(IDX));
+    return x;
 }
 
 template <int MODE, int CDT>
@@ -62,6 +85,8 @@ gemm_a8w8_wide(PersistParams pp)
     // tiled MX scales are laid out for A tiles whose rows are dealt like the B tiles' rows
     constexpr bool PERM_A = IS_MXT;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
+    // all 256 accumulator registers are in use (this is what sizes the wave's register allocation)
+    asm volatile("" ::: "a0", "a255");
     const GemmParams& p = pp.g;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -71,6 +96,13 @@ gemm_a8w8_wide(PersistParams pp)
     const int nk = p.k / BK;                       // >= 2 (checked by the host)
     const int tiles = p.tiles_m * p.tiles_n;
 
+    // LDS: [A of stage 0][A of stage 1][B of stage 0][B of stage 1], 32 KiB each.  A lane's read
+    // addresses are its row and K-piece offset inside an operand (below 32 KiB) plus the stage and the
+    // fragment's tile offset; keeping both stages of an operand within 64 KiB makes the latter two an
+    // instruction immediate, so two address registers per operand serve every read.
+    constexpr int HALF_STAGE = BM * BK;             // one operand of one stage
+    constexpr int OPERAND_BYTES = 2 * HALF_STAGE;   // both stages of one operand
+
     // ---------------------------------------------------------------- load side
     int ld_item = blockIdx.x, ld_ks = 0;           // the step whose quarters are being issued
     __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b;
@@ -79,9 +111,11 @@ gemm_a8w8_wide(PersistParams pp)
     // holds K piece slot ^ key(row), key(row) = (row & 7) ^ (((row >> 3) & 3) << 1), and bits 3-4 of
     // the tile row equal the wave number for every load this wave issues
     const int ld_piece16 = ((lane & 7) ^ (((lane >> 3) ^ (wave << 1)) & 7)) * 16;
-    // Lane offsets of the sixteen loads of a step: they change only with the tile, and this kernel
-    // has registers to keep them, so a load costs one scalar add (its LDS address) and itself.
-    int ld_voff[16];
+    // A load's address is lane offset + scalar offset: the lane part (two row groups of the tile per
+    // operand) changes only with the tile, the scalar part is the K step plus a multiple of the row
+    // stride.  Rows past the end of a matrix are past the end of its descriptor: they read
+    // as zero and only reach accumulators that are never stored.
+    int ld_voff_a[2] = {0, 0}, ld_voff_b[2] = {0, 0};   // rows 8w.. and 128 + 8w.. of the tile
     auto point_loads_at = [&](int item) __attribute__((always_inline)) {
         item = min(item, pp.items - 1);            // past the end: keep loading valid data nobody reads
         const int batch = item / tiles;
@@ -90,13 +124,10 @@ gemm_a8w8_wide(PersistParams pp)
         rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
         rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, (uint32_t)(p.n - 1) * p.ldb + p.k);
 #pragma unroll
-        for (int qt = 0; qt < 4; ++qt)
-#pragma unroll
-            for (int l = 0; l < 4; ++l) {
-                const int row = 128 * (l >> 1) + 64 * (qt & 1) + 32 * (l & 1) + ld_row;
-                ld_voff[qt * 4 + l] = qt < 2 ? __mul24(min(tm * BM + row, p.m - 1), p.lda) + ld_piece16
-                                             : __mul24(min(tn * BN + row, p.n - 1), p.ldb) + ld_piece16;
-            }
+        for (int h = 0; h < 2; ++h) {
+            ld_voff_a[h] = __mul24(tm * BM + 128 * h + ld_row, p.lda) + ld_piece16;
+            ld_voff_b[h] = __mul24(tn * BN + 128 * h + ld_row, p.ldb) + ld_piece16;
+        }
     };
     // Load l (0..3) of quarter qt (0 aL, 1 aH, 2 bL, 3 bH) of the step at the load position.  A quarter
     // is tile rows [64h, 64h + 64) and [128 + 64h, 192 + 64h) of one operand (h = qt & 1): the L or H
@@ -104,8 +135,11 @@ gemm_a8w8_wide(PersistParams pp)
     int wave_lds = wave * 1024;
     auto issue_one = [&](int stage, int qt, int l) __attribute__((always_inline)) {
         const int row0 = 128 * (l >> 1) + 64 * (qt & 1) + 32 * (l & 1);
-        A8W8_LDS char* s = (A8W8_LDS char*)smem + (stage * STAGE_BYTES + (qt >= 2 ? BM * BK : 0) + row0 * BK) + wave_lds;
-        load_to_lds_16(qt < 2 ? rsrc_a : rsrc_b, s, ld_voff[qt * 4 + l], ld_ks * BK);
+        A8W8_LDS char* s = (A8W8_LDS char*)smem + ((qt >= 2 ? OPERAND_BYTES : 0) + stage * HALF_STAGE + row0 * BK) + wave_lds;
+        // four scalar offsets per operand and step (K step + 0, 32, 64 or 96 rows), each used twice
+        const int rows = 64 * (qt & 1) + 32 * (l & 1);
+        if (qt < 2) load_to_lds_16(rsrc_a, s, ld_voff_a[l >> 1], ld_ks * BK + rows * p.lda);
+        else load_to_lds_16(rsrc_b, s, ld_voff_b[l >> 1], ld_ks * BK + rows * p.ldb);
     };
     auto advance_ld = [&]() __attribute__((always_inline)) {
         if (++ld_ks == nk) {
@@ -167,10 +201,10 @@ gemm_a8w8_wide(PersistParams pp)
         const int row_b = 8 * (r16 >> 2) + (r16 & 3);
         const int row_a = PERM_A ? row_b : r16;
         rd_a[h] = (wave_m * 128 + row_a) * BK + ((((g + 4 * h) ^ swz_key(row_a)) & 7) << 4);
-        rd_b[h] = BM * BK + (wave_n * 128 + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
+        rd_b[h] = OPERAND_BYTES + (wave_n * 128 + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
     }
     auto read_frag_at = [&](int stage, const int (&base)[2], int par, int byte_off) __attribute__((always_inline)) -> v8i {
-        const char* s = smem + stage * STAGE_BYTES + byte_off;
+        const char* s = smem + stage * HALF_STAGE + byte_off;
         const v4i lo = *(const v4i*)(s + base[par]);
         const v4i hi = *(const v4i*)(s + base[par ^ 1]);
         return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
@@ -203,83 +237,81 @@ gemm_a8w8_wide(PersistParams pp)
         n0 = tn * BN;
     };
 
-    v4f acc[WIDE_T][WIDE_T];
-    auto zero_acc = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < WIDE_T; ++i)
-#pragma unroll
-            for (int j = 0; j < WIDE_T; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
-    };
-
-    // ---------------------------------------------------------------- epilogue of one tile
+    // ---------------------------------------------------------------- epilogue, in pieces
+    // The tile whose accumulators are being written out (the current one until its last K step has
+    // begun, then it stays while the next tile's first step runs).
+    int ep_batch = 0, ep_m0 = 0, ep_n0 = 0, ep_seq = 0;
     int tile_seq = 0;                               // tiles this workgroup has started: picks the row/col scale buffer
-    auto store_tile = [&]() __attribute__((always_inline)) {
-        const float* sfa_f = (const float*)p.sfa + (long long)cur_batch * p.sfa_batch;
-        const float* sfb_f = (const float*)p.sfb + (long long)cur_batch * p.sfb_batch;
-        const int cm_base = m0 + wave_m * 128 + (PERM_A ? 8 * (r16 >> 2) + (r16 & 3) : r16);
-        auto cm_of = [&](int i) __attribute__((always_inline)) {          // C row of MFMA tile i
-            return cm_base + (PERM_A ? 32 * (i >> 1) + 4 * (i & 1) : 16 * i);
-        };
-        const int cn_base = n0 + wave_n * 128 + 8 * g;         // + 32 * (tile pair): eight consecutive n
-        float ts = 1.f;
-        if constexpr (MODE == MODE_TENSOR) ts = sfa_f[0] * sfb_f[0];
-        char* c_base = (char*)p.c + (long long)cur_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
-        const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 7) == 0 && (((uintptr_t)c_base) & 15) == 0)
-                                            : ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 15) == 0);
-        // row/col scales were staged in LDS when the tile began
-        const float* sc = (const float*)(smem + GEMM_LDS_BYTES + (tile_seq & 1) * ROWCOL_SCALE_BYTES);
-        float sa[WIDE_T];
-        if constexpr (MODE == MODE_ROWCOL) {
+    float ep_ts = 1.f;
+    bool ep_vec_ok = false;                         // C rows of this batch entry take 16-byte stores
+    // One piece = the lane's eight consecutive n of MFMA tile row i and tile pair jp: scale, convert,
+    // one 16-byte store (bf16) or two (fp32).
+    auto store_piece = [&](auto I, auto JP, bool checked) __attribute__((always_inline)) {
+        constexpr int i = decltype(I)::value, jp = decltype(JP)::value;
+        const int cm = ep_m0 + wave_m * 128 + (PERM_A ? 8 * (r16 >> 2) + (r16 & 3) + 32 * (i >> 1) + 4 * (i & 1) : r16 + 16 * i);
+        const int cn = ep_n0 + wave_n * 128 + 8 * g + 32 * jp;
+        char* c_base = (char*)p.c + (long long)ep_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
+        float v[8];
+        static_for<8>([&](auto E) {
+            constexpr int e = decltype(E)::value;
+            v[e] = acc_read<(i * 8 + 2 * jp + (e >> 2)) * 4 + (e & 3)>();
+        });
+        if constexpr (MODE == MODE_TENSOR) {
 #pragma unroll
-            for (int i = 0; i < WIDE_T; ++i) sa[i] = sc[cm_of(i) - m0];
+            for (int e = 0; e < 8; ++e) v[e] *= ep_ts;
         }
+        if constexpr (MODE == MODE_ROWCOL) {
+            // row/col scales were staged in LDS when the tile began
+            const float* sc = (const float*)(smem + GEMM_LDS_BYTES + (ep_seq & 1) * ROWCOL_SCALE_BYTES);
+            const float sa = sc[cm - ep_m0];
+            const v4f lo = *(const v4f*)(sc + BM + (cn - ep_n0)), hi = *(const v4f*)(sc + BM + (cn - ep_n0) + 4);
 #pragma unroll
-        for (int jp = 0; jp < WIDE_T / 2; ++jp) {
-            const int cn = cn_base + 32 * jp;
-            float sb[8];
-            if constexpr (MODE == MODE_ROWCOL) {
-                const v4f lo = *(const v4f*)(sc + BM + (cn - n0)), hi = *(const v4f*)(sc + BM + (cn - n0) + 4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) { sb[e] = lo[e]; sb[4 + e] = hi[e]; }
+            for (int e = 0; e < 4; ++e) {
+                v[e] *= lo[e] * sa;
+                v[4 + e] *= hi[e] * sa;
             }
+        }
+        if (checked && cm >= p.m) return;
+        const bool vec = !checked || (ep_vec_ok && cn + 7 < p.n);
+        if constexpr (CDT == C_BF16) {
+            unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
+            if (vec) {
+                v4i w;
 #pragma unroll
-            for (int i = 0; i < WIDE_T; ++i) {
-                const int cm = cm_of(i);
-                float v[8];
+                for (int e = 0; e < 4; ++e) w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+                A8W8_STORE_C((v4i*)dst, w);
+            } else {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    v[e] = acc[i][2 * jp + (e >> 2)][e & 3];
-                    if constexpr (MODE == MODE_TENSOR) v[e] *= ts;
-                    if constexpr (MODE == MODE_ROWCOL) v[e] *= sb[e] * sa[i];
-                }
-                if (cm >= p.m) continue;
-                if constexpr (CDT == C_BF16) {
-                    unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
-                    if (vec_ok && cn + 7 < p.n) {
-                        v4i w;
+                for (int e = 0; e < 8; ++e)
+                    if (cn + e < p.n) dst[e] = bf16_bits(v[e]);
+            }
+        } else {
+            float* dst = (float*)c_base + (long long)cm * p.ldc + cn;
+            if (vec) {
+                A8W8_STORE_C((v4f*)dst, (v4f{v[0], v[1], v[2], v[3]}));
+                A8W8_STORE_C((v4f*)(dst + 4), (v4f{v[4], v[5], v[6], v[7]}));
+            } else {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
-                        A8W8_STORE_C((v4i*)dst, w);
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (cn + e < p.n) dst[e] = bf16_bits(v[e]);
-                    }
-                } else {
-                    float* dst = (float*)c_base + (long long)cm * p.ldc + cn;
-                    if (vec_ok && cn + 7 < p.n) {
-                        A8W8_STORE_C((v4f*)dst, (v4f{v[0], v[1], v[2], v[3]}));
-                        A8W8_STORE_C((v4f*)(dst + 4), (v4f{v[4], v[5], v[6], v[7]}));
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (cn + e < p.n) dst[e] = v[e];
-                    }
-                }
+                for (int e = 0; e < 8; ++e)
+                    if (cn + e < p.n) dst[e] = v[e];
             }
         }
     };
+    // Piece g (0..7) of accumulator quadrant eq (0 aL x bL, 1 aL x bH, 2 aH x bL, 3 aH x bH), in the
+    // order in which the quadrant's MFMAs finished (B-major, or A-major when a_outer): the piece that
+    // holds the last MFMA's tile comes last, at least twelve MFMAs after it was issued.
+    auto flush_piece = [&](auto EQ, auto GQ, auto AO) __attribute__((always_inline)) {
+        constexpr int eq = decltype(EQ)::value, gq = decltype(GQ)::value;
+        constexpr bool a_outer = decltype(AO)::value != 0;
+        constexpr int i = (eq >> 1) * 4 + (a_outer ? (gq >> 1) : (gq & 3));
+        constexpr int jp = (eq & 1) * 2 + (a_outer ? (gq & 1) : (gq >> 2));
+        store_piece(std::integral_constant<int, i>{}, std::integral_constant<int, jp>{}, false);
+    };
+    // the whole tile with every bounds and alignment check, for tiles the pieces cannot serve
+    auto store_tile_checked = [&]() __attribute__((always_inline)) {
+        static_for<WIDE_T / 2>([&](auto JP) { static_for<WIDE_T>([&](auto I) { store_piece(I, JP, true); }); });
+    };
+    constexpr int STORES_PER_PIECE = CDT == C_BF16 ? 1 : 2;
 
     // ---------------------------------------------------------------- prologue
     const int my_items = (pp.items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
@@ -316,43 +348,59 @@ gemm_a8w8_wide(PersistParams pp)
 
     // ---------------------------------------------------------------- one quadrant
     // MFMAs of fa[IA..IA+3] x fb[JB..JB+3]; fragment set REF (0 aL, 1 aH, 2 bL, 3 bH) is re-read from
-    // stage RS; quarter LQ of the step at the load position is issued into stage LS.
-    auto quad = [&](auto IA, auto JB, auto REF, auto RS, auto LQ, auto LS, auto AOUTER, auto SPAR, auto SCREAD) __attribute__((always_inline)) {
+    // stage RS; quarter LQ of the step at the load position is issued into stage LS.  ZC: the tile's
+    // first step, the MFMAs take zero instead of the accumulator.  EQ >= 0: the previous owner of
+    // accumulator quadrant EQ is written out meanwhile, one piece per two MFMAs (EQA: that quadrant's
+    // MFMAs ran A-major).
+    bool have_prev = false;                         // a quadrant of the tile before is still to be written out
+    auto quad = [&](auto IA, auto JB, auto REF, auto RS, auto LQ, auto LS, auto AOUTER, auto SPAR, auto SCREAD, auto ZC, auto EQ,
+                    auto EQA) __attribute__((always_inline)) {
         constexpr bool a_outer = decltype(AOUTER)::value != 0;
         constexpr int sp = decltype(SPAR)::value;            // the step's parity: scale byte inside a pair
         constexpr bool SCR = decltype(SCREAD)::value != 0;   // this quadrant also fetches the next pair's scales
+        constexpr bool zc = decltype(ZC)::value != 0;
+        constexpr int eq = decltype(EQ)::value - 1;          // -1: nothing to write out
+        constexpr bool eqa = decltype(EQA)::value != 0;
         constexpr int ia = decltype(IA)::value, jb = decltype(JB)::value, ref = decltype(REF)::value;
         constexpr int rs = decltype(RS)::value, lq = decltype(LQ)::value, ls = decltype(LS)::value;
         // The MFMAs are written as assembly statements: the accumulators stay in the accumulator
         // registers and are updated in place, and the statements keep their order, so the source
         // order below is the schedule: two MFMAs, one LDS read; a load after every fourth MFMA.
         v4i half[8];
-#pragma unroll
-        for (int t = 0; t < 16; ++t) {
-            const int j = jb + (a_outer ? (t & 3) : (t >> 2)), i = ia + (a_outer ? (t >> 2) : (t & 3));
-            if constexpr (IS_MXT) {
-                mfma_mx_asm(acc[i][j], fb[j], fa[i], sc_b[j >> 2][(j >> 1) & 1], sc_a[i >> 2][(i >> 1) & 1], 2 * (j & 1) + sp, 2 * (i & 1) + sp);
-            } else {
-                asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fb[j]), "v"(fa[i]));
-            }
-            if (t & 1) {
-                const int r = t >> 1, f = (ref & 1) * 4 + (r >> 1), h = r & 1;     // half h of fragment f
-                const int par = f & 1;
+        static_for<16>([&](auto TT) {
+            constexpr int t = decltype(TT)::value;
+            constexpr int j = jb + (a_outer ? (t & 3) : (t >> 2)), i = ia + (a_outer ? (t >> 2) : (t & 3));
+            constexpr int lo = (i * 8 + j) * 4;
+            if constexpr (IS_MXT)
+                mfma_acc_mx<lo, zc, 2 * (j & 1) + sp, 2 * (i & 1) + sp>(fb[j], fa[i], sc_b[j >> 2][(j >> 1) & 1], sc_a[i >> 2][(i >> 1) & 1]);
+            else
+                mfma_acc<lo, zc>(fb[j], fa[i]);
+            if constexpr ((t & 1) != 0) {
+                constexpr int r = t >> 1, f = (ref & 1) * 4 + (r >> 1), h = r & 1;     // half h of fragment f
+                constexpr int par = f & 1;
                 const int* base = ref < 2 ? rd_a : rd_b;
-                const int off = (f >> 1) * (32 * BK) + par * (ref < 2 ? A_PAR_BYTES : B_PAR_BYTES);
-                half[r] = *(const v4i*)(smem + rs * STAGE_BYTES + off + base[par ^ h]);
+                constexpr int off = (f >> 1) * (32 * BK) + par * (ref < 2 ? A_PAR_BYTES : B_PAR_BYTES);
+                half[r] = *(const v4i*)(smem + (rs * HALF_STAGE + off) + base[par ^ h]);
             }
-            if ((t & 3) == 2) issue_one(ls, lq, t >> 2);
-            if constexpr (IS_MXT && SCR) {
+            if constexpr ((t & 3) == 2) issue_one(ls, lq, t >> 2);
+            if constexpr (IS_MXT && SCR && (t & 3) == 0) {
                 // the next pair of steps' scales, one 8-byte read after every fourth MFMA
-                if ((t & 3) == 0) {
-                    const int u = t >> 2;
-                    const v2i v = *(const v2i*)(smem + sc_rd_off + (u < 2 ? rd_sfa : rd_sfb) + (u & 1) * 1024);
-                    if (u < 2) sc_a_next[u] = v;
-                    else sc_b_next[u - 2] = v;
+                constexpr int u = t >> 2;
+                const v2i v = *(const v2i*)(smem + sc_rd_off + (u < 2 ? rd_sfa : rd_sfb) + (u & 1) * 1024);
+                if constexpr (u < 2) sc_a_next[u] = v;
+                else sc_b_next[u - 2] = v;
+            }
+            if constexpr (eq >= 0 && (t & 1) != 0) {
+                using EQT = std::integral_constant<int, eq < 0 ? 0 : eq>;
+                using GQT = std::integral_constant<int, (t >> 1)>;
+                using AOT = std::integral_constant<int, eqa ? 1 : 0>;
+                if constexpr (zc) {
+                    if (have_prev) flush_piece(EQT{}, GQT{}, AOT{});
+                } else {
+                    flush_piece(EQT{}, GQT{}, AOT{});
                 }
             }
-        }
+        });
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const v4i lo = half[2 * t], hi = half[2 * t + 1];
@@ -366,48 +414,84 @@ gemm_a8w8_wide(PersistParams pp)
     using I2 = std::integral_constant<int, 2>;
     using I3 = std::integral_constant<int, 3>;
     using I4 = std::integral_constant<int, 4>;
-    auto handover = [&]() __attribute__((always_inline)) {
-        // every LDS read issued so far is complete, and all loads but the newest 16 have landed
-        __builtin_amdgcn_s_waitcnt(0x4070);
+    // Every LDS read issued so far is complete, and all memory operations but the newest N have
+    // finished: N = the 16 loads of the last four quadrants plus the stores issued among them, so that
+    // what has finished is exactly the two quarters the next two quadrants read.
+    auto handover = [&](auto STORES) __attribute__((always_inline)) {
+        constexpr int want = 16 + decltype(STORES)::value * STORES_PER_PIECE;
+        constexpr int n = want < 63 ? want : 63;             // a 6-bit counter; fewer is only stricter
+        __builtin_amdgcn_s_waitcnt(((n & 15) | ((n >> 4) << 14)) | 0x0070);
         A8W8_RAW_BARRIER();
     };
+    using S0 = std::integral_constant<int, 0>;
+    using S8 = std::integral_constant<int, 8>;
+    using S24 = std::integral_constant<int, 24>;
 
-    auto step = [&](auto parity) __attribute__((always_inline)) {
+    // A K step.  FIRST: the tile's first step (even): accumulators start from zero, and the previous
+    // tile's last quadrant is written out behind the first 16 MFMAs.  LAST: the tile's last step
+    // (odd): each accumulator quadrant is written out behind the MFMAs of the quadrant after it.
+    auto step = [&](auto parity, auto first, auto last) __attribute__((always_inline)) {
         constexpr int P = decltype(parity)::value;
+        constexpr bool FIRST = decltype(first)::value != 0, LAST = decltype(last)::value != 0;
+        static_assert(!(FIRST && P == 1) && !(LAST && P == 0), "tiles start on even steps and end on odd ones");
         // keeps the 32 LDS addresses of the loads from being computed once and parked in registers
-        asm volatile("" : "+s"(wave_lds));
+        // (always wave * 1024, but tied to a value that changes with the step)
+        wave_lds = wave * 1024 + (ld_ks >> 30);
         using SP = std::integral_constant<int, P>;
         using SN = std::integral_constant<int, P ^ 1>;
+        using Z = std::integral_constant<int, FIRST ? 1 : 0>;
         if constexpr (P == 0) {
-            quad(I0{}, I0{}, I3{}, SP{}, I0{}, SP{}, I0{}, SP{}, I0{});      // aL x bL | read bH of this step | load aL
-            quad(I0{}, I4{}, I1{}, SP{}, I2{}, SP{}, I0{}, SP{}, I0{});      // aL x bH | read aH of this step | load bL
-            handover();
-            quad(I4{}, I4{}, I0{}, SN{}, I3{}, SP{}, I1{}, SP{}, I0{});      // aH x bH | read aL of the next step | load bH
-            quad(I4{}, I0{}, I3{}, SN{}, I1{}, SP{}, I0{}, SP{}, I0{});      // aH x bL | read bH of the next step | load aH
-        } else {
-            quad(I0{}, I4{}, I2{}, SP{}, I0{}, SP{}, I0{}, SP{}, I0{});      // aL x bH | read bL of this step | load aL
-            quad(I0{}, I0{}, I1{}, SP{}, I3{}, SP{}, I0{}, SP{}, I0{});      // aL x bL | read aH of this step | load bH
-            handover();
-            quad(I4{}, I0{}, I0{}, SN{}, I2{}, SP{}, I1{}, SP{}, I0{});      // aH x bL | read aL of the next step | load bL
-            quad(I4{}, I4{}, I2{}, SN{}, I1{}, SP{}, I0{}, SP{}, I1{});      // aH x bH | read bL of the next step | load aH
-        }
-        advance_ld();
-        if constexpr (IS_MXT && P == 1) {
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                sc_a[u] = sc_a_next[u];
-                sc_b[u] = sc_b_next[u];
+            // aL x bL | read bH of this step | load aL            (| write out aH x bH of the previous tile)
+            quad(I0{}, I0{}, I3{}, SP{}, I0{}, SP{}, I0{}, SP{}, I0{}, Z{}, std::integral_constant<int, FIRST ? 4 : 0>{}, I0{});
+            // aL x bH | read aH of this step | load bL
+            quad(I0{}, I4{}, I1{}, SP{}, I2{}, SP{}, I0{}, SP{}, I0{}, Z{}, I0{}, I0{});
+            if constexpr (FIRST) {
+                if (have_prev) handover(S24{});
+                else handover(S0{});
+            } else {
+                handover(S0{});
             }
+            // aH x bH | read aL of the next step | load bH
+            quad(I4{}, I4{}, I0{}, SN{}, I3{}, SP{}, I1{}, SP{}, I0{}, Z{}, I0{}, I0{});
+            // aH x bL | read bH of the next step | load aH
+            quad(I4{}, I0{}, I3{}, SN{}, I1{}, SP{}, I0{}, SP{}, I0{}, Z{}, I0{}, I0{});
+            advance_ld();
+            if constexpr (FIRST) {
+                if (have_prev) handover(S8{});
+                else handover(S0{});
+            } else {
+                handover(S0{});
+            }
+        } else {
+            // aL x bH | read bL of this step | load aL
+            quad(I0{}, I4{}, I2{}, SP{}, I0{}, SP{}, I0{}, SP{}, I0{}, I0{}, I0{}, I0{});
+            // aL x bL | read aH of this step | load bH             (| write out aL x bH)
+            quad(I0{}, I0{}, I1{}, SP{}, I3{}, SP{}, I0{}, SP{}, I0{}, I0{}, std::integral_constant<int, LAST ? 2 : 0>{}, I0{});
+            if constexpr (LAST) handover(S8{});
+            else handover(S0{});
+            // aH x bL | read aL of the next step | load bL         (| write out aL x bL)
+            quad(I4{}, I0{}, I0{}, SN{}, I2{}, SP{}, I1{}, SP{}, I0{}, I0{}, std::integral_constant<int, LAST ? 1 : 0>{}, I0{});
+            // aH x bH | read bL of the next step | load aH         (| write out aH x bL, whose MFMAs ran A-major)
+            quad(I4{}, I4{}, I2{}, SN{}, I1{}, SP{}, I0{}, SP{}, I1{}, I0{}, std::integral_constant<int, LAST ? 3 : 0>{}, I1{});
+            advance_ld();
+            if constexpr (IS_MXT) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    sc_a[u] = sc_a_next[u];
+                    sc_b[u] = sc_b_next[u];
+                }
+            }
+            if constexpr (LAST) handover(S24{});
+            else handover(S0{});
         }
-        handover();
     };
+    using F = std::integral_constant<int, 0>;
+    using T = std::integral_constant<int, 1>;
 
     // The K loop of a tile is an even number of steps (checked by the host), so every tile starts on
     // an even step; loads and fragment reads run on across the tile boundary.
     for (int it = 0; it < my_items; ++it) {
-        zero_acc();
         issue_rowcol_scales(cur_batch, m0, n0, tile_seq & 1);
-        asm volatile("s_nop 7" ::: "memory");           // accumulator writes -> first MFMA
         for (int ks = 0; ks < nk; ks += 2) {
             if constexpr (IS_MXT) {
                 // at the first step of a scale group: fetch the next group (of this tile or the first of
@@ -422,17 +506,43 @@ gemm_a8w8_wide(PersistParams pp)
                 const int nbuf = ks + 2 < nk ? (cur_gbase + (npair >> 1)) & 1 : (cur_gbase + groups_per_tile) & 1;
                 sc_rd_off = nbuf * MX_GROUP_BYTES + (ks + 2 < nk ? (npair & 1) * 512 : 0);
             }
-            step(std::integral_constant<int, 0>{});
-            step(std::integral_constant<int, 1>{});
+            if (ks == 0) step(F{}, T{}, F{});
+            else step(F{}, F{}, F{});
+            if (ks + 2 == nk) {
+                // from here on the accumulators are written out under this tile's coordinates
+                ep_batch = cur_batch;
+                ep_m0 = m0;
+                ep_n0 = n0;
+                ep_seq = tile_seq;
+                if constexpr (MODE == MODE_TENSOR)
+                    ep_ts = ((const float*)p.sfa + (long long)cur_batch * p.sfa_batch)[0] * ((const float*)p.sfb + (long long)cur_batch * p.sfb_batch)[0];
+                const uintptr_t c_addr = (uintptr_t)p.c + (uintptr_t)((long long)cur_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4));
+                ep_vec_ok = (p.ldc & (CDT == C_BF16 ? 7 : 3)) == 0 && (c_addr & 15) == 0;
+                // pieces are written without checks: only for whole tiles with aligned rows
+                const bool fast = ep_vec_ok && m0 + BM <= p.m && n0 + BN <= p.n;
+                if (fast) {
+                    step(T{}, F{}, T{});
+                    have_prev = true;
+                } else {
+                    step(T{}, F{}, F{});
+                    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // last MFMA -> first accumulator read
+                    store_tile_checked();
+                    have_prev = false;
+                }
+            } else {
+                step(T{}, F{}, F{});
+            }
         }
         cur_gbase += groups_per_tile;
-        // the compiler does not see the MFMAs: keep the required distance between the last of them
-        // and the first read of an accumulator
-        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-        store_tile();
         ++tile_seq;
         cur_item += gridDim.x;
         point_compute_at(cur_item);
+    }
+    // the last tile's last quadrant (the compiler does not see the MFMAs: keep the required distance
+    // between the last of them and the first read of an accumulator)
+    if (have_prev) {
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        static_for<8>([&](auto GQ) { flush_piece(std::integral_constant<int, 3>{}, GQ, std::integral_constant<int, 0>{}); });
     }
     __builtin_amdgcn_s_waitcnt(0);   // no direct-to-LDS load may outlive the workgroup's LDS allocation
 }
