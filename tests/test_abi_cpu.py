@@ -121,11 +121,14 @@ def test_pipelined_kernels_use_no_scratch():
     seen = 0
     for b in blocks:
         name = b.split()[0]
-        if "gemm_a8w8_persist" in name or "flatmm_a8w8" in name:
+        if "gemm_a8w8_persist" in name or "gemm_a8w8_wide" in name or "flatmm_a8w8" in name:
             seen += 1
             scratch = int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1))
             assert scratch == 0, (name, scratch)
-    assert seen >= 10
+    assert seen >= 16
+    # the four-wave kernels name their accumulator registers themselves: the build checks that the
+    # compiler put nothing of its own there (gcnasm_amd/csrc/check_isa.py) and records the verdict
+    assert "accumulator registers untouched by the compiler" in text
 
 
 def test_good_arguments_pass_validation_and_stop_at_the_device():
