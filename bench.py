@@ -31,7 +31,7 @@ PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA, published
 PEAK_FP4_TFLOPS = 10100.0     # MI355X dense FP4 MFMA, published
 # Bytes that crossed the L2 <-> fabric boundary per launch, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 117 MB device copy calibrates; profiles/).
-MEASURED_TRAFFIC = {"mxfp8_8192": 1.03e9, "flatmm_16x16384x7168": 1.190e8}
+MEASURED_TRAFFIC = {"mxfp8_8192": 1.08e9, "flatmm_16x16384x7168": 1.190e8}
 
 WORKLOADS = {
     # name: (mode, m, n, k, algorithmic bytes per launch)
