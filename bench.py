@@ -198,7 +198,7 @@ def run_workload(name, torch, g, steps, warmup, seed, headline=True):
                        ms_row_major_scales_one_launch=ms_direct, tflops_row_major_scales_one_launch=flops / ms_direct / 1e9,
                        step="a8w8_mx_tile_scales_ab(sfa, sfb) + a8w8_gemm(MX_TILED)")
         else:
-            res["kernel"] = ("gemm_a8w8_persist<bf16>" if mode == "bf16" else "gemm_a8w8_persist<mxfp4>" if mode == "f4"
+            res["kernel"] = ("gemm_a8w8_wide<bf16>" if mode == "bf16" else "gemm_a8w8_wide<mxfp4>" if mode == "f4"
                              else g.kernel_name(gemm_args))
             ms, wall = timer(torch, fn, steps, warmup)
         res.update(ms_per_launch=ms, wall_ms_per_launch=wall, tflops=flops / ms / 1e9, gbs=abytes / ms / 1e6)

@@ -178,7 +178,7 @@ int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
 template <int MODE, int CDT>
 int launch_wide(const GemmParams& p, int batch, hipStream_t stream)
 {
-    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT) {
+    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT || MODE == MODE_BF16 || MODE == MODE_F4T) {
         static bool attr_set[64];
         int dev = 0;
         (void)hipGetDevice(&dev);
@@ -309,6 +309,9 @@ int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
     if (fits && tiled_ok(&bytes) && persist_ok(&bytes)) {
         GemmParams p = make_params(&bytes);
         p.sfa = p.sfb = nullptr;
+        if ((bytes.k / BK) % 2 == 0)     // an even number of K steps: the four-wave kernel
+            return g->c_dtype == A8W8_C_BF16 ? launch_wide<MODE_BF16, C_BF16>(p, g->batch, s)
+                                             : launch_wide<MODE_BF16, C_FP32>(p, g->batch, s);
         return g->c_dtype == A8W8_C_BF16 ? launch_persist<MODE_BF16, C_BF16>(p, g->batch, s)
                                          : launch_persist<MODE_BF16, C_FP32>(p, g->batch, s);
     }
@@ -354,8 +357,8 @@ int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream)
     bytes.scale_mode = A8W8_SCALE_MX_E8M0_TILED;
     if (tiled && g->k % 256 == 0 && tiled_ok(&bytes) && persist_ok(&bytes)) {
         const GemmParams p = make_params(&bytes);
-        return g->c_dtype == A8W8_C_BF16 ? launch_persist<MODE_F4T, C_BF16>(p, g->batch, s)
-                                         : launch_persist<MODE_F4T, C_FP32>(p, g->batch, s);
+        return g->c_dtype == A8W8_C_BF16 ? launch_wide<MODE_F4T, C_BF16>(p, g->batch, s)
+                                         : launch_wide<MODE_F4T, C_FP32>(p, g->batch, s);
     }
     dim3 grid((unsigned)((g->n + 15) / 16), (unsigned)((g->m + 15) / 16), (unsigned)g->batch);
 #define A4W4_GENERAL(CDT, TILED)                                                                                        \

@@ -30,7 +30,7 @@ constexpr int WIDE_THREADS = 256;
 constexpr int WIDE_T = 8;                            // 8 x 8 MFMA tiles per wave
 constexpr int wide_lds_bytes(int mode)
 {
-    return GEMM_LDS_BYTES + (mode == MODE_MXT ? 2 * MX_GROUP_BYTES : mode == MODE_ROWCOL ? 2 * ROWCOL_SCALE_BYTES : 0);
+    return GEMM_LDS_BYTES + ((mode == MODE_MXT || mode == MODE_F4T) ? 2 * MX_GROUP_BYTES : mode == MODE_ROWCOL ? 2 * ROWCOL_SCALE_BYTES : 0);
 }
 
 // The 64 accumulator tiles of a wave live in accumulator registers a[0:255], tile (i, j) in
@@ -68,6 +68,24 @@ A8W8_DEV void mfma_acc_mx(const v8i& a, const v8i& b, int sa, int sb)
         asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel:[%6,%7,0] op_sel_hi:[%8,%9,0]" ::"v"(a),
                      "v"(b), "v"(sa), "v"(sb), "n"(LO), "n"(LO + 3), "n"(OA & 1), "n"(OB & 1), "n"(OA >> 1), "n"(OB >> 1));
 }
+// bf16 operands: one 16 x 16 x 32 MFMA per 16-byte half of a fragment
+template <int LO, bool ZC>
+A8W8_DEV void mfma_acc_bf16(const v4i& a, const v4i& b)
+{
+    if constexpr (ZC) asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(a), "v"(b), "n"(LO), "n"(LO + 3));
+    else asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(a), "v"(b), "n"(LO), "n"(LO + 3));
+}
+// packed E2M1 operands (format 4 for both): one 16 x 16 x 128 MFMA per 16-byte half of a fragment
+template <int LO, bool ZC, int OA, int OB>
+A8W8_DEV void mfma_acc_f4(const v4i& a, const v4i& b, int sa, int sb)
+{
+    if constexpr (ZC)
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, 0, %2, %3 op_sel:[%6,%7,0] op_sel_hi:[%8,%9,0] cbsz:4 blgp:4" ::"v"(a),
+                     "v"(b), "v"(sa), "v"(sb), "n"(LO), "n"(LO + 3), "n"(OA & 1), "n"(OB & 1), "n"(OA >> 1), "n"(OB >> 1));
+    else
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel:[%6,%7,0] op_sel_hi:[%8,%9,0] cbsz:4 blgp:4" ::"v"(a),
+                     "v"(b), "v"(sa), "v"(sb), "n"(LO), "n"(LO + 3), "n"(OA & 1), "n"(OB & 1), "n"(OA >> 1), "n"(OB >> 1));
+}
 template <int IDX>
 A8W8_DEV float acc_read()
 {
@@ -80,8 +98,15 @@ template <int MODE, int CDT>
 __global__ void __launch_bounds__(WIDE_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
 gemm_a8w8_wide(PersistParams pp)
 {
-    static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT, "scale modes of the four-wave kernel");
-    constexpr bool IS_MXT = MODE == MODE_MXT;
+    static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT || MODE == MODE_BF16 || MODE == MODE_F4T,
+                  "modes of the four-wave kernel");
+    // MODE_F4T (packed E2M1 operands): a 128-byte K step holds 256 elements = eight scale blocks = one
+    // "pair of K steps" of the tiled scale layout: the tiled-MX plumbing serves it with a scale fetch
+    // every step and two 16 x 16 x 128 FP4 MFMAs per fragment pair.  MODE_BF16: a step is 64 elements,
+    // two 16 x 16 x 32 MFMAs per fragment pair, no scales.
+    constexpr bool IS_MXT = MODE == MODE_MXT || MODE == MODE_F4T;   // tiled E8M0 scales
+    constexpr int MPF = (MODE == MODE_BF16 || MODE == MODE_F4T) ? 2 : 1;     // MFMAs per fragment pair
+    constexpr int PAIR_STEPS = MODE == MODE_F4T ? 1 : 2;             // K steps served by one fetch of scales
     // tiled MX scales are laid out for A tiles whose rows are dealt like the B tiles' rows
     constexpr bool PERM_A = IS_MXT;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -164,7 +189,8 @@ gemm_a8w8_wide(PersistParams pp)
                 const uint8_t* base = side ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
                                            : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
                 const int nblk = (rows + 63) >> 6;
-                const __amdgpu_buffer_rsrc_t rs = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, p.k));   // blocks past the edge read 0
+                const __amdgpu_buffer_rsrc_t rs =
+                    make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, MODE == MODE_F4T ? 2 * p.k : p.k));   // blocks past the edge read 0
                 const int voff = ((side ? tn * (BN / 64) : tm * (BM / 64)) + wave) * 1024 + lane * 16;
                 A8W8_LDS char* s = (A8W8_LDS char*)smem + GEMM_LDS_BYTES + buf * MX_GROUP_BYTES + side * 4096 + wave_lds;
                 load_to_lds_16(rs, s, voff, group * (nblk * 1024));
@@ -223,7 +249,7 @@ gemm_a8w8_wide(PersistParams pp)
     const int rd_sfb = GEMM_LDS_BYTES + 4096 + wave_n * 2048 + lane_rg * 8;
     v2i sc_a[2], sc_b[2], sc_a_next[2], sc_b_next[2];
     int sc_rd_off = 0;                              // LDS offset (buffer, pair) of the scales to fetch next
-    const int groups_per_tile = (nk + 3) >> 2;
+    const int groups_per_tile = (nk + 2 * PAIR_STEPS - 1) / (2 * PAIR_STEPS);   // a scale group is two pairs
     int cur_gbase = 0;                              // running group count: picks the scale buffer
 
     int cur_item = blockIdx.x;                     // the tile being multiplied
@@ -367,32 +393,47 @@ gemm_a8w8_wide(PersistParams pp)
         // registers and are updated in place, and the statements keep their order, so the source
         // order below is the schedule: two MFMAs, one LDS read; a load after every fourth MFMA.
         v4i half[8];
-        static_for<16>([&](auto TT) {
-            constexpr int t = decltype(TT)::value;
+        // 16 MPF slots: with two MFMAs per fragment pair, all first halves, then all second halves
+        // (two MFMAs in a row on one accumulator would wait for each other)
+        static_for<16 * MPF>([&](auto SS) {
+            constexpr int sl = decltype(SS)::value;
+            constexpr int hf = sl / 16, t = sl % 16;
             constexpr int j = jb + (a_outer ? (t & 3) : (t >> 2)), i = ia + (a_outer ? (t >> 2) : (t & 3));
             constexpr int lo = (i * 8 + j) * 4;
-            if constexpr (IS_MXT)
-                mfma_acc_mx<lo, zc, 2 * (j & 1) + sp, 2 * (i & 1) + sp>(fb[j], fa[i], sc_b[j >> 2][(j >> 1) & 1], sc_a[i >> 2][(i >> 1) & 1]);
-            else
-                mfma_acc<lo, zc>(fb[j], fa[i]);
-            if constexpr ((t & 1) != 0) {
-                constexpr int r = t >> 1, f = (ref & 1) * 4 + (r >> 1), h = r & 1;     // half h of fragment f
+            constexpr bool z = zc && hf == 0;
+            if constexpr (MODE == MODE_F4T) {
+                const v4i bh = hf ? v4i{fb[j][4], fb[j][5], fb[j][6], fb[j][7]} : v4i{fb[j][0], fb[j][1], fb[j][2], fb[j][3]};
+                const v4i ah = hf ? v4i{fa[i][4], fa[i][5], fa[i][6], fa[i][7]} : v4i{fa[i][0], fa[i][1], fa[i][2], fa[i][3]};
+                mfma_acc_f4<lo, z, 2 * (j & 1) + hf, 2 * (i & 1) + hf>(bh, ah, sc_b[j >> 2][(j >> 1) & 1], sc_a[i >> 2][(i >> 1) & 1]);
+            } else if constexpr (MODE == MODE_BF16) {
+                // a 128-byte row is 64 bf16: both operands split K the same way, so the order of the
+                // elements inside an instruction is immaterial
+                const v4i bh = hf ? v4i{fb[j][4], fb[j][5], fb[j][6], fb[j][7]} : v4i{fb[j][0], fb[j][1], fb[j][2], fb[j][3]};
+                const v4i ah = hf ? v4i{fa[i][4], fa[i][5], fa[i][6], fa[i][7]} : v4i{fa[i][0], fa[i][1], fa[i][2], fa[i][3]};
+                mfma_acc_bf16<lo, z>(bh, ah);
+            } else if constexpr (IS_MXT) {
+                mfma_acc_mx<lo, z, 2 * (j & 1) + sp, 2 * (i & 1) + sp>(fb[j], fa[i], sc_b[j >> 2][(j >> 1) & 1], sc_a[i >> 2][(i >> 1) & 1]);
+            } else {
+                mfma_acc<lo, z>(fb[j], fa[i]);
+            }
+            if constexpr (sl % (2 * MPF) == 2 * MPF - 1) {
+                constexpr int r = sl / (2 * MPF), f = (ref & 1) * 4 + (r >> 1), h = r & 1;     // half h of fragment f
                 constexpr int par = f & 1;
                 const int* base = ref < 2 ? rd_a : rd_b;
                 constexpr int off = (f >> 1) * (32 * BK) + par * (ref < 2 ? A_PAR_BYTES : B_PAR_BYTES);
                 half[r] = *(const v4i*)(smem + (rs * HALF_STAGE + off) + base[par ^ h]);
             }
-            if constexpr ((t & 3) == 2) issue_one(ls, lq, t >> 2);
-            if constexpr (IS_MXT && SCR && (t & 3) == 0) {
-                // the next pair of steps' scales, one 8-byte read after every fourth MFMA
-                constexpr int u = t >> 2;
+            if constexpr (sl % (4 * MPF) == 2 * MPF) issue_one(ls, lq, sl / (4 * MPF));
+            if constexpr (IS_MXT && SCR && sl % (4 * MPF) == 0) {
+                // the next pair's scales, four 8-byte reads spread over the quadrant
+                constexpr int u = sl / (4 * MPF);
                 const v2i v = *(const v2i*)(smem + sc_rd_off + (u < 2 ? rd_sfa : rd_sfb) + (u & 1) * 1024);
                 if constexpr (u < 2) sc_a_next[u] = v;
                 else sc_b_next[u - 2] = v;
             }
-            if constexpr (eq >= 0 && (t & 1) != 0) {
+            if constexpr (eq >= 0 && sl % (2 * MPF) == 2 * MPF - 1) {
                 using EQT = std::integral_constant<int, eq < 0 ? 0 : eq>;
-                using GQT = std::integral_constant<int, (t >> 1)>;
+                using GQT = std::integral_constant<int, sl / (2 * MPF)>;
                 using AOT = std::integral_constant<int, eqa ? 1 : 0>;
                 if constexpr (zc) {
                     if (have_prev) flush_piece(EQT{}, GQT{}, AOT{});
@@ -454,8 +495,15 @@ gemm_a8w8_wide(PersistParams pp)
             // aH x bH | read aL of the next step | load bH
             quad(I4{}, I4{}, I0{}, SN{}, I3{}, SP{}, I1{}, SP{}, I0{}, Z{}, I0{}, I0{});
             // aH x bL | read bH of the next step | load aH
-            quad(I4{}, I0{}, I3{}, SN{}, I1{}, SP{}, I0{}, SP{}, I0{}, Z{}, I0{}, I0{});
+            quad(I4{}, I0{}, I3{}, SN{}, I1{}, SP{}, I0{}, SP{}, std::integral_constant<int, PAIR_STEPS == 1 ? 1 : 0>{}, Z{}, I0{}, I0{});
             advance_ld();
+            if constexpr (IS_MXT && PAIR_STEPS == 1) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    sc_a[u] = sc_a_next[u];
+                    sc_b[u] = sc_b_next[u];
+                }
+            }
             if constexpr (FIRST) {
                 if (have_prev) handover(S8{});
                 else handover(S0{});
@@ -495,19 +543,27 @@ gemm_a8w8_wide(PersistParams pp)
         for (int ks = 0; ks < nk; ks += 2) {
             if constexpr (IS_MXT) {
                 // at the first step of a scale group: fetch the next group (of this tile or the first of
-                // the next tile) into the other buffer; its first pair is read three steps from here
-                if ((ks & 2) == 0) {
-                    const int g1 = (ks >> 2) + 1;
+                // the next tile) into the other buffer; its first pair is read at least a step from here
+                if (ks % (2 * PAIR_STEPS) == 0) {
+                    const int g1 = ks / (2 * PAIR_STEPS) + 1;
                     if (g1 < groups_per_tile) issue_mx_group(cur_item, g1, (cur_gbase + g1) & 1);
                     else issue_mx_group(cur_item + (int)gridDim.x, 0, (cur_gbase + groups_per_tile) & 1);
                 }
-                // where the pair after this one lives
-                const int npair = (ks >> 1) + 1;
-                const int nbuf = ks + 2 < nk ? (cur_gbase + (npair >> 1)) & 1 : (cur_gbase + groups_per_tile) & 1;
-                sc_rd_off = nbuf * MX_GROUP_BYTES + (ks + 2 < nk ? (npair & 1) * 512 : 0);
             }
+            // where the scales of the pair that starts at tile step `first` live (past the end: the next
+            // tile's first pair)
+            auto point_scale_read_at = [&](int first) __attribute__((always_inline)) {
+                if constexpr (IS_MXT) {
+                    const int q = first / PAIR_STEPS;
+                    const bool same = first < nk;
+                    const int buf = same ? (cur_gbase + (q >> 1)) & 1 : (cur_gbase + groups_per_tile) & 1;
+                    sc_rd_off = buf * MX_GROUP_BYTES + (same ? (q & 1) * 512 : 0);
+                }
+            };
+            point_scale_read_at(PAIR_STEPS == 1 ? ks + 1 : ks + 2);
             if (ks == 0) step(F{}, T{}, F{});
             else step(F{}, F{}, F{});
+            point_scale_read_at(ks + 2);
             if (ks + 2 == nk) {
                 // from here on the accumulators are written out under this tile's coordinates
                 ep_batch = cur_batch;
