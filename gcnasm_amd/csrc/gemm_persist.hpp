@@ -2,7 +2,8 @@
 //
 // Tile 256 x 256 x 128, 8 waves (4 along M x 2 along N), wave tile 64 x 128 = 4 x 8 MFMA
 // tiles of 16 x 16 x 128, operands staged global -> LDS with 16-byte direct-to-LDS loads,
-// two LDS stages of 64 KiB, 128-byte rows whose 16-byte slots are XOR-swizzled (see swz_key below).
+// two LDS stages of 64 KiB (laid out operand by operand: A of both stages, then B of both stages),
+// 128-byte rows whose 16-byte slots are XOR-swizzled (see swz_key below).
 //
 // What differs from the plain kernel:
 //  * One workgroup per CU walks a list of tiles; the K loop runs continuously across tile
@@ -47,9 +48,12 @@ constexpr int PERSIST_LDS_BYTES_ROWCOL = GEMM_LDS_BYTES + 2 * ROWCOL_SCALE_BYTES
 #ifndef A8W8_NPF_MX
 #define A8W8_NPF_MX 1
 #endif
+#ifndef A8W8_NPF_BLOCK
+#define A8W8_NPF_BLOCK 0
+#endif
 #define A8W8_PREFETCH_A(mode)                                                                        \
     ((mode) == MODE_TENSOR || (mode) == MODE_BF16 ? 4 : (mode) == MODE_ROWCOL ? A8W8_NPF_ROWCOL : (mode) == MODE_MXT || (mode) == MODE_F4T ? A8W8_NPF_MXT \
-                                                     : (mode) == MODE_MX ? A8W8_NPF_MX : 0)
+                                                     : (mode) == MODE_MX ? A8W8_NPF_MX : A8W8_NPF_BLOCK)
 #ifndef A8W8_PERSIST_BLK_LAG
 #define A8W8_PERSIST_BLK_LAG 4
 #endif
@@ -123,7 +127,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     const int groups_per_tile = (nk + GROUP_MASK) >> GROUP_SHIFT;   // MX scale groups per tile
     int ld_gbase = 0, cur_gbase = 0;                // running group count: picks the scale buffer
     __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_sf;
-    int ld_m0 = 0, ld_n0 = 0, voff_sf = 0;            // tile origin at the load position (wave-uniform)
+    int ld_voff_a = 0, ld_voff_b = 0, voff_sf = 0;  // lane offsets of the operand and scale loads at the load position
+    // LDS: [A of stage 0][A of stage 1][B of stage 0][B of stage 1], 32 KiB each: both stages of an
+    // operand lie within 64 KiB of the lane's base address, so stage and tile offsets are immediates
+    constexpr int HALF_STAGE = BM * BK, OPERAND_BYTES = 2 * HALF_STAGE;
     int sf_group_stride = 16;                       // bytes from one scale group of a row set to the next
     const int ld_row = wave * 8 + (lane >> 3);
     // lane i of a 1 KiB chunk lands on row (i>>3), slot (i&7) of the chunk's 8 rows; the slot holds
@@ -138,8 +145,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         const int m0 = tm * BM, n0 = tn * BN;
         rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
         rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, (uint32_t)(p.n - 1) * p.ldb + p.k);
-        ld_m0 = m0;
-        ld_n0 = n0;
+        ld_voff_a = __mul24(m0 + ld_row, p.lda) + ld_piece16;
+        ld_voff_b = __mul24(n0 + ld_row, p.ldb) + ld_piece16;
         if constexpr (MODE == MODE_MX) {
             const bool is_b = wave >= 4;           // waves 0-3 stage A-row scales, 4-7 B-row scales
             const int rows = is_b ? p.n : p.m;
@@ -168,18 +175,16 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     // Wave w fills rows 8w + 64j (+0..7) of each matrix; for B, j = 0, 2 are the rows of MFMA
     // tiles 0-3 of the two wave columns ("low"), j = 1, 3 those of tiles 4-7 ("high").
     auto issue_one = [&](int stage, int kstep, int which) __attribute__((always_inline)) {
-        A8W8_LDS char* s = (A8W8_LDS char*)smem + stage * STAGE_BYTES + wave * 1024;
+        A8W8_LDS char* s = (A8W8_LDS char*)smem + stage * HALF_STAGE + wave * 1024;
         const int koff = kstep * BK;
-        // the lane's byte offset is recomputed for every load (three VALU operations) rather than
-        // kept in eight registers: the kernel has none to spare, and a spilled offset would be
-        // reloaded from scratch behind a wait for every load in flight
+        // One lane offset per operand (the wave's rows of the tile's first 64, set per tile); the 64-row
+        // chunk rides in the scalar offset.  Rows past the end of a matrix are past the end of its
+        // descriptor: they read as zero and only reach accumulators that are never stored.
         if (which < 4) {
-            const int voff = __mul24(min(ld_m0 + ld_row + 64 * which, p.m - 1), p.lda) + ld_piece16;
-            load_to_lds_16(rsrc_a, s + which * 8192, voff, koff);
+            load_to_lds_16(rsrc_a, s + which * 8192, ld_voff_a, koff + 64 * which * p.lda);
         } else {
             const int j = which == 4 ? 0 : which == 5 ? 2 : which == 6 ? 1 : 3;
-            const int voff = __mul24(min(ld_n0 + ld_row + 64 * j, p.n - 1), p.ldb) + ld_piece16;
-            load_to_lds_16(rsrc_b, s + BM * BK + j * 8192, voff, koff);
+            load_to_lds_16(rsrc_b, s + OPERAND_BYTES + j * 8192, ld_voff_b, koff + 64 * j * p.ldb);
         }
     };
     auto issue_mx_group = [&](int group) __attribute__((always_inline)) {
@@ -232,10 +237,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         const int row_b = 8 * (r16 >> 2) + (r16 & 3);
         const int row_a = PERM_A ? row_b : r16;
         rd_a[h] = (wave_m * WAVE_M + row_a) * BK + ((((g + 4 * h) ^ swz_key(row_a)) & 7) << 4);
-        rd_b[h] = BM * BK + (wave_n * WAVE_N + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
+        rd_b[h] = OPERAND_BYTES + (wave_n * WAVE_N + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
     }
     auto read_frag_at = [&](int stage, const int (&base)[2], int par, int byte_off) __attribute__((always_inline)) -> v8i {
-        const char* s = smem + stage * STAGE_BYTES + byte_off;
+        const char* s = smem + stage * HALF_STAGE + byte_off;
         const v4i lo = *(const v4i*)(s + base[par]);
         const v4i hi = *(const v4i*)(s + base[par ^ 1]);
         return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
