@@ -30,7 +30,8 @@ constexpr int WIDE_THREADS = 256;
 constexpr int WIDE_T = 8;                            // 8 x 8 MFMA tiles per wave
 constexpr int wide_lds_bytes(int mode)
 {
-    return GEMM_LDS_BYTES + ((mode == MODE_MXT || mode == MODE_F4T) ? 2 * MX_GROUP_BYTES : mode == MODE_ROWCOL ? 2 * ROWCOL_SCALE_BYTES : 0);
+    // tiled MX scales: two buffers of two scale groups each, i.e. all of the 160 KiB
+    return GEMM_LDS_BYTES + ((mode == MODE_MXT || mode == MODE_F4T) ? 4 * MX_GROUP_BYTES : mode == MODE_ROWCOL ? 2 * ROWCOL_SCALE_BYTES : 0);
 }
 
 // The 64 accumulator tiles of a wave live in accumulator registers a[0:255], tile (i, j) in
@@ -176,25 +177,46 @@ gemm_a8w8_wide(PersistParams pp)
 
     // Tiled MX scales: the exponents of a 64-row block for four K steps are 1 KiB of contiguous memory
     // in the order the lanes read them ([pair of steps][lane (r16, g)][8 bytes]).  Wave w copies block w
-    // of the A tile and block w of the B tile of one scale group (four K steps) into LDS buffer `buf`.
-    auto issue_mx_group = [&](int item, int group, int buf) __attribute__((always_inline)) {
+    // of the A tile and block w of the B tile of one scale group into LDS buffer `buf`.  Everything
+    // that depends on the tile (batch entry, first block of the tile) is worked out once per tile, for
+    // this tile and the next one, so that a group costs two loads and a few scalar instructions.
+    struct ScaleTile {
+        const uint8_t* base[2];                    // scale arrays of the tile's batch entry (A side, B side)
+        int blk[2];                                // the tile's first 64-row block
+    };
+    ScaleTile sf_cur = {}, sf_next = {};
+    const int sf_nblk[2] = {(p.m + 63) >> 6, (p.n + 63) >> 6};
+    const uint32_t sf_bytes[2] = {(uint32_t)mx_tiled_bytes(p.m, MODE == MODE_F4T ? 2 * p.k : p.k),
+                                  (uint32_t)mx_tiled_bytes(p.n, MODE == MODE_F4T ? 2 * p.k : p.k)};
+    auto point_scales_at = [&](ScaleTile& t, int item) __attribute__((always_inline)) {
         if constexpr (IS_MXT) {
             item = min(item, pp.items - 1);
             const int batch = item / tiles;
             int tm, tn;
             tile_of_block(item - batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+            t.base[0] = (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
+            t.base[1] = (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch;
+            t.blk[0] = tm * (BM / 64);
+            t.blk[1] = tn * (BN / 64);
+        }
+    };
+    const int lane16 = lane * 16;
+    // The scale loads are few but slow (each touches lines that are cold in L2; measured: the same
+    // loads from an always-hot region make the 8192^3 launch 10% faster on all-zero operands and 3% on
+    // random ones).  They are issued in batches of GPB scale groups, as rarely as LDS allows.
+    constexpr int GPB = 2;
+    constexpr int BATCH_BYTES = GPB * MX_GROUP_BYTES;
+    auto issue_mx_batch = [&](const ScaleTile& t, int batch, int buf) __attribute__((always_inline)) {
+        if constexpr (IS_MXT) {
 #pragma unroll
-            for (int side = 0; side < 2; ++side) {
-                const int rows = side ? p.n : p.m;
-                const uint8_t* base = side ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
-                                           : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
-                const int nblk = (rows + 63) >> 6;
-                const __amdgpu_buffer_rsrc_t rs =
-                    make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, MODE == MODE_F4T ? 2 * p.k : p.k));   // blocks past the edge read 0
-                const int voff = ((side ? tn * (BN / 64) : tm * (BM / 64)) + wave) * 1024 + lane * 16;
-                A8W8_LDS char* s = (A8W8_LDS char*)smem + GEMM_LDS_BYTES + buf * MX_GROUP_BYTES + side * 4096 + wave_lds;
-                load_to_lds_16(rs, s, voff, group * (nblk * 1024));
-            }
+            for (int gi = 0; gi < GPB; ++gi)
+#pragma unroll
+                for (int side = 0; side < 2; ++side) {
+                    const __amdgpu_buffer_rsrc_t rs = make_rsrc(t.base[side], sf_bytes[side]);   // past the end: reads 0
+                    A8W8_LDS char* s =
+                        (A8W8_LDS char*)smem + GEMM_LDS_BYTES + buf * BATCH_BYTES + gi * MX_GROUP_BYTES + side * 4096 + wave_lds;
+                    load_to_lds_16(rs, s, lane16, ((batch * GPB + gi) * sf_nblk[side] + t.blk[side] + wave) * 1024);
+                }
         }
     };
     // Row/col scales of a tile: thread t fetches sfa[m0 + t] and sfb[n0 + t] (indices clamped) into LDS
@@ -249,8 +271,9 @@ gemm_a8w8_wide(PersistParams pp)
     const int rd_sfb = GEMM_LDS_BYTES + 4096 + wave_n * 2048 + lane_rg * 8;
     v2i sc_a[2], sc_b[2], sc_a_next[2], sc_b_next[2];
     int sc_rd_off = 0;                              // LDS offset (buffer, pair) of the scales to fetch next
-    const int groups_per_tile = (nk + 2 * PAIR_STEPS - 1) / (2 * PAIR_STEPS);   // a scale group is two pairs
-    int cur_gbase = 0;                              // running group count: picks the scale buffer
+    constexpr int BATCH_STEPS = 2 * 2 * PAIR_STEPS;  // K steps served by one batch: two scale groups of two pairs
+    const int batches_per_tile = (nk + BATCH_STEPS - 1) / BATCH_STEPS;
+    int cur_bbase = 0;                              // running batch count: picks the scale buffer
 
     int cur_item = blockIdx.x;                     // the tile being multiplied
     int cur_batch = 0, m0 = 0, n0 = 0;
@@ -344,7 +367,9 @@ gemm_a8w8_wide(PersistParams pp)
     if (my_items == 0) return;
     point_loads_at(ld_item);
     point_compute_at(cur_item);
-    issue_mx_group(cur_item, 0, 0);
+    point_scales_at(sf_cur, cur_item);
+    point_scales_at(sf_next, cur_item + (int)gridDim.x);
+    issue_mx_batch(sf_cur, 0, 0);
     // steps 0 and 1 in full
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
@@ -542,22 +567,22 @@ gemm_a8w8_wide(PersistParams pp)
         issue_rowcol_scales(cur_batch, m0, n0, tile_seq & 1);
         for (int ks = 0; ks < nk; ks += 2) {
             if constexpr (IS_MXT) {
-                // at the first step of a scale group: fetch the next group (of this tile or the first of
-                // the next tile) into the other buffer; its first pair is read at least a step from here
-                if (ks % (2 * PAIR_STEPS) == 0) {
-                    const int g1 = ks / (2 * PAIR_STEPS) + 1;
-                    if (g1 < groups_per_tile) issue_mx_group(cur_item, g1, (cur_gbase + g1) & 1);
-                    else issue_mx_group(cur_item + (int)gridDim.x, 0, (cur_gbase + groups_per_tile) & 1);
+                // at the first step of a batch of scale groups: fetch the next batch (of this tile or the
+                // first of the next tile) into the other buffer; its first pair is read steps from here
+                if (ks % BATCH_STEPS == 0) {
+                    const int b1 = ks / BATCH_STEPS + 1;
+                    if (b1 < batches_per_tile) issue_mx_batch(sf_cur, b1, (cur_bbase + b1) & 1);
+                    else issue_mx_batch(sf_next, 0, (cur_bbase + batches_per_tile) & 1);
                 }
             }
             // where the scales of the pair that starts at tile step `first` live (past the end: the next
             // tile's first pair)
             auto point_scale_read_at = [&](int first) __attribute__((always_inline)) {
                 if constexpr (IS_MXT) {
-                    const int q = first / PAIR_STEPS;
+                    const int q = first / PAIR_STEPS;          // pair; two pairs per scale group, GPB groups per batch
                     const bool same = first < nk;
-                    const int buf = same ? (cur_gbase + (q >> 1)) & 1 : (cur_gbase + groups_per_tile) & 1;
-                    sc_rd_off = buf * MX_GROUP_BYTES + (same ? (q & 1) * 512 : 0);
+                    const int buf = same ? (cur_bbase + (q >> 2)) & 1 : (cur_bbase + batches_per_tile) & 1;
+                    sc_rd_off = buf * BATCH_BYTES + (same ? ((q >> 1) & 1) * MX_GROUP_BYTES + (q & 1) * 512 : 0);
                 }
             };
             point_scale_read_at(PAIR_STEPS == 1 ? ks + 1 : ks + 2);
@@ -589,10 +614,12 @@ gemm_a8w8_wide(PersistParams pp)
                 step(T{}, F{}, F{});
             }
         }
-        cur_gbase += groups_per_tile;
+        cur_bbase += batches_per_tile;
         ++tile_seq;
         cur_item += gridDim.x;
         point_compute_at(cur_item);
+        sf_cur = sf_next;
+        point_scales_at(sf_next, cur_item + (int)gridDim.x);
     }
     // the last tile's last quadrant (the compiler does not see the MFMAs: keep the required distance
     // between the last of them and the first read of an accumulator)
