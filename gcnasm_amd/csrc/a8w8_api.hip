@@ -148,17 +148,21 @@ int launch_tiled(const GemmParams& p, int batch, hipStream_t stream)
     }
 }
 
-// Persistent pipelined kernel: one workgroup per CU walks the (batch, tile) list.
+template <int MODE, int CDT>
+int launch_wide(const GemmParams& p, int batch, hipStream_t stream);
+
+// Persistent pipelined kernel (eight waves): one workgroup per CU walks the (batch, tile) list.
 template <int MODE, int CDT>
 int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
 {
+    // tiled MX scales exist on the four-wave kernel only (whatever passes persist_ok with them also passes wide_ok)
+    if constexpr (MODE == MODE_MXT) return launch_wide<MODE, CDT>(p, batch, stream);
+    else {
     static bool attr_set[64];
     int dev = 0;
     (void)hipGetDevice(&dev);
     auto kern = gemm_a8w8_persist<MODE, CDT>;
-    constexpr int lds_bytes = (MODE == MODE_MX || MODE == MODE_MXT || MODE == MODE_F4T) ? PERSIST_LDS_BYTES_MX
-                              : MODE == MODE_ROWCOL                   ? PERSIST_LDS_BYTES_ROWCOL
-                                                                      : PERSIST_LDS_BYTES;
+    constexpr int lds_bytes = MODE == MODE_MX ? PERSIST_LDS_BYTES_MX : MODE == MODE_ROWCOL ? PERSIST_LDS_BYTES_ROWCOL : PERSIST_LDS_BYTES;
     if (!attr_set[dev & 63]) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
             return A8W8_ERR_LAUNCH;
@@ -172,6 +176,7 @@ int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
     dim3 grid((unsigned)(pp.items < cus ? pp.items : cus), 1, 1);
     hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), lds_bytes, stream, pp);
     return launch_status();
+    }
 }
 
 // Four-wave persistent kernel (one wave per SIMD, 128 x 128 per wave).

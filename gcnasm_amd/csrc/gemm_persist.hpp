@@ -42,9 +42,6 @@ constexpr int PERSIST_LDS_BYTES_ROWCOL = GEMM_LDS_BYTES + 2 * ROWCOL_SCALE_BYTES
 #ifndef A8W8_NPF_ROWCOL
 #define A8W8_NPF_ROWCOL 2
 #endif
-#ifndef A8W8_NPF_MXT
-#define A8W8_NPF_MXT 2
-#endif
 #ifndef A8W8_NPF_MX
 #define A8W8_NPF_MX 1
 #endif
@@ -52,7 +49,7 @@ constexpr int PERSIST_LDS_BYTES_ROWCOL = GEMM_LDS_BYTES + 2 * ROWCOL_SCALE_BYTES
 #define A8W8_NPF_BLOCK 0
 #endif
 #define A8W8_PREFETCH_A(mode)                                                                        \
-    ((mode) == MODE_TENSOR || (mode) == MODE_BF16 ? 4 : (mode) == MODE_ROWCOL ? A8W8_NPF_ROWCOL : (mode) == MODE_MXT || (mode) == MODE_F4T ? A8W8_NPF_MXT \
+    ((mode) == MODE_TENSOR || (mode) == MODE_BF16 ? 4 : (mode) == MODE_ROWCOL ? A8W8_NPF_ROWCOL \
                                                      : (mode) == MODE_MX ? A8W8_NPF_MX : A8W8_NPF_BLOCK)
 #ifndef A8W8_PERSIST_BLK_LAG
 #define A8W8_PERSIST_BLK_LAG 4
@@ -79,20 +76,6 @@ constexpr int PERSIST_LDS_BYTES_ROWCOL = GEMM_LDS_BYTES + 2 * ROWCOL_SCALE_BYTES
 #define A8W8_PERSIST_SCHED_BARRIER() (void)0
 #endif
 
-// scaled MFMA taking byte OA of scale_a and byte OB of scale_b (the selectors are immediates)
-template <int OA, int OB>
-A8W8_DEV v4f mfma_mx_sel(v8i a, v8i b, v4f c, int scale_a, int scale_b)
-{
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, OA, scale_a, OB, scale_b);
-}
-
-// the same for packed E2M1 operands (format 4 for A and B; only the low four operand registers are read)
-template <int OA, int OB>
-A8W8_DEV v4f mfma_f4_sel(v8i a, v8i b, v4f c, int scale_a, int scale_b)
-{
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 4, 4, OA, scale_a, OB, scale_b);
-}
-
 struct PersistParams {
     GemmParams g;
     int batch;        // work items = batch * tiles_m * tiles_n, walked with stride gridDim.x
@@ -108,15 +91,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     const int lane = tid & 63;
     const int wave = wave_uniform(tid >> 6);
     const int wave_m = wave >> 1, wave_n = wave & 1;
-    // MODE_F4T (packed E2M1 operands): a 128-byte K step holds 256 elements = eight scale blocks = one
-    // "pair of K steps" of the tiled scale layout, so the tiled-MX plumbing serves it with two steps
-    // per scale group, a scale fetch every step, and two 16x16x128 FP4 MFMAs per fragment pair.
-    constexpr bool TILED_SF = MODE == MODE_MXT || MODE == MODE_F4T;
-    constexpr bool IS_MX = MODE == MODE_MX || TILED_SF;
-    constexpr int GROUP_SHIFT = MODE == MODE_F4T ? 1 : 2;          // log2(K steps per scale group)
+    static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_BF16,
+                  "tiled MX scales and MXFP4 operands run on the four-wave kernel");
+    constexpr bool IS_MX = MODE == MODE_MX;
+    constexpr int GROUP_SHIFT = 2;                                 // log2(K steps per scale group)
     constexpr int GROUP_MASK = (1 << GROUP_SHIFT) - 1;
-    // tiled MX scales are laid out for A tiles whose rows are dealt like the B tiles' rows
-    constexpr bool PERM_A = TILED_SF;
     const int r16 = lane & 15, g = lane >> 4;
     const int nk = p.k / BK;                       // >= 2 (checked by the host)
     const int tiles = p.tiles_m * p.tiles_n;
@@ -131,7 +110,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     // LDS: [A of stage 0][A of stage 1][B of stage 0][B of stage 1], 32 KiB each: both stages of an
     // operand lie within 64 KiB of the lane's base address, so stage and tile offsets are immediates
     constexpr int HALF_STAGE = BM * BK, OPERAND_BYTES = 2 * HALF_STAGE;
-    int sf_group_stride = 16;                       // bytes from one scale group of a row set to the next
     const int ld_row = wave * 8 + (lane >> 3);
     // lane i of a 1 KiB chunk lands on row (i>>3), slot (i&7) of the chunk's 8 rows; the slot holds
     // K-piece slot ^ key(row) with key(row) = (row & 7) ^ (((row >> 3) & 3) << 1), and bits 3-4 of the
@@ -156,20 +134,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             rsrc_sf = make_rsrc(base, (uint32_t)(rows - 1) * stride + (uint32_t)(p.k >> 5));
             voff_sf = min((is_b ? n0 : m0) + (wave & 3) * 64 + lane, rows - 1) * stride;
         }
-        if constexpr (TILED_SF) {
-            // tiled scales: a 64-row block's exponents for four K steps are 1 KiB of contiguous memory
-            // in the order the lanes read them, so wave w copies block (w & 3) of the A tile (waves
-            // 0-3) or of the B tile (waves 4-7) with one load of eight whole cache lines.
-            const bool is_b = wave >= 4;
-            const int rows = is_b ? p.n : p.m;
-            const uint8_t* base = is_b ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
-                                       : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
-            const int nblk = (rows + 63) >> 6;
-            const int k_elems = MODE == MODE_F4T ? 2 * p.k : p.k;
-            rsrc_sf = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, k_elems));   // blocks past the edge read 0
-            voff_sf = (((is_b ? n0 : m0) >> 6) + (wave & 3)) * 1024 + lane * 16;
-            sf_group_stride = wave_uniform(nblk * 1024);
-        }
     };
     // one of the eight loads of a stage: 0..3 = A chunks, 4,5 = low B chunks, 6,7 = high B chunks.
     // Wave w fills rows 8w + 64j (+0..7) of each matrix; for B, j = 0, 2 are the rows of MFMA
@@ -191,7 +155,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         if constexpr (IS_MX) {
             A8W8_LDS char* s =
                 (A8W8_LDS char*)smem + GEMM_LDS_BYTES + ((ld_gbase + group) & 1) * MX_GROUP_BYTES + wave * 1024;
-            load_to_lds_16(rsrc_sf, s, voff_sf, group * sf_group_stride);
+            load_to_lds_16(rsrc_sf, s, voff_sf, group * 16);   // 16 scale bytes per row and group
         }
     };
     int tile_seq = 0;                               // tiles this workgroup has started: picks the scale buffer
@@ -224,18 +188,17 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     //     tile j, operand row 4g' + i  <-  row 32*(j/2) + 8g' + 4*(j%2) + i.
     // The swizzle key (row & 7) ^ (((row >> 3) & 3) << 1) keeps both read patterns free of LDS bank
     // conflicts (measured).  Only the tile's parity enters the key, the rest is an immediate offset.
-    const int lane_rg = r16 * 4 + g;
     auto swz_key = [](int row) __attribute__((always_inline)) { return ((row & 7) ^ (((row >> 3) & 3) << 1)) & 7; };
     // For the rows of tile parity 1 the key differs from parity 0's in bit 2 only, and so do the two
     // K halves h of a fragment: slot(par, h) = slot(0, 0) ^ 4 (par ^ h).  Two address registers per
     // operand (h = 0, 1 of parity 0) therefore serve all four combinations; parity 1 swaps them and
     // adds its row offset as an immediate.
-    constexpr int A_PAR_BYTES = (PERM_A ? 4 : 16) * BK, B_PAR_BYTES = 4 * BK;
+    constexpr int A_PAR_BYTES = 16 * BK, B_PAR_BYTES = 4 * BK;
     int rd_a[2], rd_b[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         const int row_b = 8 * (r16 >> 2) + (r16 & 3);
-        const int row_a = PERM_A ? row_b : r16;
+        const int row_a = r16;
         rd_a[h] = (wave_m * WAVE_M + row_a) * BK + ((((g + 4 * h) ^ swz_key(row_a)) & 7) << 4);
         rd_b[h] = OPERAND_BYTES + (wave_n * WAVE_N + row_b) * BK + ((((g + 4 * h) ^ swz_key(row_b)) & 7) << 4);
     }
@@ -251,13 +214,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     auto read_frag_b = [&](int stage, int j) __attribute__((always_inline)) -> v8i {
         return read_frag_at(stage, rd_b, j & 1, (j >> 1) * (32 * BK) + (j & 1) * B_PAR_BYTES);
     };
-    // natural MX scales: B tile t at + (t >> 1) * 512 + (t & 1) * 64; tiled: tile t at + t * 256, dword g
-    // tiled: 1 KiB per 64-row block = [pair of K steps][lane (r16, g)][8 bytes]
-    const int rd_sfa = TILED_SF ? GEMM_LDS_BYTES + wave_m * 1024 + lane_rg * 8
-                                        : GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16;
-    const int rd_sfb = TILED_SF
-                           ? GEMM_LDS_BYTES + 4096 + wave_n * 2048 + lane_rg * 8
-                           : GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + 8 * (r16 >> 2) + (r16 & 3)) * 16;
+    // MX scales (16 bytes per row per group of four K steps): B tile t at + (t >> 1) * 512 + (t & 1) * 64
+    const int rd_sfa = GEMM_LDS_BYTES + (wave_m * WAVE_M + r16) * 16;
+    const int rd_sfb = GEMM_LDS_BYTES + BM * 16 + (wave_n * WAVE_N + 8 * (r16 >> 2) + (r16 & 3)) * 16;
 
     int cur_item = blockIdx.x, cur_ks = 0;         // the step being multiplied
     int cur_batch = 0, m0 = 0, n0 = 0;
@@ -280,8 +239,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     // scales consumed by the MFMAs of a step (BLOCK: fp32 per row x per column block, MX: E8M0 bytes)
     float blk_s[TM], blk_s_next[TM];
     int mx_sa[TM], mx_sb[TN], mx_sa_next[TM], mx_sb_next[TN];
-    v2i mxt_a, mxt_a_next;      // tiled MX: dword t/2 serves tiles t, t^1 and both steps of a pair
-    v4i mxt_b, mxt_b_next;
     __amdgpu_buffer_rsrc_t blk_rs;                  // block scales of the tile whose scales are being fetched
     const float* blk_sfb_row = nullptr;
     int blk_voff[TM] = {0, 0, 0, 0};
@@ -322,15 +279,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             for (int t = 0; t < TN; ++t)
                 mx_sb_next[t] = *(const int*)(s + rd_sfb + (t >> 1) * 512 + (t & 1) * 64);
         }
-        if constexpr (TILED_SF) {
-            // called for the first step of a pair (FP4: for every step, which is a pair by itself): the
-            // lane's eight bytes per 64-row block
-            const int pair = MODE == MODE_F4T ? (kstep & 1) : ((kstep >> 1) & 1);
-            const char* s = smem + ((gbase + (kstep >> GROUP_SHIFT)) & 1) * MX_GROUP_BYTES + pair * 512;
-            mxt_a_next = *(const v2i*)(s + rd_sfa);
-            const v2i lo = *(const v2i*)(s + rd_sfb), hi = *(const v2i*)(s + rd_sfb + 1024);
-            mxt_b_next = v4i{lo.x, lo.y, hi.x, hi.y};
-        }
     };
     auto rotate_step_scales = [&]() __attribute__((always_inline)) {
         if constexpr (MODE == MODE_BLOCK) {
@@ -343,20 +291,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
 #pragma unroll
             for (int t = 0; t < TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe((unsigned)mx_sb_next[t], 8 * g, 8);
         }
-        if constexpr (TILED_SF) {
-            mxt_a = mxt_a_next;
-            mxt_b = mxt_b_next;
-        }
     };
 
     // ---------------------------------------------------------------- epilogue of one tile
     auto store_tile = [&]() __attribute__((always_inline)) {
         const float* sfa_f = (const float*)p.sfa + (long long)cur_batch * p.sfa_batch;
         const float* sfb_f = (const float*)p.sfb + (long long)cur_batch * p.sfb_batch;
-        const int cm_base = m0 + wave_m * WAVE_M + (PERM_A ? 8 * (r16 >> 2) + (r16 & 3) : r16);
-        auto cm_of = [&](int i) __attribute__((always_inline)) {          // C row of MFMA tile i
-            return cm_base + (PERM_A ? 32 * (i >> 1) + 4 * (i & 1) : 16 * i);
-        };
+        const int cm_base = m0 + wave_m * WAVE_M + r16;
+        auto cm_of = [&](int i) __attribute__((always_inline)) { return cm_base + 16 * i; };   // C row of MFMA tile i
         const int cn_base = n0 + wave_n * WAVE_N + 8 * g;      // + 32 * (tile pair): eight consecutive n
         float sa[TM];
         float ts = 1.f;
@@ -469,7 +411,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         constexpr int P = decltype(parity)::value;
         Frags& cur = F[PREFETCH_FRAGS ? P : 0];
         Frags& nxt = F[PREFETCH_FRAGS ? P ^ 1 : 0];
-        if constexpr (MODE != MODE_MXT || P == 0) rotate_step_scales();   // tiled MXFP8: one dword serves two steps
+        rotate_step_scales();
 #pragma unroll
         for (int t = NPF; t < TM; ++t) cur.a[t] = read_frag_a(P, t);
         if constexpr (!PREFETCH_FRAGS) cur.b0 = read_frag_b(P, 0);
@@ -500,23 +442,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             A8W8_PERSIST_SCHED_BARRIER();
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                if constexpr (MODE == MODE_F4T) {
-                    // first halves of the fragments here (op_sel byte 2*(tile parity)), second halves after
-                    // the loop: format 4 = E2M1 for both operands, the upper four operand registers unused
-                    const int sb = mxt_b[j >> 1], sa = mxt_a[i >> 1];
-                    const v8i fb4 = {fb[j][0], fb[j][1], fb[j][2], fb[j][3], 0, 0, 0, 0};
-                    const v8i fa4 = {cur.a[i][0], cur.a[i][1], cur.a[i][2], cur.a[i][3], 0, 0, 0, 0};
-                    acc[i][j] = (j & 1) ? ((i & 1) ? mfma_f4_sel<2, 2>(fb4, fa4, acc[i][j], sb, sa) : mfma_f4_sel<2, 0>(fb4, fa4, acc[i][j], sb, sa))
-                                        : ((i & 1) ? mfma_f4_sel<0, 2>(fb4, fa4, acc[i][j], sb, sa) : mfma_f4_sel<0, 0>(fb4, fa4, acc[i][j], sb, sa));
-                } else if constexpr (MODE == MODE_MXT) {
-                    // K steps come in pairs and tiles start on even steps, so the step inside the
-                    // pair is the LDS stage parity P
-                    const int sb = mxt_b[j >> 1], sa = mxt_a[i >> 1];
-                    acc[i][j] = (j & 1) ? ((i & 1) ? mfma_mx_sel<2 + P, 2 + P>(fb[j], cur.a[i], acc[i][j], sb, sa)
-                                                   : mfma_mx_sel<2 + P, P>(fb[j], cur.a[i], acc[i][j], sb, sa))
-                                        : ((i & 1) ? mfma_mx_sel<P, 2 + P>(fb[j], cur.a[i], acc[i][j], sb, sa)
-                                                   : mfma_mx_sel<P, P>(fb[j], cur.a[i], acc[i][j], sb, sa));
-                } else if constexpr (MODE == MODE_MX) {
+                if constexpr (MODE == MODE_MX) {
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], cur.a[i], acc[i][j], 0, 0, 0,
                                                                                  mx_sb[j], 0, mx_sa[i]);
                 } else if constexpr (MODE == MODE_BLOCK) {
@@ -547,16 +473,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                                                                                  0, 0, 0);
                 }
             }
-            if constexpr (MODE == MODE_F4T) {
-#pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    const int sb = mxt_b[j >> 1], sa = mxt_a[i >> 1];
-                    const v8i fb4 = {fb[j][4], fb[j][5], fb[j][6], fb[j][7], 0, 0, 0, 0};
-                    const v8i fa4 = {cur.a[i][4], cur.a[i][5], cur.a[i][6], cur.a[i][7], 0, 0, 0, 0};
-                    acc[i][j] = (j & 1) ? ((i & 1) ? mfma_f4_sel<3, 3>(fb4, fa4, acc[i][j], sb, sa) : mfma_f4_sel<3, 1>(fb4, fa4, acc[i][j], sb, sa))
-                                        : ((i & 1) ? mfma_f4_sel<1, 3>(fb4, fa4, acc[i][j], sb, sa) : mfma_f4_sel<1, 1>(fb4, fa4, acc[i][j], sb, sa));
-                }
-            }
             if constexpr (MODE == MODE_BF16) {
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
@@ -570,7 +486,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
 #if A8W8_PERSIST_SG
             if constexpr (MODE != MODE_BLOCK) {
                 // spread the two LDS reads of the next B fragment between this group's MFMAs
-                constexpr int MPF = (MODE == MODE_BF16 || MODE == MODE_F4T) ? 2 : 1;      // MFMAs per operand fragment pair
+                constexpr int MPF = MODE == MODE_BF16 ? 2 : 1;      // MFMAs per operand fragment pair
                 if (j + 1 < TN) {
                     __builtin_amdgcn_sched_group_barrier(0x008, MPF, 0);
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -614,8 +530,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                     nxt.b0 = read_frag_b(P ^ 1, 0);
                 }
                 if constexpr (MODE == MODE_MX) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
-                if constexpr (MODE == MODE_MXT && P == 1) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
-                if constexpr (MODE == MODE_F4T) fetch_step_scales(nx_batch, nx_m0, nx_n0, nx_ks, nx_gbase);
             }
             if (j == 7) {
                 issue_one(P, ld_ks, 4);
