@@ -213,6 +213,36 @@ def run_workload(name, torch, g, steps, warmup, seed, headline=True):
     return res, inp, c
 
 
+def run_quantizers(torch, g, steps, warmup, seed):
+    """The quantisation front end on the headline's activation shape (fp32 8192 x 8192 in, E4M3 + scales out):
+    HBM-bound byte work, priced against the HBM peak with each byte counted once."""
+    import ctypes
+    rows, k = 8192, 8192
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    x = torch.randn((rows, k), generator=gen, device="cuda", dtype=torch.float32)
+    q = torch.empty((rows, k), dtype=torch.uint8, device="cuda")
+    L = g.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = []
+    for name, mode, scale_bytes in (("quantize_mx_tiled_8192", g.MX_TILED, g.mx_tiled_bytes(rows, k)),
+                                    ("quantize_rowcol_8192", g.ROWCOL, rows * 4)):
+        sc = torch.empty(scale_bytes, dtype=torch.uint8, device="cuda")
+        xp, qp, sp = (ctypes.c_void_p(t.data_ptr()) for t in (x, q, sc))
+
+        def fn(i):
+            if L.a8w8_quantize(xp, rows, k, k, qp, sp, mode, 1, stream) != 0:
+                raise RuntimeError("a8w8_quantize failed")
+
+        ms, wall = time_best_of(torch, fn, steps, warmup)
+        abytes = rows * k * 5 + scale_bytes
+        out.append({"workload": name, "rows": rows, "k": k, "kernel": "a8w8_quantize", "ms_per_launch": ms,
+                    "wall_ms_per_launch": wall, "algorithmic_bytes": abytes, "gbs": abytes / ms / 1e6,
+                    "frac_hbm_peak": abytes / ms / 1e6 / PEAK_HBM_GBS,
+                    "timing": "best of 3 regions of K launches after 100 ms of warm-up"})
+    return out
+
+
 def cpu_baseline(name, inp, c_gpu, torch, budget_s=15.0):
     """Times the oracle (port of the reference's host GEMM: per-MAC software fp8 decode,
     OpenMP over (i, j), gemm_a8w8_blockscale_host.cc:66-90) on the first rows of the same
@@ -302,6 +332,7 @@ def main():
             others.append(r)
             del i2, c2
             torch.cuda.empty_cache()
+        others.extend(run_quantizers(torch, g, args.steps, args.warmup, args.seed + 2))
         line["other_workloads"] = others
     print(json.dumps(line))
 

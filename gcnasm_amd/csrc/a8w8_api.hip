@@ -378,6 +378,13 @@ int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream)
     return launch_status();
 }
 
+// the vectorised quantisers read 16 bytes per lane and write packed words
+static bool quant_vec_ok(const float* src, int rows, int k, int ld, const uint8_t* q, int q_align)
+{
+    return aligned16(src) && ld % 4 == 0 && k % 4 == 0 && ((uintptr_t)q & (uintptr_t)(q_align - 1)) == 0 &&
+           (long long)rows * k < (1ll << 31);
+}
+
 int a4w4_quantize_mx(const float* src, int rows, int k, int ld, uint8_t* q, uint8_t* scale, int tiled, void* hip_stream)
 {
     if (!src || !q || !scale) return A8W8_ERR_NULL_POINTER;
@@ -393,9 +400,15 @@ int a4w4_quantize_mx(const float* src, int rows, int k, int ld, uint8_t* q, uint
             const size_t dwords = mx_tiled_bytes(rows, k) / 4;
             hipLaunchKernelGGL(mx_tiled_fill_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0, s, (uint32_t*)scale, dwords);
         }
-        hipLaunchKernelGGL(quant_mxfp4_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+        if (quant_vec_ok(src, rows, k, ld, q, 4))
+            hipLaunchKernelGGL(quant_mxfp4_vec_kernel<true>, dim3((unsigned)((threads / 8 + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+        else
+            hipLaunchKernelGGL(quant_mxfp4_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
     } else {
-        hipLaunchKernelGGL(quant_mxfp4_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+        if (quant_vec_ok(src, rows, k, ld, q, 4))
+            hipLaunchKernelGGL(quant_mxfp4_vec_kernel<false>, dim3((unsigned)((threads / 8 + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+        else
+            hipLaunchKernelGGL(quant_mxfp4_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
     }
     return launch_status();
 }
@@ -530,22 +543,39 @@ int a8w8_quantize(const float* src, int rows, int k, int ld, uint8_t* q, void* s
             const long long total = (long long)rows * k;
             const unsigned grid = (unsigned)(total / 256 + 1 < 4096 ? total / 256 + 1 : 4096);
             hipLaunchKernelGGL(quant_tensor_clear_kernel, dim3(1), dim3(1), 0, s, (float*)scale);
-            hipLaunchKernelGGL(quant_tensor_amax_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, (float*)scale);
-            hipLaunchKernelGGL(quant_tensor_apply_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, q, (const float*)scale);
+            if (ld == k && total % 4 == 0 && aligned16(src) && ((uintptr_t)q & 3) == 0) {
+                const size_t units = (size_t)(total / 4);
+                const unsigned vgrid = (unsigned)(units / 1024 + 1 < 2048 ? units / 1024 + 1 : 2048);
+                hipLaunchKernelGGL(quant_tensor_amax_vec_kernel, dim3(vgrid), dim3(256), 0, s, (const float4*)src, units, (float*)scale);
+                hipLaunchKernelGGL(quant_tensor_apply_vec_kernel, dim3(vgrid), dim3(256), 0, s, (const float4*)src, units, (uint32_t*)q,
+                                   (const float*)scale);
+            } else {
+                hipLaunchKernelGGL(quant_tensor_amax_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, (float*)scale);
+                hipLaunchKernelGGL(quant_tensor_apply_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, q, (const float*)scale);
+            }
             hipLaunchKernelGGL(quant_tensor_finish_kernel, dim3(1), dim3(1), 0, s, (float*)scale);
             return launch_status();
         }
         case A8W8_SCALE_ROWCOL:
             if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-            hipLaunchKernelGGL(quant_rowwise_kernel, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
+            if (quant_vec_ok(src, rows, k, ld, q, 4) && k <= 8192)
+                hipLaunchKernelGGL(quant_rowwise_vec_kernel<true>, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
+            else if (quant_vec_ok(src, rows, k, ld, q, 4))
+                hipLaunchKernelGGL(quant_rowwise_vec_kernel<false>, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
+            else
+                hipLaunchKernelGGL(quant_rowwise_kernel, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
             return launch_status();
         case A8W8_SCALE_BLOCK_1x128_128x128:
             if (k % 128 != 0) return A8W8_ERR_BAD_GROUP;
             if (group_rows == 1) {
                 if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
                 const long long waves = (long long)rows * (k / 128);
-                hipLaunchKernelGGL(quant_1x128_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, src, rows, k,
-                                   ld, q, (float*)scale);
+                if (quant_vec_ok(src, rows, k, ld, q, 4))
+                    hipLaunchKernelGGL(quant_1x128_vec_kernel, dim3((unsigned)((waves + 8 * QUANT_1X128_GROUPS - 1) / (8 * QUANT_1X128_GROUPS))), dim3(256), 0, s, src, rows, k, ld, q,
+                                       (float*)scale);
+                else
+                    hipLaunchKernelGGL(quant_1x128_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, src, rows, k,
+                                       ld, q, (float*)scale);
                 return launch_status();
             }
             if (group_rows == 128) {
@@ -560,8 +590,12 @@ int a8w8_quantize(const float* src, int rows, int k, int ld, uint8_t* q, void* s
             if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
             if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
             const long long threads = (long long)rows * k;
-            hipLaunchKernelGGL(quant_mx_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k,
-                               ld, q, (uint8_t*)scale);
+            if (quant_vec_ok(src, rows, k, ld, q, 4))
+                hipLaunchKernelGGL(quant_mx_vec_kernel<false>, dim3((unsigned)((threads / (4 * QUANT_MX_CHUNKS) + 255) / 256)), dim3(256), 0, s, src,
+                                   rows, k, ld, q, (uint8_t*)scale);
+            else
+                hipLaunchKernelGGL(quant_mx_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k,
+                                   ld, q, (uint8_t*)scale);
             return launch_status();
         }
         case A8W8_SCALE_MX_E8M0_TILED: {
@@ -574,8 +608,12 @@ int a8w8_quantize(const float* src, int rows, int k, int ld, uint8_t* q, void* s
                 hipLaunchKernelGGL(mx_tiled_fill_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0, s,
                                    (uint32_t*)scale, dwords);
             }
-            hipLaunchKernelGGL(quant_mx_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows,
-                               k, ld, q, (uint8_t*)scale);
+            if (quant_vec_ok(src, rows, k, ld, q, 4))
+                hipLaunchKernelGGL(quant_mx_vec_kernel<true>, dim3((unsigned)((threads / (4 * QUANT_MX_CHUNKS) + 255) / 256)), dim3(256), 0, s, src,
+                                   rows, k, ld, q, (uint8_t*)scale);
+            else
+                hipLaunchKernelGGL(quant_mx_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows,
+                                   k, ld, q, (uint8_t*)scale);
             return launch_status();
         }
         default:

@@ -292,6 +292,228 @@ __global__ void __launch_bounds__(256) quant_mxfp4_kernel(const float* src, int 
     if ((l & 1) == 0) q[(long long)row * (k >> 1) + ((g * 32 + l) >> 1)] = (uint8_t)(code | (hi << 4));
 }
 
+// ------------------------------------------------------------ vectorised quantisers
+// The kernels above move one element per thread (4-byte loads, 1-byte stores).  When rows are
+// 16-byte aligned (src, ld % 4 == 0, k % 4 == 0) the kernels below do the same arithmetic on four
+// elements per thread per chunk: 16-byte loads, one packed store, same bits out.
+A8W8_DEV uint32_t pack4_e4m3(float a, float b, float c, float d)
+{
+    uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    return __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+}
+A8W8_DEV int mx_block_exponent(float amax, float top)
+{
+    const float t = __fdiv_rn(amax, top);
+    int e = -127;
+    if (t > 0.f) {
+        int ex;
+        const float f = frexpf(t, &ex);          // t = f * 2^ex, f in [0.5, 1)
+        e = (f == 0.5f) ? ex - 1 : ex;
+        e = max(-127, min(127, e));
+    }
+    return e;
+}
+
+// MX E4M3 with one E8M0 exponent per 32 elements.  A wave takes 1024 consecutive elements of the
+// flattened [rows, k] array as four chunks of 256: lane l owns elements 4l..4l+3 of each chunk, eight
+// lanes share a block.  Every load and store instruction of a wave covers one contiguous run of memory;
+// all loads are issued before any chunk is processed.
+constexpr int QUANT_MX_CHUNKS = 4;
+template <bool TILED>
+__global__ void __launch_bounds__(256) quant_mx_vec_kernel(const float* __restrict__ src, int rows, int k, int ld,
+                                                           uint8_t* __restrict__ q, uint8_t* __restrict__ scale)
+{
+    const unsigned total = (unsigned)rows * (unsigned)k;            // < 2^31 (checked by the host)
+    const unsigned wave = (blockIdx.x * 256u + threadIdx.x) >> 6;
+    const unsigned lane = threadIdx.x & 63;
+    const int blocks = k >> 5;
+    constexpr int CH = QUANT_MX_CHUNKS;
+    unsigned row[CH], col[CH];
+    bool live[CH];
+    float4 v[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const unsigned e0 = wave * (256u * CH) + c * 256u + lane * 4u;
+        live[c] = e0 < total;
+        row[c] = live[c] ? e0 / (unsigned)k : 0u;
+        col[c] = live[c] ? e0 % (unsigned)k : 0u;
+        v[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live[c]) v[c] = *(const float4*)(src + (size_t)row[c] * ld + col[c]);
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        float amax = fmaxf(fmaxf(fabsf(v[c].x), fabsf(v[c].y)), fmaxf(fabsf(v[c].z), fabsf(v[c].w)));
+#pragma unroll
+        for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        const int e = mx_block_exponent(amax, 448.0f);
+        if (!live[c]) continue;
+        if ((lane & 7) == 0) {
+            const int g = (int)(col[c] >> 5);
+            scale[TILED ? mx_tiled_index(rows, (int)row[c], g) : (size_t)row[c] * blocks + g] = (uint8_t)(e + 127);
+        }
+        *(uint32_t*)(q + (size_t)row[c] * k + col[c]) =
+            pack4_e4m3(ldexpf(v[c].x, -e), ldexpf(v[c].y, -e), ldexpf(v[c].z, -e), ldexpf(v[c].w, -e));
+    }
+}
+
+// MXFP4 (packed E2M1): lane l owns eight consecutive elements (two 16-byte loads, one 4-byte store),
+// four lanes share a block, a wave takes 512 consecutive elements.
+template <bool TILED>
+__global__ void __launch_bounds__(256) quant_mxfp4_vec_kernel(const float* __restrict__ src, int rows, int k, int ld,
+                                                              uint8_t* __restrict__ q, uint8_t* __restrict__ scale)
+{
+    const unsigned total = (unsigned)rows * (unsigned)k;            // < 2^31 (checked by the host)
+    const unsigned e0 = (blockIdx.x * 256u + threadIdx.x) * 8u;
+    const bool live = e0 < total;
+    const unsigned row = live ? e0 / (unsigned)k : 0u, col = live ? e0 % (unsigned)k : 0u;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+    if (live) {
+        const float4* p = (const float4*)(src + (size_t)row * ld + col);
+        a = p[0];
+        b = p[1];
+    }
+    float amax = fmaxf(fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))),
+                       fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
+#pragma unroll
+    for (int off = 2; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const int e = mx_block_exponent(amax, 6.0f);
+    if (!live) return;
+    if ((threadIdx.x & 3) == 0) {
+        const int g = (int)(col >> 5);
+        scale[TILED ? mx_tiled_index(rows, (int)row, g) : (size_t)row * (k >> 5) + g] = (uint8_t)(e + 127);
+    }
+    const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    unsigned w = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w |= e2m1_encode(ldexpf(x[i], -e)) << (4 * i);     // even K in the low nibble
+    *(uint32_t*)(q + (size_t)row * (k >> 1) + (col >> 1)) = w;
+}
+
+// per-row scale, one workgroup per row.  HOLD: the row has at most 8192 elements and stays in registers
+// between the amax pass and the quantisation (one read of the input); otherwise it is read twice.
+template <bool HOLD>
+__global__ void __launch_bounds__(256) quant_rowwise_vec_kernel(const float* __restrict__ src, int k, int ld,
+                                                                uint8_t* __restrict__ q, float* __restrict__ scale)
+{
+    __shared__ float part[4];
+    const int row = blockIdx.x;
+    const float* x = src + (size_t)row * ld;
+    float4 held[8];
+    float amax = 0.f;
+    if constexpr (HOLD) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = threadIdx.x * 4 + u * 1024;
+            held[u] = i < k ? *(const float4*)(x + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(held[u].x), fabsf(held[u].y)), fmaxf(fabsf(held[u].z), fabsf(held[u].w))));
+        }
+    } else {
+        for (int i = threadIdx.x * 4; i < k; i += 1024) {
+            const float4 v = *(const float4*)(x + i);
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        }
+    }
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    const float s = amax > 0.f ? __fdiv_rn(amax, 448.0f) : 1.0f;   // an all-zero group keeps scale 1
+    if (threadIdx.x == 0) scale[row] = s;
+    if constexpr (HOLD) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = threadIdx.x * 4 + u * 1024;
+            if (i < k)
+                *(uint32_t*)(q + (size_t)row * k + i) = pack4_e4m3(__fdiv_rn(held[u].x, s), __fdiv_rn(held[u].y, s),
+                                                                   __fdiv_rn(held[u].z, s), __fdiv_rn(held[u].w, s));
+        }
+    } else {
+        for (int i = threadIdx.x * 4; i < k; i += 1024) {
+            const float4 v = *(const float4*)(x + i);
+            *(uint32_t*)(q + (size_t)row * k + i) =
+                pack4_e4m3(__fdiv_rn(v.x, s), __fdiv_rn(v.y, s), __fdiv_rn(v.z, s), __fdiv_rn(v.w, s));
+        }
+    }
+}
+
+// 1 x 128 blocks: 32 lanes per (row, 128-group); a half wave takes four consecutive groups, loads first.
+// Scale stored [k/128][rows].
+constexpr int QUANT_1X128_GROUPS = 4;
+__global__ void __launch_bounds__(256) quant_1x128_vec_kernel(const float* __restrict__ src, int rows, int k, int ld,
+                                                              uint8_t* __restrict__ q, float* __restrict__ scale)
+{
+    constexpr int G = QUANT_1X128_GROUPS;
+    const int groups = k >> 7;
+    const long long total = (long long)rows * groups;
+    const long long w0 = (((long long)blockIdx.x * 256 + threadIdx.x) >> 5) * G;
+    const int l = threadIdx.x & 31;
+    float4 v[G];
+    int row[G], g[G];
+    bool live[G];
+#pragma unroll
+    for (int u = 0; u < G; ++u) {
+        live[u] = w0 + u < total;
+        row[u] = live[u] ? (int)((w0 + u) / groups) : 0;
+        g[u] = live[u] ? (int)((w0 + u) % groups) : 0;
+        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live[u]) v[u] = *(const float4*)(src + (size_t)row[u] * ld + g[u] * 128 + 4 * l);
+    }
+#pragma unroll
+    for (int u = 0; u < G; ++u) {
+        float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        if (!live[u]) continue;
+        const float s = amax > 0.f ? __fdiv_rn(amax, 448.0f) : 1.0f;   // an all-zero group keeps scale 1
+        if (l == 0) scale[(size_t)g[u] * rows + row[u]] = s;
+        *(uint32_t*)(q + (size_t)row[u] * k + g[u] * 128 + 4 * l) =
+            pack4_e4m3(__fdiv_rn(v[u].x, s), __fdiv_rn(v[u].y, s), __fdiv_rn(v[u].z, s), __fdiv_rn(v[u].w, s));
+    }
+}
+
+// per-tensor scale over a contiguous array (ld == k): the amax and apply passes on 16-byte units, four
+// units per thread and iteration (loads first)
+__global__ void __launch_bounds__(256) quant_tensor_amax_vec_kernel(const float4* __restrict__ src, size_t units, float* scale)
+{
+    __shared__ float part[4];
+    float amax = 0.f;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < units; i += 4 * stride) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = i + u * stride < units ? src[i + u * stride] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w))));
+    }
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+        // thousands of atomics on one address take longer than the pass over the data: only a
+        // workgroup that would raise the maximum sends one
+        if (__float_as_uint(amax) > __hip_atomic_load((unsigned int*)scale, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+            atomicMax((unsigned int*)scale, __float_as_uint(amax));
+    }
+}
+__global__ void __launch_bounds__(256) quant_tensor_apply_vec_kernel(const float4* __restrict__ src, size_t units,
+                                                                     uint32_t* __restrict__ q, const float* __restrict__ amax_slot)
+{
+    const float amax = *amax_slot;
+    const float s = amax > 0.f ? __fdiv_rn(amax, 448.0f) : 1.0f;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < units; i += 4 * stride) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = i + u * stride < units ? src[i + u * stride] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (i + u * stride < units)
+                q[i + u * stride] = pack4_e4m3(__fdiv_rn(v[u].x, s), __fdiv_rn(v[u].y, s), __fdiv_rn(v[u].z, s), __fdiv_rn(v[u].w, s));
+    }
+}
+
 // One launch for one or two scale arrays (the A-side and the B-side scales of a GEMM).  A group of
 // 64 threads handles one 1 KiB unit (64 rows x 16 K blocks): thread r copies the 16 bytes of row r
 // into LDS, then thread t gathers and writes bytes 16t..16t+15 of the unit.  256 threads = 4 units.

@@ -108,3 +108,31 @@ def test_quantize_then_gemm_matches_oracle_pipeline(orc):
         ob, osb = orc.quantize(b, omode, gb)
         ref = orc.gemm_ref(oa, ob, osa, osb, omode)
         assert (np.abs(c - ref) <= 1e-2 * np.abs(ref) + 1e-2).all(), mode
+
+
+def test_vector_and_scalar_kernels_agree_with_the_oracle_on_views(orc):
+    """16-byte aligned rows take the vectorised kernels (four or eight elements per thread), anything
+    else the one-element-per-thread kernels: an aligned view with padded rows, a view that starts four
+    bytes into its rows, and a row longer than a workgroup holds in registers."""
+    rows, k = 70, 512
+    big = _x(rows, 2 * k + 32, 123)
+    views = {"padded rows": (slice(None), slice(0, k)), "offset by one element": (slice(None), slice(1, 1 + k))}
+    for name, (r, c) in views.items():
+        want = np.ascontiguousarray(big[r, c])
+        xv = dev(big)[r, c]
+        assert (xv.data_ptr() % 16 == 0) == (name == "padded rows")
+        for mode, gr in ((g.TENSOR, 1), (g.ROWCOL, 1), (g.BLOCK, 1), (g.MX, 1), (g.MX_TILED, 1)):
+            q, s = g.quantize(xv, mode, gr)
+            qr, sr = orc.quantize(want, orc.MX if mode == g.MX_TILED else mode, gr)
+            assert (q.cpu().numpy() == qr).all(), (name, mode)
+            if mode == g.MX_TILED:
+                assert (s.cpu().numpy() == orc.mx_tile_scales(sr)).all(), (name, mode)
+            else:
+                assert (s.cpu().numpy().view(np.uint8) == sr.view(np.uint8)).all(), (name, mode)
+        q4, s4 = g.quantize_mxfp4(xv)
+        qr4, sr4 = orc.quantize_mxfp4(want)
+        assert (q4.cpu().numpy() == qr4).all() and (s4.cpu().numpy() == sr4).all(), name
+    long_rows = _x(5, 16384, 124)
+    q, s = _run(long_rows, g.ROWCOL)
+    qr, sr = orc.quantize(long_rows, orc.ROWCOL)
+    assert (q == qr).all() and (s.view(np.uint32) == sr.view(np.uint32)).all()
