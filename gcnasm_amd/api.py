@@ -147,10 +147,15 @@ def mx_tiled_bytes(rows, k):
 
 
 def _out(c, shape, c_dtype, device):
+    """The output tensor and its C type code: a caller's tensor decides the type (bf16 or fp32 only)."""
     import torch
     if c is None:
-        c = torch.empty(shape, dtype=torch.bfloat16 if c_dtype == BF16 else torch.float32, device=device)
-    return c
+        return torch.empty(shape, dtype=torch.bfloat16 if c_dtype == BF16 else torch.float32, device=device), c_dtype
+    if c.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"output tensor must be bfloat16 or float32, got {c.dtype}")
+    if tuple(c.shape) != tuple(shape):
+        raise ValueError(f"output tensor has shape {tuple(c.shape)}, expected {tuple(shape)}")
+    return c, (BF16 if c.dtype == torch.bfloat16 else FP32)
 
 
 def _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, b_preshuffled, n=None):
@@ -159,7 +164,7 @@ def _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, b_preshuffled, n=
     if n is None:
         n = b.shape[-2]
     shape = (batch, m, n) if a.dim() == 3 else (m, n)
-    c = _out(c, shape, c_dtype, a.device)
+    c, c_dtype = _out(c, shape, c_dtype, a.device)
     g = raw_gemm_args(a.data_ptr(), b.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, scale_mode,
                       c_dtype, batch, stride_a=a.stride(-2), stride_b=(k if b_preshuffled else b.stride(-2)),
                       stride_c=c.stride(-2), b_preshuffled=b_preshuffled)
@@ -211,7 +216,7 @@ def quantize_mxfp4(x, tiled=False):
 def gemm_a4w4(a, b, sfa, sfb, scale_mode=MX_TILED, c=None, c_dtype=BF16):
     """MXFP4 GEMM through a4w4_gemm: a [M, K/2], b [N, K/2] packed E2M1 (uint8 on the GPU)."""
     m, n, k = a.shape[-2], b.shape[-2], a.shape[-1] * 2
-    c = _out(c, (m, n), c_dtype, a.device)
+    c, c_dtype = _out(c, (m, n), c_dtype, a.device)
     g = raw_gemm_args(a.data_ptr(), b.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, scale_mode, c_dtype,
                       stride_a=a.stride(-2) * 2, stride_b=b.stride(-2) * 2, stride_c=c.stride(-2))
     _check(lib().a4w4_gemm(ctypes.byref(g), _stream()), "a4w4_gemm")

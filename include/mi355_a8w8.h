@@ -101,7 +101,8 @@ A8W8_API int a16w16_gemm(const a8w8_gemm_args* args, void* hip_stream);
 
 /* The bf16 flat GEMM (flatmm_a16w16_gfx950, opus_fmm/README.md:10,51-57; source absent): A [batch, m, k]
  * bf16 with m <= 64, B bf16 pre-shuffled as a byte matrix -- a8w8_preshuffle_b[_device](b, out, n, 2*k) --
- * n % 16 == 0, k % 32 == 0, no scales, bf16 or fp32 C.  Same streaming kernel as a8w8_flatmm. */
+ * n % 16 == 0, k % 32 == 0, a, b and the rows of A 16-byte aligned, no scales, bf16 or fp32 C.  Same
+ * streaming kernel as a8w8_flatmm. */
 A8W8_API int a16w16_flatmm(const a8w8_gemm_args* args, void* hip_stream);
 
 /* MXFP4 (OCP MX: E2M1 elements, two per byte with the even K index in the low nibble, one E8M0 scale per
@@ -124,8 +125,8 @@ A8W8_API int a8w8_gemm_blockscale(const a8w8_gemm_args* args, void* hip_stream);
 
 /* Skinny-M GEMM over pre-shuffled weights (the flatmm_a8w8_gfx950 program listed at
  * opus_fmm/README.md:9, built by opus_fmm/rebuild.sh:3-13).  Requires b_preshuffled != 0,
- * scale_mode ROWCOL or TENSOR, m <= 64, n % 16 == 0, k % 64 == 0.  B is streamed once with
- * 16-byte non-temporal loads. */
+ * scale_mode ROWCOL or TENSOR, m <= 64, n % 16 == 0, k % 64 == 0, a, b and the rows of A 16-byte
+ * aligned (A8W8_ERR_MISALIGNED otherwise).  B is streamed once with 16-byte non-temporal loads. */
 A8W8_API int a8w8_flatmm(const a8w8_gemm_args* args, void* hip_stream);
 
 /* Host-side weight pre-shuffle, row-major b[n][k] -> Bshuf[n/16][k/64][4][16][16 bytes]:
