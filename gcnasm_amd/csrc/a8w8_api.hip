@@ -3,12 +3,14 @@
 
 #include <hip/hip_runtime.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "cvt.hpp"
 #include "flatmm.hpp"
 #include "gemm_general.hpp"
 #include "gemm_persist.hpp"
+#include "gemm_small.hpp"
 #include "gemm_tile.hpp"
 #include "gemm_wide.hpp"
 
@@ -127,6 +129,52 @@ bool wide_ok(const a8w8_gemm_args* g)
 template <int MODE, int CDT>
 int launch_general(const GemmParams& p, int batch, hipStream_t stream);
 
+int num_cus()
+{
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    return g_num_cus[dev & 63] > 0 ? g_num_cus[dev & 63] : 256;
+}
+
+// 128 x 128 tiles (fp32-scale modes) when 256 x 256 tiles would leave most compute units without work.
+// Measured crossover on 256 compute units: the block-scale mode gains up to 128 tiles of 256 x 256 (2.2x at
+// 16 tiles, +14% at 100, even at 128), per-tensor and row/col up to 64 (1.6x there, -3% at 81) -- their
+// 256-tile kernel is the faster one.  The scale loads of the block mode use 32-bit byte offsets.
+bool small_ok(const a8w8_gemm_args* g)
+{
+    const bool block = g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128;
+    if (!block && g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_ROWCOL) return false;
+    const long long items256 = (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN);
+    if (items256 * (block ? 2 : 4) > num_cus()) return false;
+    if (block && (long long)(g->k / BK) * g->stride_sfa * 4 >= (1ll << 31)) return false;
+    return true;
+}
+
+template <int MODE, int CDT>
+int launch_small(const GemmParams& p, int batch, hipStream_t stream)
+{
+    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_BF16) {
+        static bool attr_set[64];
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        auto kern = gemm_a8w8_tile128<MODE, CDT>;
+        constexpr int lds_bytes = small_lds_bytes(MODE);
+        if (!attr_set[dev & 63]) {
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+                return A8W8_ERR_LAUNCH;
+            attr_set[dev & 63] = true;
+        }
+        GemmParams q = p;
+        q.tiles_m = (p.m + SM_BM - 1) / SM_BM;
+        q.tiles_n = (p.n + SM_BN - 1) / SM_BN;
+        dim3 grid((unsigned)(q.tiles_m * q.tiles_n), 1, (unsigned)batch);
+        hipLaunchKernelGGL(kern, grid, dim3(SM_THREADS), lds_bytes, stream, q);
+        return launch_status();
+    } else {
+        return A8W8_ERR_BAD_MODE;
+    }
+}
+
 template <int MODE, int CDT>
 int launch_tiled(const GemmParams& p, int batch, hipStream_t stream)
 {
@@ -243,6 +291,10 @@ int dispatch_wide(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
 {
     A8W8_DISPATCH(launch_wide, g->scale_mode, g->c_dtype, p, g->batch, s)
 }
+int dispatch_small(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
+{
+    A8W8_DISPATCH(launch_small, g->scale_mode, g->c_dtype, p, g->batch, s)
+}
 int dispatch_general(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
 {
     A8W8_DISPATCH(launch_general, g->scale_mode, g->c_dtype, p, g->batch, s)
@@ -286,6 +338,7 @@ int a8w8_gemm(const a8w8_gemm_args* g, void* hip_stream)
     const GemmParams p = make_params(g);
     hipStream_t s = (hipStream_t)hip_stream;
     if (!tiled_ok(g)) return dispatch_general(g, p, s);
+    if (small_ok(g)) return dispatch_small(g, p, s);
     if (wide_ok(g)) return dispatch_wide(g, p, s);
     return persist_ok(g) ? dispatch_persist(g, p, s) : dispatch_tiled(g, p, s);
 }
@@ -314,6 +367,9 @@ int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
     if (fits && tiled_ok(&bytes) && persist_ok(&bytes)) {
         GemmParams p = make_params(&bytes);
         p.sfa = p.sfb = nullptr;
+        if (small_ok(&bytes))            // few tiles: 128 x 128 ones
+            return g->c_dtype == A8W8_C_BF16 ? launch_small<MODE_BF16, C_BF16>(p, g->batch, s)
+                                             : launch_small<MODE_BF16, C_FP32>(p, g->batch, s);
         if ((bytes.k / BK) % 2 == 0)     // an even number of K steps: the four-wave kernel
             return g->c_dtype == A8W8_C_BF16 ? launch_wide<MODE_BF16, C_BF16>(p, g->batch, s)
                                              : launch_wide<MODE_BF16, C_FP32>(p, g->batch, s);
@@ -769,6 +825,7 @@ const char* a8w8_kernel_name(const a8w8_gemm_args* g)
     if (g->b_preshuffled) return validate_flat(g) == A8W8_OK ? "flatmm_a8w8" : nullptr;
     if (validate_common(g) != A8W8_OK) return nullptr;
     if (!tiled_ok(g)) return "gemm_a8w8_general";
+    if (small_ok(g)) return "gemm_a8w8_tile128";
     if (wide_ok(g)) return "gemm_a8w8_wide";
     if (persist_ok(g)) return "gemm_a8w8_persist";
     return g->scale_mode == A8W8_SCALE_MX_E8M0_TILED ? "gemm_a8w8_general" : "gemm_a8w8_tile256";

@@ -80,6 +80,10 @@ A8W8_DEV void load_to_lds_16(__amdgpu_buffer_rsrc_t rsrc, A8W8_LDS void* lds_bas
 #define A8W8_STORE_C(ptr, val) (*(ptr) = (val))
 #endif
 
+// Barrier without the wait for every outstanding load that __syncthreads() implies: the pipelined kernels
+// keep direct-to-LDS loads in flight across it and place their own s_waitcnt.
+#define A8W8_RAW_BARRIER() asm volatile("s_barrier" ::: "memory")
+
 A8W8_DEV int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // fp32 -> bf16 bits, round to nearest even, through the hardware convert.

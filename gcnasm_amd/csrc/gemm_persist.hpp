@@ -35,7 +35,6 @@ constexpr int PERSIST_LDS_BYTES_MX = GEMM_LDS_BYTES_MX;
 constexpr int ROWCOL_SCALE_BYTES = (BM + BN) * 4;
 constexpr int PERSIST_LDS_BYTES_ROWCOL = GEMM_LDS_BYTES + 2 * ROWCOL_SCALE_BYTES;
 
-#define A8W8_RAW_BARRIER() asm volatile("s_barrier" ::: "memory")
 // How many of the next step's four A fragments (plus the first B fragment) are fetched from LDS in
 // the shadow of the current step's last MFMA group.  Bounded by the registers each mode has left:
 // a spill inside the K loop is reloaded behind a wait for every load in flight.

@@ -1,0 +1,241 @@
+// Dense A8W8 GEMM for problems too small to fill the chip with 256 x 256 tiles: 128 x 128 x 128 tile,
+// 4 waves (2 along M x 2 along N), each wave owning a 64 x 64 block of C as 4 x 4 MFMA tiles of
+// 16 x 16 x 128.  A quarter of the work per workgroup means four times as many workgroups, and a
+// problem of this size is bound by latency (first loads, the K loop's dependent steps, the C stores of
+// one compute unit), not by the matrix cores.
+//
+// Data path as in the 256-tile kernels: 16-byte direct-to-LDS loads, 128-byte LDS rows whose 16-byte
+// slots are XOR-swizzled with (row & 7), operand roles swapped so that a lane ends up with
+// C[m = lane%16][n = 4*(lane/16) .. +3].  Four LDS stages of 32 KiB: the loads of K step s+3 are issued
+// when step s begins, one raw barrier per step.  Block scales (fp32 per row and K step for A, one per
+// 128 x 128 block for B) ride in the same pipeline: each stage carries its step's 128 row scales and
+// the block's B scale, fetched by one extra direct-to-LDS load per wave, so that the loop's wait counts
+// stay fixed and no global load has to be waited for inside a step.
+#pragma once
+#include "gemm_tile.hpp"
+
+namespace a8w8 {
+
+constexpr int SM_BM = 128, SM_BN = 128;
+constexpr int SM_THREADS = 256;
+constexpr int SM_STAGES = 4;
+constexpr int SM_STAGE_BYTES = (SM_BM + SM_BN) * BK;   // 32768
+constexpr int SM_SCALE_BYTES = 1024;                   // block mode, per stage: 128 A-row scales, the B scale at +512 and +768
+constexpr int SM_TM = 4, SM_TN = 4;                    // MFMA tiles per wave
+constexpr int small_lds_bytes(int mode)
+{
+    return SM_STAGES * (SM_STAGE_BYTES + (mode == MODE_BLOCK ? SM_SCALE_BYTES : 0));
+}
+
+// p.tiles_m / p.tiles_n count 128 x 128 tiles here; grid = (tiles, 1, batch).  The launch bound asks for a
+// 256-register budget: with 512 the compiler parks the block mode's partial tiles in accumulation registers
+// and copies each value back before its multiply-add.
+template <int MODE, int CDT>
+__global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
+{
+    static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_BF16,
+                  "fp32-scale modes and bf16 operands (byte rows of 2k columns, no scales)");
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = wave_uniform(tid >> 6);
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int batch = blockIdx.z;
+    const int r16 = lane & 15, g = lane >> 4;
+
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * SM_BM, n0 = tile_n * SM_BN;
+    const int nk = p.k / BK;
+
+    const uint8_t* a_base = p.a + (long long)batch * p.a_batch;
+    const uint8_t* b_base = p.b + (long long)batch * p.b_batch;
+    const float* sfa_f = (const float*)p.sfa + (long long)batch * p.sfa_batch;
+    const float* sfb_f = (const float*)p.sfb + (long long)batch * p.sfb_batch;
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(a_base, (uint32_t)(p.m - 1) * p.lda + p.k);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(b_base, (uint32_t)(p.n - 1) * p.ldb + p.k);
+
+    // ---- global -> LDS.  A stage holds 16 A chunks then 16 B chunks of 1 KiB (8 rows x 128 B); wave w
+    // fills chunks w, w+4, w+8, w+12 of each matrix.  Lane i of a load lands on row i/8, slot i%8 of its
+    // chunk and therefore fetches K-piece slot ^ (row & 7) = (i%8) ^ (i/8).
+    const int ld_row = wave * 8 + (lane >> 3);
+    const int ld_piece16 = ((lane & 7) ^ (lane >> 3)) * 16;
+    int voff_a[4], voff_b[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        voff_a[j] = min(m0 + ld_row + 32 * j, p.m - 1) * p.lda + ld_piece16;
+        voff_b[j] = min(n0 + ld_row + 32 * j, p.n - 1) * p.ldb + ld_piece16;
+    }
+    // block mode: waves 0 and 1 fetch the step's 128 A-row scales (64 each), waves 2 and 3 the B scale
+    // of the tile's 128 x 128 block (every lane the same dword: the stage's copy at +512 is the one read)
+    constexpr int LOADS_PER_STAGE = 8 + (MODE == MODE_BLOCK ? 1 : 0);
+    __amdgpu_buffer_rsrc_t rsrc_sf = rsrc_a;
+    int voff_sf = 0, sf_step_bytes = 0;
+    if constexpr (MODE == MODE_BLOCK) {
+        if (wave < 2) {
+            rsrc_sf = make_rsrc(sfa_f, (uint32_t)((nk - 1) * p.stride_sfa + p.m) * 4u);
+            voff_sf = min(m0 + wave * 64 + lane, p.m - 1) * 4;
+            sf_step_bytes = p.stride_sfa * 4;
+        } else {
+            rsrc_sf = make_rsrc(sfb_f + (long long)(n0 >> 7) * p.stride_sfb, (uint32_t)nk * 4u);
+            voff_sf = 0;
+            sf_step_bytes = 4;
+        }
+    }
+    auto issue_stage = [&](int stage, int kstep) __attribute__((always_inline)) {
+        kstep = min(kstep, nk - 1);         // past the end: reload the last step into a stage nobody reads (fixed wait counts)
+        A8W8_LDS char* s = (A8W8_LDS char*)smem + stage * SM_STAGE_BYTES + wave * 1024;
+        const int koff = kstep * BK;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_a, s + j * 4096, voff_a[j], koff);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_b, s + SM_BM * BK + j * 4096, voff_b[j], koff);
+        if constexpr (MODE == MODE_BLOCK) {
+            A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 256;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sf, sc, 4, voff_sf, kstep * sf_step_bytes, 0, 0);
+        }
+    };
+
+    // ---- LDS -> registers: a lane reads K-pieces g and g+4 of tile row r16; slot = piece ^ (row & 7), and
+    // row & 7 = lane & 7 for every tile
+    int rd_a[2], rd_b[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int slot = (g + 4 * h) ^ (lane & 7);
+        rd_a[h] = (wave_m * 64 + r16) * BK + (slot << 4);
+        rd_b[h] = SM_BM * BK + (wave_n * 64 + r16) * BK + (slot << 4);
+    }
+    auto read_frag = [&](int stage, const int (&base)[2], int t) __attribute__((always_inline)) -> v8i {
+        const char* s = smem + stage * SM_STAGE_BYTES + t * (16 * BK);
+        const v4i lo = *(const v4i*)(s + base[0]);
+        const v4i hi = *(const v4i*)(s + base[1]);
+        return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    };
+
+    const int cm_base = m0 + wave_m * 64 + r16;          // + 16 * i
+    const int cn_base = n0 + wave_n * 64 + 4 * g;        // + 16 * j + e
+
+    v4f acc[SM_TM][SM_TN];
+#pragma unroll
+    for (int i = 0; i < SM_TM; ++i)
+#pragma unroll
+        for (int j = 0; j < SM_TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    issue_stage(0, 0);
+    issue_stage(1, 1);
+    issue_stage(2, 2);
+
+    for (int ks = 0; ks < nk; ++ks) {
+        const int cur = ks & (SM_STAGES - 1);
+        // this wave's loads of stage `cur` have landed once at most the two younger stages are in flight
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LOADS_PER_STAGE) : "memory");
+        A8W8_RAW_BARRIER();                 // ... everyone's have; and everyone is done reading the stage of step ks-1
+        issue_stage((ks + 3) & (SM_STAGES - 1), ks + 3);
+
+        v8i fa[SM_TM], fb[2];
+#pragma unroll
+        for (int t = 0; t < SM_TM; ++t) fa[t] = read_frag(cur, rd_a, t);
+        fb[0] = read_frag(cur, rd_b, 0);
+        if constexpr (MODE == MODE_BLOCK) {
+            const float* sc = (const float*)(smem + SM_STAGES * SM_STAGE_BYTES + cur * SM_SCALE_BYTES);
+            const float sb = sc[128];
+            float blk_s[SM_TM];
+#pragma unroll
+            for (int t = 0; t < SM_TM; ++t) blk_s[t] = sc[wave_m * 64 + 16 * t + r16] * sb;
+            // acc += part * (sfa * sfb); the multiply-adds trail the MFMAs by BLK_LAG tiles so that they never
+            // wait on a matrix-core result that is still in flight
+            constexpr int BLK_LAG = 4;
+            v4f part[BLK_LAG + 1];
+#pragma unroll
+            for (int t = 0; t < SM_TM * SM_TN + BLK_LAG; ++t) {
+                if (t < SM_TM * SM_TN) {
+                    const int j = t / SM_TM, i = t % SM_TM;
+                    if (i == 0 && j + 1 < SM_TN) fb[(j + 1) & 1] = read_frag(cur, rd_b, j + 1);
+                    part[t % (BLK_LAG + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                        fb[j & 1], fa[i], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);   // keep the lag: the scheduler would pull the FMAs up
+                if (t >= BLK_LAG) {
+                    const int u = t - BLK_LAG;
+                    acc[u % SM_TM][u / SM_TM] += part[u % (BLK_LAG + 1)] * blk_s[u % SM_TM];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < SM_TN; ++j) {
+                if (j + 1 < SM_TN) fb[(j + 1) & 1] = read_frag(cur, rd_b, j + 1);
+                if constexpr (MODE == MODE_BF16) {
+                    // a 128-byte row is 64 bf16: the fragment's two 16-byte halves feed one 16x16x32 MFMA each (both
+                    // operands split K the same way); first halves for all four tiles, then second halves:
+                    // back-to-back MFMAs on one accumulator stall
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+#pragma unroll
+                        for (int i = 0; i < SM_TM; ++i) {
+                            const v8i& fbj = fb[j & 1];
+                            const v4i bh = {fbj[4 * h], fbj[4 * h + 1], fbj[4 * h + 2], fbj[4 * h + 3]};
+                            const v4i ah = {fa[i][4 * h], fa[i][4 * h + 1], fa[i][4 * h + 2], fa[i][4 * h + 3]};
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, bh), __builtin_bit_cast(v8bf, ah),
+                                                                                acc[i][j], 0, 0, 0);
+                        }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < SM_TM; ++i)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j & 1], fa[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // ---- epilogue: dequantise in fp32, convert, store
+    float sa[SM_TM];
+    float ts = 1.f;
+    if constexpr (MODE == MODE_TENSOR) ts = sfa_f[0] * sfb_f[0];
+    if constexpr (MODE == MODE_ROWCOL) {
+#pragma unroll
+        for (int i = 0; i < SM_TM; ++i) sa[i] = sfa_f[min(cm_base + 16 * i, p.m - 1)];
+    }
+    char* c_base = (char*)p.c + (long long)batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
+    const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 7) == 0)
+                                        : ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 15) == 0);
+#pragma unroll
+    for (int j = 0; j < SM_TN; ++j) {
+        const int cn = cn_base + 16 * j;
+        v4f sb = v4f{1.f, 1.f, 1.f, 1.f};
+        if constexpr (MODE == MODE_ROWCOL) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sb[e] = sfb_f[min(cn + e, p.n - 1)];
+        }
+#pragma unroll
+        for (int i = 0; i < SM_TM; ++i) {
+            const int cm = cm_base + 16 * i;
+            v4f v = acc[i][j];
+            if constexpr (MODE == MODE_TENSOR) v *= ts;
+            if constexpr (MODE == MODE_ROWCOL) v *= sb * sa[i];
+            if (cm >= p.m) continue;
+            if constexpr (CDT == C_BF16) {
+                unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
+                if (vec_ok && cn + 3 < p.n) {
+                    A8W8_STORE_C((v4u16*)dst, (v4u16{bf16_bits(v.x), bf16_bits(v.y), bf16_bits(v.z), bf16_bits(v.w)}));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (cn + e < p.n) dst[e] = bf16_bits(v[e]);
+                }
+            } else {
+                float* dst = (float*)c_base + (long long)cm * p.ldc + cn;
+                if (vec_ok && cn + 3 < p.n) {
+                    A8W8_STORE_C((v4f*)dst, v);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (cn + e < p.n) dst[e] = v[e];
+                }
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct-to-LDS load may outlive the workgroup's LDS allocation
+}
+
+}  // namespace a8w8

@@ -74,13 +74,23 @@ def test_flatmm_preconditions():
 
 
 def test_kernel_selection():
-    assert g.kernel_name(_ok_args()) == "gemm_a8w8_persist"
-    assert g.kernel_name(_ok_args(mode=g.MX)) == "gemm_a8w8_persist"
+    big = dict(m=4096, n=4096)                       # 256 tiles of 256 x 256: enough for every compute unit
+    assert g.kernel_name(_ok_args(**big)) == "gemm_a8w8_persist"
+    assert g.kernel_name(_ok_args(mode=g.MX, **big)) == "gemm_a8w8_persist"
     # per-tensor, row/col and tiled-MX scales with an even number of K steps: the four-wave kernel
-    assert g.kernel_name(_ok_args(mode=g.ROWCOL)) == "gemm_a8w8_wide"
-    assert g.kernel_name(_ok_args(mode=g.TENSOR, k=1024)) == "gemm_a8w8_wide"
-    assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=384)) == "gemm_a8w8_persist"
-    assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=128)) == "gemm_a8w8_tile256"
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL, **big)) == "gemm_a8w8_wide"
+    assert g.kernel_name(_ok_args(mode=g.TENSOR, k=1024, **big)) == "gemm_a8w8_wide"
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=384, **big)) == "gemm_a8w8_persist"
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=128, **big)) == "gemm_a8w8_tile256"
+    # fp32-scale modes whose 256 x 256 tiles would occupy at most half of the compute units: 128 x 128 tiles
+    assert g.kernel_name(_ok_args()) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL, m=1024, n=2048, k=128)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(mode=g.TENSOR, m=2048, n=2048)) == "gemm_a8w8_tile128"      # 64 tiles of 256 x 256
+    assert g.kernel_name(_ok_args(mode=g.TENSOR, m=2304, n=2048)) == "gemm_a8w8_wide"
+    assert g.kernel_name(_ok_args(mode=g.TENSOR, m=1024, n=1024, batch=5)) == "gemm_a8w8_wide"
+    assert g.kernel_name(_ok_args(m=2048, n=4096)) == "gemm_a8w8_tile128"                     # block scales: up to 128 tiles
+    assert g.kernel_name(_ok_args(m=2304, n=4096)) == "gemm_a8w8_persist"
+    assert g.kernel_name(_ok_args(mode=g.MX)) == "gemm_a8w8_persist"                  # MX scales stay on the 256 tiles
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=200)) == "gemm_a8w8_general"
     a = _ok_args(mode=g.ROWCOL)
     a.a = 0x1004

@@ -48,7 +48,8 @@ def test_random_case(case):
         k = max(128, k // 128 * 128)
     if mode == g.MX_TILED:
         k = max(128, k // 128 * 128)            # the tiled scale layout covers whole 128-wide K steps
-    batch = int(r.choice([1, 1, 2, 3]))
+    # small problems run on 128 x 128 tiles; many batch entries of a small shape put the same ragged tiles on the 256 x 256 kernels
+    batch = int(r.choice([1, 1, 2, 3, 70, 140])) if m <= 300 and n <= 300 else int(r.choice([1, 1, 2, 3]))
     c_dtype = [g.BF16, g.FP32][int(r.integers(0, 2))]
     a = r.integers(-4, 5, (batch, m, k)).astype(np.float32)
     b = r.integers(-4, 5, (batch, n, k)).astype(np.float32)
