@@ -136,16 +136,17 @@ int num_cus()
     return g_num_cus[dev & 63] > 0 ? g_num_cus[dev & 63] : 256;
 }
 
-// 128 x 128 tiles (fp32-scale modes) when 256 x 256 tiles would leave most compute units without work.
-// Measured crossover on 256 compute units: the block-scale mode gains up to 128 tiles of 256 x 256 (2.2x at
-// 16 tiles, +14% at 100, even at 128), per-tensor and row/col up to 64 (1.6x there, -3% at 81) -- their
-// 256-tile kernel is the faster one.  The scale loads of the block mode use 32-bit byte offsets.
+// 128 x 128 tiles when 256 x 256 tiles would leave most compute units without work.  Measured crossover on
+// 256 compute units: block scales and row-major MX scales (eight-wave kernel otherwise) gain up to 128 tiles of
+// 256 x 256 (2.2x at 16 tiles, +14% at 100, even at 128); per-tensor, row/col and tiled MX (four-wave kernel
+// otherwise) up to 64 (1.5-1.6x there, -3% at 81).  The scale loads of the block mode use 32-bit byte offsets.
 bool small_ok(const a8w8_gemm_args* g)
 {
     const bool block = g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128;
-    if (!block && g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_ROWCOL) return false;
+    const bool mx = g->scale_mode == A8W8_SCALE_MX_E8M0_1x32, mxt = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;
+    if (!block && !mx && !mxt && g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_ROWCOL) return false;
     const long long items256 = (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN);
-    if (items256 * (block ? 2 : 4) > num_cus()) return false;
+    if (items256 * (block || mx ? 2 : 4) > num_cus()) return false;
     if (block && (long long)(g->k / BK) * g->stride_sfa * 4 >= (1ll << 31)) return false;
     return true;
 }
@@ -153,7 +154,7 @@ bool small_ok(const a8w8_gemm_args* g)
 template <int MODE, int CDT>
 int launch_small(const GemmParams& p, int batch, hipStream_t stream)
 {
-    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_BF16) {
+    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT || MODE == MODE_BF16) {
         static bool attr_set[64];
         int dev = 0;
         (void)hipGetDevice(&dev);

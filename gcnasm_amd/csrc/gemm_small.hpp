@@ -20,11 +20,14 @@ constexpr int SM_BM = 128, SM_BN = 128;
 constexpr int SM_THREADS = 256;
 constexpr int SM_STAGES = 4;
 constexpr int SM_STAGE_BYTES = (SM_BM + SM_BN) * BK;   // 32768
-constexpr int SM_SCALE_BYTES = 1024;                   // block mode, per stage: 128 A-row scales, the B scale at +512 and +768
+// Scale bytes per stage.  Block mode: 128 A-row scales, the B scale at +512 and +768.  Row-major MX: the step's
+// four E8M0 bytes of 128 A rows, then of 128 B rows.  Tiled MX: 1 KiB per wave, whose first half is the 512-byte
+// unit (64 rows x one pair of K steps) of the wave's row block.
+constexpr int small_scale_bytes(int mode) { return mode == MODE_MXT ? 4096 : (mode == MODE_BLOCK || mode == MODE_MX) ? 1024 : 0; }
 constexpr int SM_TM = 4, SM_TN = 4;                    // MFMA tiles per wave
 constexpr int small_lds_bytes(int mode)
 {
-    return SM_STAGES * (SM_STAGE_BYTES + (mode == MODE_BLOCK ? SM_SCALE_BYTES : 0));
+    return SM_STAGES * (SM_STAGE_BYTES + small_scale_bytes(mode));
 }
 
 // p.tiles_m / p.tiles_n count 128 x 128 tiles here; grid = (tiles, 1, batch).  The launch bound asks for a
@@ -33,8 +36,10 @@ constexpr int small_lds_bytes(int mode)
 template <int MODE, int CDT>
 __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 {
-    static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_BF16,
-                  "fp32-scale modes and bf16 operands (byte rows of 2k columns, no scales)");
+    static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT || MODE == MODE_BF16,
+                  "fp32 scales, MX scales, or bf16 operands (byte rows of 2k columns, no scales)");
+    constexpr bool STEP_SCALES = MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT;      // scales that change with the K step
+    constexpr int SM_SCALE_BYTES = small_scale_bytes(MODE);
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -68,7 +73,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     }
     // block mode: waves 0 and 1 fetch the step's 128 A-row scales (64 each), waves 2 and 3 the B scale
     // of the tile's 128 x 128 block (every lane the same dword: the stage's copy at +512 is the one read)
-    constexpr int LOADS_PER_STAGE = 8 + (MODE == MODE_BLOCK ? 1 : 0);
+    constexpr int LOADS_PER_STAGE = 8 + (STEP_SCALES ? 1 : 0);
     __amdgpu_buffer_rsrc_t rsrc_sf = rsrc_a;
     int voff_sf = 0, sf_step_bytes = 0;
     if constexpr (MODE == MODE_BLOCK) {
@@ -82,6 +87,31 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
             sf_step_bytes = 4;
         }
     }
+    // MX: waves 0 and 1 fetch the step's dword (four E8M0 bytes, one per 32 of K) of 64 A rows each, waves 2
+    // and 3 those of 64 B rows each
+    if constexpr (MODE == MODE_MX) {
+        const bool is_b = wave >= 2;
+        const int rows = is_b ? p.n : p.m;
+        const int stride = is_b ? p.stride_sfb : p.stride_sfa;
+        const uint8_t* base = is_b ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
+                                   : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
+        rsrc_sf = make_rsrc(base, (uint32_t)(rows - 1) * stride + (uint32_t)(p.k >> 5));
+        voff_sf = min((is_b ? n0 : m0) + (wave & 1) * 64 + lane, rows - 1) * stride;
+        sf_step_bytes = 4;
+    }
+    // tiled MX: wave w fetches the 512-byte unit of its 64-row block (waves 0, 1: the tile's A blocks, 2, 3: its B
+    // blocks) for the step's pair of K steps with one 16-byte load; lanes 32-63 bring the next unit along, unused
+    int mxt_nblk = 1, mxt_blk = 0;
+    if constexpr (MODE == MODE_MXT) {
+        const bool is_b = wave >= 2;
+        const int rows = is_b ? p.n : p.m;
+        const uint8_t* base = is_b ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
+                                   : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
+        rsrc_sf = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, p.k));
+        voff_sf = lane * 16;
+        mxt_nblk = (rows + 63) >> 6;
+        mxt_blk = min(((is_b ? n0 : m0) >> 6) + (wave & 1), mxt_nblk - 1);     // a block past the last row: its rows are never stored
+    }
     auto issue_stage = [&](int stage, int kstep) __attribute__((always_inline)) {
         kstep = min(kstep, nk - 1);         // past the end: reload the last step into a stage nobody reads (fixed wait counts)
         A8W8_LDS char* s = (A8W8_LDS char*)smem + stage * SM_STAGE_BYTES + wave * 1024;
@@ -90,7 +120,10 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
         for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_a, s + j * 4096, voff_a[j], koff);
 #pragma unroll
         for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_b, s + SM_BM * BK + j * 4096, voff_b[j], koff);
-        if constexpr (MODE == MODE_BLOCK) {
+        if constexpr (MODE == MODE_MXT) {
+            A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 1024;
+            load_to_lds_16(rsrc_sf, sc, voff_sf, ((((kstep >> 2) * mxt_nblk + mxt_blk) * 2 + ((kstep >> 1) & 1)) * 512));
+        } else if constexpr (STEP_SCALES) {
             A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 256;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sf, sc, 4, voff_sf, kstep * sf_step_bytes, 0, 0);
         }
@@ -111,6 +144,17 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
         const v4i hi = *(const v4i*)(s + base[1]);
         return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     };
+
+    // tiled MX: byte of (row 16 t + r16 of a 64-row block, 32-block g of the K step, step s of the pair) inside the
+    // block's unit, without s (see mx_tiled_index); the same for A tiles and B tiles
+    int mxt_off[4];
+    if constexpr (MODE == MODE_MXT) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int x = (2 * t + (r16 >> 3)) & 3, y = r16 & 3, par = (r16 >> 2) & 1;
+            mxt_off[t] = ((4 * x + y) * 4 + g) * 8 + (t >> 1) * 4 + par * 2;
+        }
+    }
 
     const int cm_base = m0 + wave_m * 64 + r16;          // + 16 * i
     const int cn_base = n0 + wave_n * 64 + 4 * g;        // + 16 * j + e
@@ -162,10 +206,31 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
                 __builtin_amdgcn_sched_barrier(0);
             }
         } else {
+            int mx_sa[SM_TM], mx_sb[SM_TN];
+            if constexpr (MODE == MODE_MX) {
+                // lane (r16, g) scales K [32g, 32g+32) of its row: byte g of the row's dword
+                const unsigned* sc = (const unsigned*)(smem + SM_STAGES * SM_STAGE_BYTES + cur * SM_SCALE_BYTES);
+#pragma unroll
+                for (int t = 0; t < SM_TM; ++t) mx_sa[t] = (int)__builtin_amdgcn_ubfe(sc[wave_m * 64 + 16 * t + r16], 8 * g, 8);
+#pragma unroll
+                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe(sc[128 + wave_n * 64 + 16 * t + r16], 8 * g, 8);
+            }
+            if constexpr (MODE == MODE_MXT) {
+                const uint8_t* sc = (const uint8_t*)(smem + SM_STAGES * SM_STAGE_BYTES + cur * SM_SCALE_BYTES) + (ks & 1);
+#pragma unroll
+                for (int t = 0; t < SM_TM; ++t) mx_sa[t] = sc[wave_m * 1024 + mxt_off[t]];
+#pragma unroll
+                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = sc[(2 + wave_n) * 1024 + mxt_off[t]];
+            }
 #pragma unroll
             for (int j = 0; j < SM_TN; ++j) {
                 if (j + 1 < SM_TN) fb[(j + 1) & 1] = read_frag(cur, rd_b, j + 1);
-                if constexpr (MODE == MODE_BF16) {
+                if constexpr (MODE == MODE_MX || MODE == MODE_MXT) {
+#pragma unroll
+                    for (int i = 0; i < SM_TM; ++i)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j & 1], fa[i], acc[i][j], 0, 0, 0, mx_sb[j], 0,
+                                                                                     mx_sa[i]);
+                } else if constexpr (MODE == MODE_BF16) {
                     // a 128-byte row is 64 bf16: the fragment's two 16-byte halves feed one 16x16x32 MFMA each (both
                     // operands split K the same way); first halves for all four tiles, then second halves:
                     // back-to-back MFMAs on one accumulator stall

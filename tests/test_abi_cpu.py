@@ -90,7 +90,10 @@ def test_kernel_selection():
     assert g.kernel_name(_ok_args(mode=g.TENSOR, m=1024, n=1024, batch=5)) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(m=2048, n=4096)) == "gemm_a8w8_tile128"                     # block scales: up to 128 tiles
     assert g.kernel_name(_ok_args(m=2304, n=4096)) == "gemm_a8w8_persist"
-    assert g.kernel_name(_ok_args(mode=g.MX)) == "gemm_a8w8_persist"                  # MX scales stay on the 256 tiles
+    assert g.kernel_name(_ok_args(mode=g.MX)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(mode=g.MX, m=2048, n=4096)) == "gemm_a8w8_tile128"          # row-major MX: up to 128 tiles
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, m=2048, n=2048)) == "gemm_a8w8_tile128"    # tiled MX: up to 64
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, m=2304, n=2048)) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=200)) == "gemm_a8w8_general"
     a = _ok_args(mode=g.ROWCOL)
     a.a = 0x1004
@@ -98,9 +101,11 @@ def test_kernel_selection():
 
 
 def test_tiled_mx_mode_selection_and_reorder_preconditions():
-    assert g.kernel_name(_ok_args(mode=g.MX_TILED)) == "gemm_a8w8_wide"
-    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=384)) == "gemm_a8w8_general"      # odd number of K steps
-    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=128)) == "gemm_a8w8_general"
+    big = dict(m=4096, n=4096)
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, **big)) == "gemm_a8w8_wide"
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=384, **big)) == "gemm_a8w8_general"      # odd number of K steps
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=128, **big)) == "gemm_a8w8_general"
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=384)) == "gemm_a8w8_tile128"             # few tiles: any number of K steps
     a = _ok_args(mode=g.MX_TILED, k=48)
     assert g.lib().a8w8_gemm(ctypes.byref(a), None) == -3
     a = _ok_args(mode=g.MX_TILED)
