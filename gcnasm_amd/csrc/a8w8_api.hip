@@ -146,6 +146,8 @@ bool small_ok(const a8w8_gemm_args* g)
     const bool mx = g->scale_mode == A8W8_SCALE_MX_E8M0_1x32, mxt = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;
     if (!block && !mx && !mxt && g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_ROWCOL) return false;
     const long long items256 = (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN);
+    // tiled MX scales with an odd number of K steps have no 256-tile kernel: any size runs here
+    if (mxt && (g->k / BK) % 2 != 0) return true;
     if (items256 * (block || mx ? 2 : 4) > num_cus()) return false;
     if (block && (long long)(g->k / BK) * g->stride_sfa * 4 >= (1ll << 31)) return false;
     return true;

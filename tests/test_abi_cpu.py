@@ -103,9 +103,11 @@ def test_kernel_selection():
 def test_tiled_mx_mode_selection_and_reorder_preconditions():
     big = dict(m=4096, n=4096)
     assert g.kernel_name(_ok_args(mode=g.MX_TILED, **big)) == "gemm_a8w8_wide"
-    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=384, **big)) == "gemm_a8w8_general"      # odd number of K steps
-    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=128, **big)) == "gemm_a8w8_general"
-    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=384)) == "gemm_a8w8_tile128"             # few tiles: any number of K steps
+    # an odd number of K steps: the 128-tile kernel whatever the size (the four-wave kernel walks K in pairs)
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=384, **big)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=128, **big)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=384)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(mode=g.MX_TILED, k=352, stride_a=352, stride_b=352)) == "gemm_a8w8_general"
     a = _ok_args(mode=g.MX_TILED, k=48)
     assert g.lib().a8w8_gemm(ctypes.byref(a), None) == -3
     a = _ok_args(mode=g.MX_TILED)
