@@ -316,15 +316,28 @@ int validate_flat(const a8w8_gemm_args* g)
     return A8W8_OK;
 }
 
-constexpr int FLAT_NT = 4;   // weight tiles per wave: the activation fragment is re-used 4 times
+// Weight tiles (16 rows of B) per workgroup: the activation fragment of a K block is re-used by all of them, but
+// the grid shrinks by the same factor: the largest of 4, 2, 1 that still gives every compute unit a workgroup
+// (16 x 4096 x 4096: 8.6 us with 4 tiles per workgroup on 64 compute units, 5.4 us with 1 on 256).
+// Several groups of 16 activation rows per workgroup (one pass over B for m > 16) were measured slower: the
+// activation gather (16 cache lines per load instruction) then costs more than re-reading B from cache.
+template <int NT, int CDT, int MODE>
+int launch_flat_nt(const GemmParams& p, int batch, hipStream_t stream)
+{
+    const int n_tiles = p.n / 16;
+    dim3 grid((unsigned)((n_tiles + NT - 1) / NT), (unsigned)((p.m + 15) / 16), (unsigned)batch);
+    hipLaunchKernelGGL((flatmm_a8w8<NT, CDT, MODE>), grid, dim3(FLAT_THREADS), 0, stream, p);
+    return launch_status();
+}
 
 template <int CDT, int MODE>
 int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 {
-    const int n_tiles = p.n / 16;
-    dim3 grid((unsigned)((n_tiles + FLAT_NT - 1) / FLAT_NT), (unsigned)((p.m + 15) / 16), (unsigned)batch);
-    hipLaunchKernelGGL((flatmm_a8w8<FLAT_NT, CDT, MODE>), grid, dim3(FLAT_THREADS), 0, stream, p);
-    return launch_status();
+    const long long tiles = (long long)(p.n / 16) * ((p.m + 15) / 16) * batch;
+    const int cus = num_cus();
+    if (tiles >= 4ll * cus) return launch_flat_nt<4, CDT, MODE>(p, batch, stream);
+    if (tiles >= 2ll * cus) return launch_flat_nt<2, CDT, MODE>(p, batch, stream);
+    return launch_flat_nt<1, CDT, MODE>(p, batch, stream);
 }
 
 }  // namespace
