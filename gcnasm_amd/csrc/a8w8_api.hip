@@ -155,7 +155,8 @@ bool small_ok(const a8w8_gemm_args* g)
 template <int MODE, int CDT>
 int launch_small(const GemmParams& p, int batch, hipStream_t stream)
 {
-    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT || MODE == MODE_BF16) {
+    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT ||
+                  MODE == MODE_BF16 || MODE == MODE_F4T) {
         static bool attr_set[64];
         int dev = 0;
         (void)hipGetDevice(&dev);
@@ -431,10 +432,14 @@ int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream)
     bytes.stride_a = g->stride_a / 2; bytes.stride_b = g->stride_b / 2;
     bytes.stride_a_batch = g->stride_a_batch / 2; bytes.stride_b_batch = g->stride_b_batch / 2;
     bytes.scale_mode = A8W8_SCALE_MX_E8M0_TILED;
-    if (tiled && g->k % 256 == 0 && tiled_ok(&bytes) && persist_ok(&bytes)) {
+    if (tiled && g->k % 256 == 0 && tiled_ok(&bytes)) {
         const GemmParams p = make_params(&bytes);
-        return g->c_dtype == A8W8_C_BF16 ? launch_wide<MODE_F4T, C_BF16>(p, g->batch, s)
-                                         : launch_wide<MODE_F4T, C_FP32>(p, g->batch, s);
+        if (small_ok(&bytes))       // few tiles, or an odd number of 128-byte K steps
+            return g->c_dtype == A8W8_C_BF16 ? launch_small<MODE_F4T, C_BF16>(p, g->batch, s)
+                                             : launch_small<MODE_F4T, C_FP32>(p, g->batch, s);
+        if (persist_ok(&bytes))
+            return g->c_dtype == A8W8_C_BF16 ? launch_wide<MODE_F4T, C_BF16>(p, g->batch, s)
+                                             : launch_wide<MODE_F4T, C_FP32>(p, g->batch, s);
     }
     dim3 grid((unsigned)((g->n + 15) / 16), (unsigned)((g->m + 15) / 16), (unsigned)g->batch);
 #define A4W4_GENERAL(CDT, TILED)                                                                                        \

@@ -23,7 +23,7 @@ constexpr int SM_STAGE_BYTES = (SM_BM + SM_BN) * BK;   // 32768
 // Scale bytes per stage.  Block mode: 128 A-row scales, the B scale at +512 and +768.  Row-major MX: the step's
 // four E8M0 bytes of 128 A rows, then of 128 B rows.  Tiled MX: 1 KiB per wave, whose first half is the 512-byte
 // unit (64 rows x one pair of K steps) of the wave's row block.
-constexpr int small_scale_bytes(int mode) { return mode == MODE_MXT ? 4096 : (mode == MODE_BLOCK || mode == MODE_MX) ? 1024 : 0; }
+constexpr int small_scale_bytes(int mode) { return mode == MODE_MXT || mode == MODE_F4T ? 4096 : (mode == MODE_BLOCK || mode == MODE_MX) ? 1024 : 0; }
 constexpr int SM_TM = 4, SM_TN = 4;                    // MFMA tiles per wave
 constexpr int small_lds_bytes(int mode)
 {
@@ -36,9 +36,13 @@ constexpr int small_lds_bytes(int mode)
 template <int MODE, int CDT>
 __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 {
-    static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT || MODE == MODE_BF16,
-                  "fp32 scales, MX scales, or bf16 operands (byte rows of 2k columns, no scales)");
-    constexpr bool STEP_SCALES = MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT;      // scales that change with the K step
+    static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT ||
+                      MODE == MODE_BF16 || MODE == MODE_F4T,
+                  "fp32 scales, MX scales, bf16 operands (byte rows of 2k columns, no scales) or packed E2M1 operands (byte "
+                  "rows of k/2 columns) with tiled MX scales");
+    // tiled scales: of FP8 operands (a K step is 4 blocks of 32: one step of a pair) or of FP4 operands (8 blocks: a pair)
+    constexpr bool TILED_SCALES = MODE == MODE_MXT || MODE == MODE_F4T;
+    constexpr bool STEP_SCALES = MODE == MODE_BLOCK || MODE == MODE_MX || TILED_SCALES;      // scales that change with the K step
     constexpr int SM_SCALE_BYTES = small_scale_bytes(MODE);
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     const int tid = threadIdx.x;
@@ -102,12 +106,12 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     // tiled MX: wave w fetches the 512-byte unit of its 64-row block (waves 0, 1: the tile's A blocks, 2, 3: its B
     // blocks) for the step's pair of K steps with one 16-byte load; lanes 32-63 bring the next unit along, unused
     int mxt_nblk = 1, mxt_blk = 0;
-    if constexpr (MODE == MODE_MXT) {
+    if constexpr (TILED_SCALES) {
         const bool is_b = wave >= 2;
         const int rows = is_b ? p.n : p.m;
         const uint8_t* base = is_b ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
                                    : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
-        rsrc_sf = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, p.k));
+        rsrc_sf = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, MODE == MODE_F4T ? 2 * p.k : p.k));      // k in elements
         voff_sf = lane * 16;
         mxt_nblk = (rows + 63) >> 6;
         mxt_blk = min(((is_b ? n0 : m0) >> 6) + (wave & 1), mxt_nblk - 1);     // a block past the last row: its rows are never stored
@@ -120,9 +124,11 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
         for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_a, s + j * 4096, voff_a[j], koff);
 #pragma unroll
         for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_b, s + SM_BM * BK + j * 4096, voff_b[j], koff);
-        if constexpr (MODE == MODE_MXT) {
+        if constexpr (TILED_SCALES) {
             A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 1024;
-            load_to_lds_16(rsrc_sf, sc, voff_sf, ((((kstep >> 2) * mxt_nblk + mxt_blk) * 2 + ((kstep >> 1) & 1)) * 512));
+            // the pair of 128-element K steps this step belongs to (FP8: two byte steps) or is (FP4: 256 elements)
+            const int pair = MODE == MODE_F4T ? kstep : kstep >> 1;
+            load_to_lds_16(rsrc_sf, sc, voff_sf, ((((pair >> 1) * mxt_nblk + mxt_blk) * 2 + (pair & 1)) * 512));
         } else if constexpr (STEP_SCALES) {
             A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 256;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sf, sc, 4, voff_sf, kstep * sf_step_bytes, 0, 0);
@@ -148,7 +154,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     // tiled MX: byte of (row 16 t + r16 of a 64-row block, 32-block g of the K step, step s of the pair) inside the
     // block's unit, without s (see mx_tiled_index); the same for A tiles and B tiles
     int mxt_off[4];
-    if constexpr (MODE == MODE_MXT) {
+    if constexpr (TILED_SCALES) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int x = (2 * t + (r16 >> 3)) & 3, y = r16 & 3, par = (r16 >> 2) & 1;
@@ -215,6 +221,14 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
                 for (int t = 0; t < SM_TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe(sc[128 + wave_n * 64 + 16 * t + r16], 8 * g, 8);
             }
+            if constexpr (MODE == MODE_F4T) {
+                // both halves' bytes sit side by side: one 16-bit read, the half is chosen by op_sel
+                const char* sc = smem + SM_STAGES * SM_STAGE_BYTES + cur * SM_SCALE_BYTES;
+#pragma unroll
+                for (int t = 0; t < SM_TM; ++t) mx_sa[t] = *(const unsigned short*)(sc + wave_m * 1024 + mxt_off[t]);
+#pragma unroll
+                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = *(const unsigned short*)(sc + (2 + wave_n) * 1024 + mxt_off[t]);
+            }
             if constexpr (MODE == MODE_MXT) {
                 const uint8_t* sc = (const uint8_t*)(smem + SM_STAGES * SM_STAGE_BYTES + cur * SM_SCALE_BYTES) + (ks & 1);
 #pragma unroll
@@ -225,7 +239,24 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
             for (int j = 0; j < SM_TN; ++j) {
                 if (j + 1 < SM_TN) fb[(j + 1) & 1] = read_frag(cur, rd_b, j + 1);
-                if constexpr (MODE == MODE_MX || MODE == MODE_MXT) {
+                if constexpr (MODE == MODE_F4T) {
+                    // two FP4 MFMAs per fragment pair: elements [0, 128) of the step sit in the fragments' first 16
+                    // bytes, [128, 256) in the second; op_sel picks the half's scale byte
+#pragma unroll
+                    for (int i = 0; i < SM_TM; ++i) {
+                        const v8i& fbj = fb[j & 1];
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                            (v8i{fbj[0], fbj[1], fbj[2], fbj[3], 0, 0, 0, 0}), (v8i{fa[i][0], fa[i][1], fa[i][2], fa[i][3], 0, 0, 0, 0}),
+                            acc[i][j], 4, 4, 0, mx_sb[j], 0, mx_sa[i]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < SM_TM; ++i) {
+                        const v8i& fbj = fb[j & 1];
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                            (v8i{fbj[4], fbj[5], fbj[6], fbj[7], 0, 0, 0, 0}), (v8i{fa[i][4], fa[i][5], fa[i][6], fa[i][7], 0, 0, 0, 0}),
+                            acc[i][j], 4, 4, 1, mx_sb[j], 1, mx_sa[i]);
+                    }
+                } else if constexpr (MODE == MODE_MX || MODE == MODE_MXT) {
 #pragma unroll
                     for (int i = 0; i < SM_TM; ++i)
                         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j & 1], fa[i], acc[i][j], 0, 0, 0, mx_sb[j], 0,

@@ -109,8 +109,8 @@ A8W8_API int a16w16_flatmm(const a8w8_gemm_args* args, void* hip_stream);
  * 32 elements) through the same f8f6f4 instruction in its FP4 format (the reference names the format,
  * wmma_opus_rdna4/opus/opus.hpp:1854-1855, and has no program for it).  A [batch, m, k/2 bytes],
  * B [batch, n, k/2 bytes]; m, n, k and every stride count ELEMENTS (strides even); scale_mode is
- * MX_E8M0_1x32 (row-major scales, general kernel) or MX_E8M0_TILED (pipelined kernel when k % 256 == 0,
- * k >= 512 and rows are 16-byte aligned). */
+ * MX_E8M0_1x32 (row-major scales, general kernel) or MX_E8M0_TILED (MFMA kernels when k % 256 == 0 and rows
+ * are 16-byte aligned). */
 A8W8_API int a4w4_gemm(const a8w8_gemm_args* args, void* hip_stream);
 /* fp32 rows -> packed E2M1 + E8M0 scales: e = clamp(ceil(log2(amax32/6)), -127, 127), row-major scales
  * scale[r*(k/32) + p/32] or (tiled != 0) the MX_TILED layout. */

@@ -35,7 +35,7 @@ def test_quantiser_matches_oracle(orc, rows, k):
     assert torch.equal(qt, q) and (st.cpu().numpy() == orc.mx_tile_scales(sr)).all()
 
 
-@pytest.mark.parametrize("shape", [(37, 53, 96), (64, 64, 256), (70, 40, 384)])
+@pytest.mark.parametrize("shape", [(37, 53, 96), (64, 64, 224), (70, 40, 384)])       # k % 256 != 0: no MFMA kernel
 def test_general_kernel_is_bit_exact(orc, shape):
     m, n, k = shape
     qa, ea = orc.quantize_mxfp4(_x(m, k, 11))
