@@ -243,6 +243,53 @@ def run_quantizers(torch, g, steps, warmup, seed):
     return out
 
 
+# What the reference publishes for its own block-scale program (fp32 C, A~U[0,1), B~U[-.5,.5), scales~U[.8,1.2);
+# opus_gemm/block_scale_gemm/README.md:111-114) and as the expected output of its flat program
+# (opus_fmm/README.md:43-49, 2*16*4096*4096 flops), on MI355X.
+REFERENCE_PUBLISHED = {"block_fp32_1024": 118.96, "block_fp32_2048": 616.77, "block_fp32_4096": 2237.77, "block_fp32_8192": 2710.24,
+                       "flatmm_16x4096x4096": 20.64}
+
+
+def run_reference_program_sizes(torch, g, steps, warmup, seed):
+    """The reference's own programs at the sizes it publishes numbers for, with its inputs and its metric
+    (2*M*N*K / average launch time): the ratio to the published TFlops is reported beside each."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+
+    def uniform(shape, lo, hi):
+        return torch.rand(shape, generator=gen, device="cuda", dtype=torch.float32) * (hi - lo) + lo
+
+    out = []
+    for size in (1024, 2048, 4096, 8192):
+        m = n = k = size
+        a = g.cvt_f32_to_e4m3(uniform((m, k), 0.0, 1.0))
+        b = g.cvt_f32_to_e4m3(uniform((n, k), -0.5, 0.5))
+        sfa, sfb = uniform((k // 128, m), 0.8, 1.2), uniform((n // 128, k // 128), 0.8, 1.2)
+        c = torch.empty((m, n), dtype=torch.float32, device="cuda")
+        ms, wall = time_best_of(torch, lambda i: g.gemm_blockscale(a, b, sfa, sfb, c=c), steps, warmup)
+        name = f"block_fp32_{size}"
+        tf = 2.0 * m * n * k / ms / 1e9
+        out.append({"workload": name, "m": m, "n": n, "k": k, "kernel": g.kernel_name(g.raw_gemm_args(
+            1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, m, n, k, g.BLOCK, c_dtype=g.FP32)), "ms_per_launch": ms,
+            "wall_ms_per_launch": wall, "tflops": tf, "reference_published_tflops": REFERENCE_PUBLISHED[name],
+            "vs_reference_published": tf / REFERENCE_PUBLISHED[name]})
+        del a, b, sfa, sfb, c
+        torch.cuda.empty_cache()
+    m, n, k = 16, 4096, 4096
+    a, sfa = g.quantize(torch.randn((m, k), generator=gen, device="cuda"), g.ROWCOL)
+    b, sfb = g.quantize(torch.randn((n, k), generator=gen, device="cuda"), g.ROWCOL)
+    bs = g.preshuffle_b_device(b)
+    c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    ms, wall = time_best_of(torch, lambda i: g.flatmm(a, bs, sfa, sfb, n, c=c), steps, warmup)
+    tf = 2.0 * m * n * k / ms / 1e9
+    out.append({"workload": "flatmm_16x4096x4096", "m": m, "n": n, "k": k, "kernel": "flatmm_a8w8", "ms_per_launch": ms,
+                "wall_ms_per_launch": wall, "tflops": tf, "reference_published_tflops": REFERENCE_PUBLISHED["flatmm_16x4096x4096"],
+                "vs_reference_published": tf / REFERENCE_PUBLISHED["flatmm_16x4096x4096"],
+                "note": "a launch from Python through ctypes costs about 9 us, which bounds this entry; the C++ program "
+                        "tests/harness/flatmm_a8w8.exe -m 16 -n 4096 -k 4096 measures the kernel's own rate"})
+    return out
+
+
 def cpu_baseline(name, inp, c_gpu, torch, budget_s=15.0):
     """Times the oracle (port of the reference's host GEMM: per-MAC software fp8 decode,
     OpenMP over (i, j), gemm_a8w8_blockscale_host.cc:66-90) on the first rows of the same
@@ -333,6 +380,7 @@ def main():
             del i2, c2
             torch.cuda.empty_cache()
         others.extend(run_quantizers(torch, g, args.steps, args.warmup, args.seed + 2))
+        others.extend(run_reference_program_sizes(torch, g, args.steps, args.warmup, args.seed + 3))
         line["other_workloads"] = others
     print(json.dumps(line))
 
