@@ -320,6 +320,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                 for (int e = 0; e < 4; ++e) { sb[jp][e] = lo[e]; sb[jp][4 + e] = hi[e]; }
             }
         }
+        // a tile that lies inside the matrix and takes 16-byte stores is written without per-lane checks (the
+        // checked path spends more instructions on masks and branches than on stores)
+        const bool whole = vec_ok && m0 + BM <= p.m && n0 + BN <= p.n;
 #pragma unroll
         for (int jp = 0; jp < TN / 2; ++jp) {
             const int cn = cn_base + 32 * jp;
@@ -332,6 +335,20 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                     v[e] = acc[i][2 * jp + (e >> 2)][e & 3];
                     if constexpr (MODE == MODE_TENSOR) v[e] *= ts;
                     if constexpr (MODE == MODE_ROWCOL) v[e] *= sb[jp][e] * sa[i];
+                }
+                if (whole) {
+                    if constexpr (CDT == C_BF16) {
+                        v4i w;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+                        A8W8_STORE_C((v4i*)((unsigned short*)c_base + (long long)cm * p.ldc + cn), w);
+                    } else {
+                        float* dst = (float*)c_base + (long long)cm * p.ldc + cn;
+                        A8W8_STORE_C((v4f*)dst, (v4f{v[0], v[1], v[2], v[3]}));
+                        A8W8_STORE_C((v4f*)(dst + 4), (v4f{v[4], v[5], v[6], v[7]}));
+                    }
+                    continue;
                 }
                 if (cm >= p.m) continue;
                 if constexpr (CDT == C_BF16) {

@@ -295,6 +295,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     char* c_base = (char*)p.c + (long long)batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
     const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 7) == 0)
                                         : ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 15) == 0);
+    const bool whole = vec_ok && m0 + SM_BM <= p.m && n0 + SM_BN <= p.n;
 #pragma unroll
     for (int j = 0; j < SM_TN; ++j) {
         const int cn = cn_base + 16 * j;
@@ -309,6 +310,14 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
             v4f v = acc[i][j];
             if constexpr (MODE == MODE_TENSOR) v *= ts;
             if constexpr (MODE == MODE_ROWCOL) v *= sb * sa[i];
+            if (whole) {        // inside the matrix, aligned rows: no per-lane checks
+                if constexpr (CDT == C_BF16)
+                    A8W8_STORE_C((v4u16*)((unsigned short*)c_base + (long long)cm * p.ldc + cn),
+                                 (v4u16{bf16_bits(v.x), bf16_bits(v.y), bf16_bits(v.z), bf16_bits(v.w)}));
+                else
+                    A8W8_STORE_C((v4f*)((float*)c_base + (long long)cm * p.ldc + cn), v);
+                continue;
+            }
             if (cm >= p.m) continue;
             if constexpr (CDT == C_BF16) {
                 unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
