@@ -135,44 +135,53 @@ int num_cus()
     return g_num_cus[dev & 63] > 0 ? g_num_cus[dev & 63] : 256;
 }
 
-// 128 x 128 tiles when 256 x 256 tiles would leave most compute units without work.  Measured crossover on
-// 256 compute units: block scales and row-major MX scales (eight-wave kernel otherwise) gain up to 128 tiles of
-// 256 x 256 (2.2x at 16 tiles, +14% at 100, even at 128); per-tensor, row/col and tiled MX (four-wave kernel
-// otherwise) up to 64 (1.5-1.6x there, -3% at 81).  The scale loads of the block mode use 32-bit byte offsets.
+// 128 x 128 tiles when all of them fit on the chip at once, two workgroups per compute unit: a problem of that
+// size leaves 256 x 256 tiles with at most half of the compute units.  Measured on 256 compute units against the
+// 256-tile kernels (block / row-col / tiled MX): 2.2x / 1.7x / 1.6x at 64 workgroups, 1.9x / 1.6x / 1.5x at 256,
+// +45% / +21% / +15% at 400, +37% / +17% / +9% at 512; beyond that the second round of workgroups costs more than
+// the idle compute units did (-9% for row/col at 576).  The scale loads of the block mode use 32-bit byte offsets.
 bool small_ok(const a8w8_gemm_args* g)
 {
     const bool block = g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128;
-    const bool mx = g->scale_mode == A8W8_SCALE_MX_E8M0_1x32, mxt = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;
-    if (!block && !mx && !mxt && g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_ROWCOL) return false;
-    const long long items256 = (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN);
+    const bool mxt = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;
+    if (block && (long long)(g->k / BK) * g->stride_sfa * 4 >= (1ll << 31)) return false;
     // tiled MX scales with an odd number of K steps have no 256-tile kernel: any size runs here
     if (mxt && (g->k / BK) % 2 != 0) return true;
-    if (items256 * (block || mx ? 2 : 4) > num_cus()) return false;
-    if (block && (long long)(g->k / BK) * g->stride_sfa * 4 >= (1ll << 31)) return false;
-    return true;
+    const long long items128 = (long long)g->batch * ((g->m + SM_BM - 1) / SM_BM) * ((g->n + SM_BN - 1) / SM_BN);
+    return items128 <= 2ll * num_cus();
 }
 
+template <int MODE, int CDT, int STAGES>
+int launch_small_stages(const GemmParams& q, int batch, hipStream_t stream)
+{
+    static bool attr_set[64];
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    auto kern = gemm_a8w8_tile128<MODE, CDT, STAGES>;
+    constexpr int lds_bytes = small_lds_bytes(MODE, STAGES);
+    if (!attr_set[dev & 63]) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+            return A8W8_ERR_LAUNCH;
+        attr_set[dev & 63] = true;
+    }
+    dim3 grid((unsigned)(q.tiles_m * q.tiles_n), 1, (unsigned)batch);
+    hipLaunchKernelGGL(kern, grid, dim3(SM_THREADS), lds_bytes, stream, q);
+    return launch_status();
+}
+
+// Up to one workgroup per compute unit: four LDS stages (deep prefetch, one workgroup per compute unit).  More: two
+// stages, so that two workgroups share a compute unit and hide each other's waits.
 template <int MODE, int CDT>
 int launch_small(const GemmParams& p, int batch, hipStream_t stream)
 {
     if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT ||
                   MODE == MODE_BF16 || MODE == MODE_F4T) {
-        static bool attr_set[64];
-        int dev = 0;
-        (void)hipGetDevice(&dev);
-        auto kern = gemm_a8w8_tile128<MODE, CDT>;
-        constexpr int lds_bytes = small_lds_bytes(MODE);
-        if (!attr_set[dev & 63]) {
-            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-                return A8W8_ERR_LAUNCH;
-            attr_set[dev & 63] = true;
-        }
         GemmParams q = p;
         q.tiles_m = (p.m + SM_BM - 1) / SM_BM;
         q.tiles_n = (p.n + SM_BN - 1) / SM_BN;
-        dim3 grid((unsigned)(q.tiles_m * q.tiles_n), 1, (unsigned)batch);
-        hipLaunchKernelGGL(kern, grid, dim3(SM_THREADS), lds_bytes, stream, q);
-        return launch_status();
+        if ((long long)q.tiles_m * q.tiles_n * batch <= num_cus())
+            return launch_small_stages<MODE, CDT, 4>(q, batch, stream);
+        return launch_small_stages<MODE, CDT, 2>(q, batch, stream);
     } else {
         return A8W8_ERR_BAD_MODE;
     }

@@ -18,24 +18,28 @@ namespace a8w8 {
 
 constexpr int SM_BM = 128, SM_BN = 128;
 constexpr int SM_THREADS = 256;
-constexpr int SM_STAGES = 4;
 constexpr int SM_STAGE_BYTES = (SM_BM + SM_BN) * BK;   // 32768
 // Scale bytes per stage.  Block mode: 128 A-row scales, the B scale at +512 and +768.  Row-major MX: the step's
 // four E8M0 bytes of 128 A rows, then of 128 B rows.  Tiled MX: 1 KiB per wave, whose first half is the 512-byte
 // unit (64 rows x one pair of K steps) of the wave's row block.
 constexpr int small_scale_bytes(int mode) { return mode == MODE_MXT || mode == MODE_F4T ? 4096 : (mode == MODE_BLOCK || mode == MODE_MX) ? 1024 : 0; }
 constexpr int SM_TM = 4, SM_TN = 4;                    // MFMA tiles per wave
-constexpr int small_lds_bytes(int mode)
+constexpr int small_lds_bytes(int mode, int stages)
 {
-    return SM_STAGES * (SM_STAGE_BYTES + small_scale_bytes(mode));
+    return stages * (SM_STAGE_BYTES + small_scale_bytes(mode));
 }
 
 // p.tiles_m / p.tiles_n count 128 x 128 tiles here; grid = (tiles, 1, batch).  The launch bound asks for a
 // 256-register budget: with 512 the compiler parks the block mode's partial tiles in accumulation registers
 // and copies each value back before its multiply-add.
-template <int MODE, int CDT>
+// SM_STAGES = 4: loads three K steps ahead, one barrier per step, one workgroup per compute unit (132-144 KiB of
+// LDS) -- for grids of at most one workgroup per compute unit, where nothing else hides the load latency.
+// SM_STAGES = 2: loads issued when a stage has been read, two barriers per step, two workgroups per compute unit
+// that hide each other's waits -- for larger grids.
+template <int MODE, int CDT, int SM_STAGES>
 __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 {
+    static_assert(SM_STAGES == 2 || SM_STAGES == 4, "two or four LDS stages");
     static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT ||
                       MODE == MODE_BF16 || MODE == MODE_F4T,
                   "fp32 scales, MX scales, bf16 operands (byte rows of 2k columns, no scales) or packed E2M1 operands (byte "
@@ -173,14 +177,14 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 
     issue_stage(0, 0);
     issue_stage(1, 1);
-    issue_stage(2, 2);
+    if constexpr (SM_STAGES == 4) issue_stage(2, 2);
 
     for (int ks = 0; ks < nk; ++ks) {
         const int cur = ks & (SM_STAGES - 1);
-        // this wave's loads of stage `cur` have landed once at most the two younger stages are in flight
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LOADS_PER_STAGE) : "memory");
-        A8W8_RAW_BARRIER();                 // ... everyone's have; and everyone is done reading the stage of step ks-1
-        issue_stage((ks + 3) & (SM_STAGES - 1), ks + 3);
+        // this wave's loads of stage `cur` have landed once only the younger stages (two of four, one of two) are in flight
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SM_STAGES / 2) * LOADS_PER_STAGE) : "memory");
+        A8W8_RAW_BARRIER();                 // ... everyone's have; and (four stages) everyone is done reading the stage of step ks-1
+        if constexpr (SM_STAGES == 4) issue_stage((ks + 3) & 3, ks + 3);
 
         v8i fa[SM_TM], fb[2];
 #pragma unroll
@@ -281,6 +285,12 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
                         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j & 1], fa[i], acc[i][j], 0, 0, 0, 0, 0, 0);
                 }
             }
+        }
+        if constexpr (SM_STAGES == 2) {
+            // everyone is done reading stage `cur`: refill it with the step after next (the next step's wait lets
+            // exactly these loads stay in flight)
+            A8W8_RAW_BARRIER();
+            issue_stage(cur, ks + 2);
         }
     }
 

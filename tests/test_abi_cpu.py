@@ -82,18 +82,16 @@ def test_kernel_selection():
     assert g.kernel_name(_ok_args(mode=g.TENSOR, k=1024, **big)) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=384, **big)) == "gemm_a8w8_persist"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=128, **big)) == "gemm_a8w8_tile256"
-    # fp32-scale modes whose 256 x 256 tiles would occupy at most half of the compute units: 128 x 128 tiles
+    # every scale mode: 128 x 128 tiles while all of them fit on the chip at once (two workgroups per compute unit)
     assert g.kernel_name(_ok_args()) == "gemm_a8w8_tile128"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, m=1024, n=2048, k=128)) == "gemm_a8w8_tile128"
-    assert g.kernel_name(_ok_args(mode=g.TENSOR, m=2048, n=2048)) == "gemm_a8w8_tile128"      # 64 tiles of 256 x 256
-    assert g.kernel_name(_ok_args(mode=g.TENSOR, m=2304, n=2048)) == "gemm_a8w8_wide"
-    assert g.kernel_name(_ok_args(mode=g.TENSOR, m=1024, n=1024, batch=5)) == "gemm_a8w8_wide"
-    assert g.kernel_name(_ok_args(m=2048, n=4096)) == "gemm_a8w8_tile128"                     # block scales: up to 128 tiles
+    for mode in (g.TENSOR, g.ROWCOL, g.BLOCK, g.MX, g.MX_TILED):
+        assert g.kernel_name(_ok_args(mode=mode, m=2048, n=4096)) == "gemm_a8w8_tile128"       # 512 workgroups
+        assert g.kernel_name(_ok_args(mode=mode, m=2049, n=4096)) != "gemm_a8w8_tile128"       # 544
+        assert g.kernel_name(_ok_args(mode=mode, m=1024, n=1024, batch=8)) == "gemm_a8w8_tile128"
+        assert g.kernel_name(_ok_args(mode=mode, m=1024, n=1024, batch=9)) != "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(mode=g.TENSOR, m=2304, n=4096)) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(m=2304, n=4096)) == "gemm_a8w8_persist"
-    assert g.kernel_name(_ok_args(mode=g.MX)) == "gemm_a8w8_tile128"
-    assert g.kernel_name(_ok_args(mode=g.MX, m=2048, n=4096)) == "gemm_a8w8_tile128"          # row-major MX: up to 128 tiles
-    assert g.kernel_name(_ok_args(mode=g.MX_TILED, m=2048, n=2048)) == "gemm_a8w8_tile128"    # tiled MX: up to 64
-    assert g.kernel_name(_ok_args(mode=g.MX_TILED, m=2304, n=2048)) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=200)) == "gemm_a8w8_general"
     a = _ok_args(mode=g.ROWCOL)
     a.a = 0x1004
