@@ -1,16 +1,16 @@
-// Dense A8W8 GEMM for problems too small to fill the chip with 256 x 256 tiles: 128 x 128 x 128 tile,
-// 4 waves (2 along M x 2 along N), each wave owning a 64 x 64 block of C as 4 x 4 MFMA tiles of
-// 16 x 16 x 128.  A quarter of the work per workgroup means four times as many workgroups, and a
-// problem of this size is bound by latency (first loads, the K loop's dependent steps, the C stores of
-// one compute unit), not by the matrix cores.
+// Dense GEMM for problems too small to fill the chip with 256 x 256 tiles: 128 x 128 x 128 tile, 4 waves
+// (2 along M x 2 along N), each wave owning a 64 x 64 block of C as 4 x 4 MFMA tiles of 16 x 16 x 128.
+// A quarter of the work per workgroup means four times as many workgroups, and a problem of this size is
+// bound by latency (first loads, the K loop's dependent steps, the C stores of one compute unit), not by the
+// matrix cores.
 //
-// Data path as in the 256-tile kernels: 16-byte direct-to-LDS loads, 128-byte LDS rows whose 16-byte
-// slots are XOR-swizzled with (row & 7), operand roles swapped so that a lane ends up with
-// C[m = lane%16][n = 4*(lane/16) .. +3].  Four LDS stages of 32 KiB: the loads of K step s+3 are issued
-// when step s begins, one raw barrier per step.  Block scales (fp32 per row and K step for A, one per
-// 128 x 128 block for B) ride in the same pipeline: each stage carries its step's 128 row scales and
-// the block's B scale, fetched by one extra direct-to-LDS load per wave, so that the loop's wait counts
-// stay fixed and no global load has to be waited for inside a step.
+// Data path as in the 256-tile kernels: 16-byte direct-to-LDS loads, 128-byte LDS rows whose 16-byte slots are
+// XOR-swizzled with (row & 7), operand roles swapped so that a lane ends up with
+// C[m = lane%16][n = 4*(lane/16) .. +3].  LDS stages of 32 KiB, four (loads three K steps ahead, one raw
+// barrier per step) or two (see the kernel's template parameter).  Scales that change with the K step -- block
+// scales, MX exponents -- ride in the same pipeline: each stage carries its step's scales, fetched by one extra
+// direct-to-LDS load per wave, so that the loop's wait counts stay fixed and no global load has to be waited
+// for inside a step.  Operands: FP8 E4M3, bf16 (byte rows of 2k columns), packed E2M1 (byte rows of k/2 columns).
 #pragma once
 #include "gemm_tile.hpp"
 
