@@ -136,14 +136,61 @@ def test_pipelined_kernels_use_no_scratch():
     seen = 0
     for b in blocks:
         name = b.split()[0]
-        if "gemm_a8w8_persist" in name or "gemm_a8w8_wide" in name or "flatmm_a8w8" in name:
+        if "gemm_a8w8_persist" in name or "gemm_a8w8_wide" in name or "gemm_a8w8_tile128" in name or "flatmm_a8w8" in name:
             seen += 1
             scratch = int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b).group(1))
             assert scratch == 0, (name, scratch)
-    assert seen >= 16
+    assert seen >= 40
     # the four-wave kernels name their accumulator registers themselves: the build checks that the
     # compiler put nothing of its own there (gcnasm_amd/csrc/check_isa.py) and records the verdict
     assert "accumulator registers untouched by the compiler" in text
+
+
+def test_sibling_entry_points_reject_bad_arguments():
+    """bf16, MXFP4, quantiser and conversion entry points: every reject happens before any device call."""
+    L = g.lib()
+    ref = ctypes.byref
+    # a16w16_gemm: strides in bf16 elements
+    a = _ok_args(mode=g.TENSOR)
+    for mutate, want in [(lambda x: setattr(x, "c", None), -1), (lambda x: setattr(x, "k", 0), -2),
+                         (lambda x: setattr(x, "c_dtype", 7), -6), (lambda x: setattr(x, "b_preshuffled", 1), -6),
+                         (lambda x: setattr(x, "stride_b", 100), -4)]:
+        b = _ok_args(mode=g.TENSOR)
+        mutate(b)
+        assert L.a16w16_gemm(ref(b), None) == want
+    assert L.a16w16_gemm(None, None) == -1
+    # a16w16_flatmm
+    for mutate, want in [(lambda x: setattr(x, "b_preshuffled", 0), -6), (lambda x: setattr(x, "m", 65), -2),
+                         (lambda x: setattr(x, "n", 250), -3), (lambda x: setattr(x, "k", 48), -3),
+                         (lambda x: setattr(x, "stride_a", 260), -5), (lambda x: setattr(x, "a", 0x1008), -5)]:
+        b = _ok_args(mode=g.TENSOR, m=16, n=256, k=256, b_preshuffled=1)
+        mutate(b)
+        assert L.a16w16_flatmm(ref(b), None) == want, want
+    # a4w4_gemm: m, n, k and strides in E2M1 elements
+    for mutate, want in [(lambda x: setattr(x, "sfa", None), -1), (lambda x: setattr(x, "scale_mode", g.ROWCOL), -6),
+                         (lambda x: setattr(x, "k", 48), -3), (lambda x: setattr(x, "stride_a", 200), -4),
+                         (lambda x: setattr(x, "stride_a", 259), -5),       # rows must start on a byte
+                         (lambda x: setattr(x, "stride_sfa", 4), -4)]:
+        b = _ok_args(mode=g.MX, m=64, n=64, k=256)
+        mutate(b)
+        assert L.a4w4_gemm(ref(b), None) == want, want
+    # quantisers
+    assert L.a8w8_quantize(None, 4, 32, 32, 0x2000, 0x3000, g.ROWCOL, 1, None) == -1
+    assert L.a8w8_quantize(0x1000, 0, 32, 32, 0x2000, 0x3000, g.ROWCOL, 1, None) == -2
+    assert L.a8w8_quantize(0x1000, 4, 32, 16, 0x2000, 0x3000, g.ROWCOL, 1, None) == -4
+    assert L.a8w8_quantize(0x1000, 4, 100, 100, 0x2000, 0x3000, g.BLOCK, 1, None) == -3
+    assert L.a8w8_quantize(0x1000, 100, 128, 128, 0x2000, 0x3000, g.BLOCK, 128, None) == -3
+    assert L.a8w8_quantize(0x1000, 4, 48, 48, 0x2000, 0x3000, g.MX, 1, None) == -3
+    assert L.a8w8_quantize(0x1000, 4, 32, 32, 0x2000, 0x3000, 9, 1, None) == -6
+    assert L.a4w4_quantize_mx(0x1000, 4, 48, 48, 0x2000, 0x3000, 0, None) == -3
+    assert L.a4w4_quantize_mx(0x1000, 4, 64, 32, 0x2000, 0x3000, 0, None) == -4
+    assert L.a4w4_quantize_mx(0x1000, 4, 64, 64, 0x2000, 0x3002, 1, None) == -5
+    # conversions return the number of elements converted: nothing on bad arguments
+    assert L.a8w8_cvt_f32_to_e4m3(None, 0x2000, 16, g.OCP, 0, None) == 0
+    assert L.a8w8_cvt_f32_to_e4m3(0x1000, 0x2000, 16, 5, 0, None) == 0
+    assert L.a8w8_cvt_e4m3_to_f32(0x1000, None, 16, g.OCP, None) == 0
+    assert L.a8w8_preshuffle_b_device(0x1000, 0x2000, 40, 192, None) == -3
+    assert L.a8w8_preshuffle_b_device(0x1000, 0x2004, 48, 192, None) == -5
 
 
 def test_good_arguments_pass_validation_and_stop_at_the_device():
