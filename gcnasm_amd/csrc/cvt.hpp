@@ -539,8 +539,11 @@ __global__ void __launch_bounds__(256) mx_tile_scales_kernel(const uint8_t* sf0,
     }
     const int blocks = k >> 5;
     if (live) {
-        const int nblk = (rows + 63) >> 6;
-        const int blk = (int)(unit % nblk), kg = (int)(unit / nblk);
+        // the workgroup's four units are consecutive K groups of one 64-row block: together they read 64
+        // contiguous bytes of every row (the units themselves lie K group by K group in the output)
+        const int nblk = (rows + 63) >> 6, kgroups = (k + 511) >> 9;
+        const int kg = (int)(unit % kgroups), blk = (int)(unit / kgroups);
+        unit = (size_t)kg * nblk + blk;
         const int row = blk * 64 + t;
         const uint8_t* src = sf + (size_t)row * stride + kg * 16;
         const bool vec = row < rows && kg * 16 + 16 <= blocks && (((uintptr_t)src) & 3) == 0;
