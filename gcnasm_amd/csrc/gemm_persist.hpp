@@ -1,4 +1,6 @@
-// Persistent, software-pipelined dense A8W8 GEMM for gfx950 (the fast path of a8w8_gemm).
+// Persistent, software-pipelined dense A8W8 GEMM for gfx950, eight waves: block scales, row-major MX scales,
+// and the per-tensor / row-col / bf16 cases with an odd number of K steps (the four-wave kernel of
+// gemm_wide.hpp takes the even ones and tiled MX scales, gemm_small.hpp the problems of few tiles).
 //
 // Tile 256 x 256 x 128, 8 waves (4 along M x 2 along N), wave tile 64 x 128 = 4 x 8 MFMA
 // tiles of 16 x 16 x 128, operands staged global -> LDS with 16-byte direct-to-LDS loads,
