@@ -72,6 +72,7 @@ def lib():
         L.a16w16_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a16w16_flatmm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a4w4_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.a4w4_flatmm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a4w4_quantize_mx.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_int, vp]
         L.a8w8_flatmm.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.a8w8_preshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
@@ -220,6 +221,17 @@ def gemm_a4w4(a, b, sfa, sfb, scale_mode=MX_TILED, c=None, c_dtype=BF16):
     g = raw_gemm_args(a.data_ptr(), b.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, scale_mode, c_dtype,
                       stride_a=a.stride(-2) * 2, stride_b=b.stride(-2) * 2, stride_c=c.stride(-2))
     _check(lib().a4w4_gemm(ctypes.byref(g), _stream()), "a4w4_gemm")
+    return c
+
+
+def flatmm_a4w4(a, b_shuffled, sfa_tiled, sfb_tiled, n, c=None, c_dtype=BF16):
+    """MXFP4 skinny-M GEMM through a4w4_flatmm: a [M, K/2] packed E2M1 with M <= 64, b_shuffled from
+    preshuffle_b_device on the packed weight bytes [N, K/2], both scale arrays in the MX_TILED layout."""
+    m, k = a.shape[-2], a.shape[-1] * 2
+    c, c_dtype = _out(c, (m, n), c_dtype, a.device)
+    g = raw_gemm_args(a.data_ptr(), b_shuffled.data_ptr(), c.data_ptr(), sfa_tiled.data_ptr(), sfb_tiled.data_ptr(), m, n, k,
+                      MX_TILED, c_dtype, stride_a=a.stride(-2) * 2, stride_b=k, stride_c=c.stride(-2), b_preshuffled=1)
+    _check(lib().a4w4_flatmm(ctypes.byref(g), _stream()), "a4w4_flatmm")
     return c
 
 

@@ -350,6 +350,25 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
     return launch_flat_nt<1, CDT, MODE>(p, batch, stream);
 }
 
+template <int NT, int CDT>
+int launch_flat_f4_nt(const GemmParams& p, int batch, hipStream_t stream)
+{
+    const int n_tiles = p.n / 16;
+    dim3 grid((unsigned)((n_tiles + NT - 1) / NT), (unsigned)((p.m + 15) / 16), (unsigned)batch);
+    hipLaunchKernelGGL((flatmm_a4w4<NT, CDT>), grid, dim3(FLAT_THREADS), 0, stream, p);
+    return launch_status();
+}
+
+template <int CDT>
+int launch_flat_f4(const GemmParams& p, int batch, hipStream_t stream)
+{
+    const long long tiles = (long long)(p.n / 16) * ((p.m + 15) / 16) * batch;
+    const int cus = num_cus();
+    if (tiles >= 4ll * cus) return launch_flat_f4_nt<4, CDT>(p, batch, stream);
+    if (tiles >= 2ll * cus) return launch_flat_f4_nt<2, CDT>(p, batch, stream);
+    return launch_flat_f4_nt<1, CDT>(p, batch, stream);
+}
+
 }  // namespace
 
 extern "C" {
@@ -461,6 +480,34 @@ int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream)
     else { if (tiled) A4W4_GENERAL(C_FP32, true); else A4W4_GENERAL(C_FP32, false); }
 #undef A4W4_GENERAL
     return launch_status();
+}
+
+int a4w4_flatmm(const a8w8_gemm_args* g, void* hip_stream)
+{
+    if (!g) return A8W8_ERR_NULL_POINTER;
+    if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
+    if (!g->b_preshuffled || g->scale_mode != A8W8_SCALE_MX_E8M0_TILED) return A8W8_ERR_BAD_MODE;
+    if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0 || g->m > 64) return A8W8_ERR_BAD_SHAPE;
+    if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
+    if (g->n % 16 != 0 || g->k % 128 != 0) return A8W8_ERR_BAD_GROUP;
+    if (g->stride_c < g->n || g->stride_a < g->k) return A8W8_ERR_BAD_STRIDE;
+    if (g->batch > 1 && (g->stride_a_batch < 0 || g->stride_b_batch < 0 || g->stride_c_batch < 0 ||
+                         g->stride_sfa_batch < 0 || g->stride_sfb_batch < 0))
+        return A8W8_ERR_BAD_STRIDE;
+    if (!aligned16(g->a) || !aligned16(g->b) || !aligned16(g->sfa) || !aligned16(g->sfb) || g->stride_a % 32 != 0)
+        return A8W8_ERR_MISALIGNED;
+    if (g->batch > 1 && (g->stride_a_batch % 32 != 0 || g->stride_b_batch % 32 != 0 || g->stride_sfa_batch % 16 != 0 ||
+                         g->stride_sfb_batch % 16 != 0))
+        return A8W8_ERR_MISALIGNED;
+    if ((long long)g->n * g->k / 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
+    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    a8w8_gemm_args bytes = *g;      // packed rows as byte rows of k/2 columns
+    bytes.k = g->k / 2;
+    bytes.stride_a = g->stride_a / 2; bytes.stride_b = g->k / 2;
+    bytes.stride_a_batch = g->stride_a_batch / 2; bytes.stride_b_batch = g->stride_b_batch / 2;
+    const GemmParams p = make_params(&bytes);
+    hipStream_t s = (hipStream_t)hip_stream;
+    return g->c_dtype == A8W8_C_BF16 ? launch_flat_f4<C_BF16>(p, g->batch, s) : launch_flat_f4<C_FP32>(p, g->batch, s);
 }
 
 // the vectorised quantisers read 16 bytes per lane and write packed words

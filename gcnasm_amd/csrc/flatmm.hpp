@@ -144,4 +144,130 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     }
 }
 
+// The MXFP4 flat GEMM: A and B hold packed E2M1 (two elements per byte), B pre-shuffled as the byte matrix
+// [n][k/2] with the same 1 KiB blocks -- a block is 16 rows x 64 bytes = 16 rows x 128 elements, exactly one
+// operand of the FP4 form of the 16 x 16 x 128 MFMA (lane (kq, r) supplies elements [32 kq, 32 kq + 32) of
+// row r, one 32-element scale block).  E8M0 scales of both operands come in the tiled layout of the dense
+// kernels (mx_tiled_index): the two bytes of (row, 32-block g) for the two 128-element blocks of a pair sit side
+// by side, so a lane fetches one 16-bit word per tile and pair of blocks and op_sel picks the block's byte.
+// p.k, p.lda count bytes (k/2 of the element counts); p.m, p.n count rows.
+template <int NT, int CDT>
+__global__ void __launch_bounds__(FLAT_THREADS) flatmm_a4w4(GemmParams p)
+{
+    static_assert(NT <= FLAT_WAVES, "wave t finishes weight tile t");
+    __shared__ v4f red[FLAT_WAVES][NT][64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = wave_uniform(tid >> 6);
+    const int batch = blockIdx.z;
+    const int r16 = lane & 15, kq = lane >> 4;
+
+    const int n_tiles = p.n >> 4;
+    const int k_tiles = p.k >> 6;                  // blocks of 64 bytes = 128 elements = one MFMA
+    const int nt0 = blockIdx.x * NT;
+    const int m_tile = blockIdx.y;
+    const int m0 = m_tile * 16;
+    const int cm = m0 + r16;
+    const int cn = (nt0 + wave) * 16 + 4 * kq;
+    const bool finisher = wave < NT && cm < p.m && nt0 + wave < n_tiles;
+
+    const uint8_t* a_row = p.a + (long long)batch * p.a_batch + (long long)min(m0 + r16, p.m - 1) * p.lda + kq * 16;
+    const uint8_t* b_base = p.b + (long long)batch * p.b_batch + lane * 16;
+    const uint8_t* b_tile[NT];
+    // scale words: inside a 64-row block, row 16 i + r16 of 32-block kq lives at ((4x + y) * 4 + kq) * 8 + jp * 4 +
+    // par * 2 + s with x = (2 i + r16 / 8) % 4, y = r16 % 4, jp = i / 2, par = (r16 / 4) % 2; the unit of (K group of
+    // 512 elements, row block, pair of 128-element blocks) starts at ((kgroup * nblk + blk) * 2 + pair) * 512
+    const int y = r16 & 3, par = (r16 >> 2) & 1;
+    auto scale_lane_off = [&](int i) { return ((4 * ((2 * i + (r16 >> 3)) & 3) + y) * 4 + kq) * 8 + (i >> 1) * 4 + par * 2; };
+    const int nblk_a = (p.m + 63) >> 6, nblk_b = (p.n + 63) >> 6;
+    const uint8_t* sfa = (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch + (size_t)(m_tile >> 2) * 1024 + scale_lane_off(m_tile & 3);
+    const uint8_t* sfb[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int nt = min(nt0 + t, n_tiles - 1);
+        b_tile[t] = b_base + (long long)nt * k_tiles * 1024;
+        sfb[t] = (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch + (size_t)(nt >> 2) * 1024 + scale_lane_off(nt & 3);
+    }
+
+    // pairs of blocks; this wave's share
+    const int pairs = (k_tiles + 1) >> 1;
+    const int pp_begin = wave * pairs / FLAT_WAVES;
+    const int pp_end = (wave + 1) * pairs / FLAT_WAVES;
+
+    v4f acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    struct Frag {
+        v4i a[2];
+        v4i b[NT][2];
+        int sa, sb[NT];
+    };
+    auto load = [&](int pp, Frag& f) {
+        const int kt0 = 2 * pp, kt1 = 2 * pp + 1;
+        const bool has1 = kt1 < k_tiles;
+        f.a[0] = *(const v4i*)(a_row + kt0 * 64);
+        f.a[1] = has1 ? *(const v4i*)(a_row + kt1 * 64) : v4i{0, 0, 0, 0};
+        // pair pp of the tiled layout: K group pp / 2, pair pp % 2
+        const size_t unit_a = ((size_t)(pp >> 1) * nblk_a * 2 + (pp & 1)) * 512, unit_b = ((size_t)(pp >> 1) * nblk_b * 2 + (pp & 1)) * 512;
+        f.sa = *(const unsigned short*)(sfa + unit_a);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            f.b[t][0] = __builtin_nontemporal_load((const v4i*)(b_tile[t] + (long long)kt0 * 1024));
+            f.b[t][1] = has1 ? __builtin_nontemporal_load((const v4i*)(b_tile[t] + (long long)kt1 * 1024))
+                             : v4i{0, 0, 0, 0};
+            f.sb[t] = *(const unsigned short*)(sfb[t] + unit_b);
+        }
+    };
+    auto mma = [&](const Frag& f) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                (v8i{f.b[t][0].x, f.b[t][0].y, f.b[t][0].z, f.b[t][0].w, 0, 0, 0, 0}), (v8i{f.a[0].x, f.a[0].y, f.a[0].z, f.a[0].w, 0, 0, 0, 0}),
+                acc[t], 4, 4, 0, f.sb[t], 0, f.sa);
+            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                (v8i{f.b[t][1].x, f.b[t][1].y, f.b[t][1].z, f.b[t][1].w, 0, 0, 0, 0}), (v8i{f.a[1].x, f.a[1].y, f.a[1].z, f.a[1].w, 0, 0, 0, 0}),
+                acc[t], 4, 4, 1, f.sb[t], 1, f.sa);
+        }
+    };
+
+    if (pp_begin < pp_end) {
+        Frag f0, f1;
+        load(pp_begin, f0);
+        int pp = pp_begin;
+        while (true) {
+            if (pp + 1 < pp_end) load(pp + 1, f1);
+            mma(f0);
+            if (++pp >= pp_end) break;
+            if (pp + 1 < pp_end) load(pp + 1, f0);
+            mma(f1);
+            if (++pp >= pp_end) break;
+        }
+    }
+
+#pragma unroll
+    for (int t = 0; t < NT; ++t) red[wave][t][lane] = acc[t];
+    __syncthreads();
+
+    if (finisher) {
+        v4f s = red[0][wave][lane];
+#pragma unroll
+        for (int w = 1; w < FLAT_WAVES; ++w) s += red[w][wave][lane];
+        const long long ci = (long long)batch * p.c_batch + (long long)cm * p.ldc + cn;
+        if constexpr (CDT == C_BF16) {
+            unsigned short* dst = (unsigned short*)p.c + ci;
+            if ((p.ldc & 3) == 0 && (((uintptr_t)p.c + 2 * (long long)batch * p.c_batch) & 7) == 0) {
+                *(v4u16*)dst = v4u16{bf16_bits(s.x), bf16_bits(s.y), bf16_bits(s.z), bf16_bits(s.w)};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[e] = bf16_bits(s[e]);
+            }
+        } else {
+            float* dst = (float*)p.c + ci;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[e] = s[e];
+        }
+    }
+}
+
 }  // namespace a8w8

@@ -112,6 +112,13 @@ A8W8_API int a16w16_flatmm(const a8w8_gemm_args* args, void* hip_stream);
  * MX_E8M0_1x32 (row-major scales, general kernel) or MX_E8M0_TILED (MFMA kernels when k % 256 == 0 and rows
  * are 16-byte aligned). */
 A8W8_API int a4w4_gemm(const a8w8_gemm_args* args, void* hip_stream);
+/* MXFP4 skinny-M GEMM over pre-shuffled weights (no counterpart in the reference, which has neither an FP4
+ * program nor a flat one for it; it is a8w8_flatmm for the FP4 form of the same instruction).  A [batch, m, k/2
+ * bytes] with m <= 64; B pre-shuffled as the byte matrix it is -- a8w8_preshuffle_b[_device](b, out, n, k/2) --
+ * with b_preshuffled != 0; sfa, sfb E8M0 in the MX_E8M0_TILED layout (a4w4_quantize_mx(tiled) or
+ * a8w8_mx_tile_scales), scale_mode = MX_E8M0_TILED; n % 16 == 0, k % 128 == 0; m, n, k and the strides count
+ * elements; a, b, sfa, sfb and the rows of A 16-byte aligned.  B is streamed once with 16-byte non-temporal loads. */
+A8W8_API int a4w4_flatmm(const a8w8_gemm_args* args, void* hip_stream);
 /* fp32 rows -> packed E2M1 + E8M0 scales: e = clamp(ceil(log2(amax32/6)), -127, 127), row-major scales
  * scale[r*(k/32) + p/32] or (tiled != 0) the MX_TILED layout. */
 A8W8_API int a4w4_quantize_mx(const float* src_dev, int rows, int k, int ld, uint8_t* q_dev, uint8_t* scale_dev,

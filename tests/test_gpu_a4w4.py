@@ -99,3 +99,61 @@ def test_full_size_8192(orc):
     e_np = orc.mx_untile_scales(ta.cpu().numpy(), m, k)          # row-major scales of A, to permute and re-tile
     tp = g.mx_tile_scales(dev(e_np[perm.cpu().numpy()]))
     assert torch.equal(g.gemm_a4w4(qa_p, qb, tp, tb), c[perm])
+
+
+# ---------------------------------------------------------------- flat (skinny-M) MXFP4 GEMM over pre-shuffled weights
+
+def _flat(qa, qb, ea, eb, c_dtype=g.FP32):
+    n = qb.shape[0]
+    bs = g.preshuffle_b_device(dev(qb))                     # the packed weight bytes [N, K/2], shuffled as bytes
+    c = g.flatmm_a4w4(dev(qa), bs, g.mx_tile_scales(dev(ea)), g.mx_tile_scales(dev(eb)), n, c_dtype=c_dtype)
+    torch.cuda.synchronize()
+    return c.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("shape", [(16, 256, 512), (16, 1024, 7168), (5, 48, 128), (33, 128, 384), (64, 4096, 1024), (1, 16, 128)])
+def test_flat_against_the_oracle(orc, shape):
+    m, n, k = shape
+    qa, ea = orc.quantize_mxfp4(_x(m, k, 61 + m))
+    qb, eb = orc.quantize_mxfp4(_x(n, k, 62 + n))
+    want = orc.gemm_ref_mxfp4(qa, qb, ea, eb)
+    exact, mag = _exact(orc, qa, qb, ea, eb)
+    got = _flat(qa, qb, ea, eb)
+    assert (np.abs(got - exact) <= MFMA_ACC_ERR * mag + 1e-30).all()
+    got16 = _flat(qa, qb, ea, eb, g.BF16)
+    miss = ~(np.abs(got16 - want) <= 1e-2 * np.abs(want) + 1e-2)
+    assert miss.mean() <= 1e-3
+    assert (np.abs(got16 - exact)[miss] <= MFMA_ACC_ERR * mag[miss] + 2.0 ** -8 * np.abs(exact)[miss]).all()
+
+
+@pytest.mark.parametrize("case", range(24))
+def test_flat_scale_bytes_reach_the_right_lane_and_block(orc, case):
+    """Random E2M1 codes with a distinct power of two per (row, 32-block): every value is a multiple of 0.5 of
+    magnitude <= 6 and the scales are 2^-1..2^1, so sums are exact in fp32 and any mix-up of row, block or the
+    pair's byte changes the result."""
+    r = np.random.default_rng(8000 + case)
+    m = int(r.integers(1, 65))
+    n = 16 * int(r.integers(1, 70))
+    k = 128 * int(r.integers(1, 24))
+    qa = r.integers(0, 256, (m, k // 2)).astype(np.uint8)
+    qb = r.integers(0, 256, (n, k // 2)).astype(np.uint8)
+    ea = r.integers(126, 129, (m, k // 32)).astype(np.uint8)
+    eb = r.integers(126, 129, (n, k // 32)).astype(np.uint8)
+    exact, _ = _exact(orc, qa, qb, ea, eb)
+    got = _flat(qa, qb, ea, eb)
+    bad = np.argwhere(got != exact.astype(np.float32))
+    assert bad.size == 0, f"{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
+    assert (_flat(qa, qb, ea, eb, g.BF16) == torch.from_numpy(exact.astype(np.float32)).to(torch.bfloat16).float().numpy()).all()
+
+
+def test_flat_rejects_what_it_cannot_run():
+    qa = torch.zeros((16, 64), dtype=torch.uint8, device="cuda")
+    bs = torch.zeros(16 * 64, dtype=torch.uint8, device="cuda")
+    t = torch.full((1024,), 127, dtype=torch.uint8, device="cuda")
+    assert g.flatmm_a4w4(qa, bs, t, t, 16).shape == (16, 16)
+    with pytest.raises(g.A8W8Error, match="aligned"):
+        g.flatmm_a4w4(torch.zeros((16, 64 + 8), dtype=torch.uint8, device="cuda")[:, :64], bs, t, t, 16)
+    with pytest.raises(g.A8W8Error):
+        g.flatmm_a4w4(torch.zeros((65, 64), dtype=torch.uint8, device="cuda"), bs, t, t, 16)
+    with pytest.raises(g.A8W8Error):
+        g.flatmm_a4w4(torch.zeros((16, 32), dtype=torch.uint8, device="cuda"), bs, t, t, 16)      # k = 64: not a whole block
