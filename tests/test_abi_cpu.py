@@ -174,6 +174,14 @@ def test_sibling_entry_points_reject_bad_arguments():
         b = _ok_args(mode=g.MX, m=64, n=64, k=256)
         mutate(b)
         assert L.a4w4_gemm(ref(b), None) == want, want
+    # a4w4_flatmm: pre-shuffled packed weights, tiled scales only
+    for mutate, want in [(lambda x: setattr(x, "b_preshuffled", 0), -6), (lambda x: setattr(x, "scale_mode", g.MX), -6),
+                         (lambda x: setattr(x, "m", 65), -2), (lambda x: setattr(x, "n", 250), -3),
+                         (lambda x: setattr(x, "k", 192), -3), (lambda x: setattr(x, "stride_a", 272), -5),
+                         (lambda x: setattr(x, "sfb", 0x5004), -5), (lambda x: setattr(x, "sfa", None), -1)]:
+        b = _ok_args(mode=g.MX_TILED, m=16, n=256, k=256, b_preshuffled=1)
+        mutate(b)
+        assert L.a4w4_flatmm(ref(b), None) == want, want
     # quantisers
     assert L.a8w8_quantize(None, 4, 32, 32, 0x2000, 0x3000, g.ROWCOL, 1, None) == -1
     assert L.a8w8_quantize(0x1000, 0, 32, 32, 0x2000, 0x3000, g.ROWCOL, 1, None) == -2
