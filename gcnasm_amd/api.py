@@ -243,7 +243,8 @@ def gemm_blockscale(a, b, sfa, sfb, c=None, c_dtype=FP32):
 
 
 def flatmm(a, b_shuffled, sfa, sfb, n, scale_mode=ROWCOL, c=None, c_dtype=BF16):
-    """Skinny-M GEMM over weights in the a8w8_preshuffle_b layout (flat u8 tensor of n*k bytes)."""
+    """Skinny-M GEMM over weights in the a8w8_preshuffle_b layout (flat u8 tensor of n*k bytes); scale_mode ROWCOL,
+    TENSOR or MX_TILED (MXFP8: both scale arrays in the tiled layout)."""
     g, c = _args_from_tensors(a, b_shuffled, sfa, sfb, scale_mode, c, c_dtype, 1, n=n)
     _check(lib().a8w8_flatmm(ctypes.byref(g), _stream()), "a8w8_flatmm")
     return c

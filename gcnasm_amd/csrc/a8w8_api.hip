@@ -316,13 +316,17 @@ int validate_flat(const a8w8_gemm_args* g)
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
     if (!g->b_preshuffled) return A8W8_ERR_BAD_MODE;
-    if (g->scale_mode != A8W8_SCALE_ROWCOL && g->scale_mode != A8W8_SCALE_TENSOR) return A8W8_ERR_BAD_MODE;
+    if (g->scale_mode != A8W8_SCALE_ROWCOL && g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_MX_E8M0_TILED)
+        return A8W8_ERR_BAD_MODE;
     const int st = validate_common(g);
     if (st != A8W8_OK) return st;
     if (g->m > 64) return A8W8_ERR_BAD_SHAPE;
     if (g->n % 16 != 0 || g->k % 64 != 0) return A8W8_ERR_BAD_GROUP;
     if (!aligned16(g->a) || !aligned16(g->b) || g->stride_a % 16 != 0) return A8W8_ERR_MISALIGNED;
     if (g->batch > 1 && (g->stride_a_batch % 16 != 0 || g->stride_b_batch % 16 != 0)) return A8W8_ERR_MISALIGNED;
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED &&
+        (!aligned16(g->sfa) || !aligned16(g->sfb) || (g->batch > 1 && (g->stride_sfa_batch % 16 != 0 || g->stride_sfb_batch % 16 != 0))))
+        return A8W8_ERR_MISALIGNED;
     return A8W8_OK;
 }
 
@@ -585,6 +589,8 @@ int a8w8_flatmm(const a8w8_gemm_args* g, void* hip_stream)
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
     const GemmParams p = make_params(g);
     hipStream_t s = (hipStream_t)hip_stream;
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED)
+        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_MXT>(p, g->batch, s) : launch_flat<C_FP32, MODE_MXT>(p, g->batch, s);
     const bool tensor = g->scale_mode == A8W8_SCALE_TENSOR;
     if (g->c_dtype == A8W8_C_BF16)
         return tensor ? launch_flat<C_BF16, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_BF16, MODE_ROWCOL>(p, g->batch, s);

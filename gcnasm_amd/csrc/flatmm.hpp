@@ -44,8 +44,8 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     if (finisher) {
         const float* sfa = (const float*)p.sfa + (long long)batch * p.sfa_batch;
         const float* sfb = (const float*)p.sfb + (long long)batch * p.sfb_batch;
-        if constexpr (MODE == MODE_BF16) {
-            // bf16 operands carry no scales
+        if constexpr (MODE == MODE_BF16 || MODE == MODE_MXT) {
+            // bf16 operands carry no scales; MX scales go into the MFMAs
         } else if constexpr (MODE == MODE_TENSOR) {
             sa = sfa[0] * sfb[0];
         } else {
@@ -59,6 +59,25 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     const uint8_t* b_tile[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) b_tile[t] = b_base + (long long)min(nt0 + t, n_tiles - 1) * k_tiles * 1024;
+    // MX scales in the tiled layout of the dense kernels (mx_tiled_index): a pair of K blocks is one 128-wide K
+    // step ks; lane (r16, kq) scales 32-block kq of its row, whose byte for step ks sits at
+    // ((ks / 4 * nblk + blk) * 2 + (ks / 2) % 2) * 512 + ((4x + y) * 4 + kq) * 8 + jp * 4 + par * 2 + ks % 2
+    // with, for row 16 i + r16 of a 64-row block, x = (2 i + r16 / 8) % 4, y = r16 % 4, jp = i / 2, par = (r16 / 4) % 2
+    const uint8_t* mx_a = nullptr;
+    const uint8_t* mx_b[NT];
+    int mx_nblk_a = 1, mx_nblk_b = 1;
+    if constexpr (MODE == MODE_MXT) {
+        auto lane_off = [&](int i) { return ((4 * ((2 * i + (r16 >> 3)) & 3) + (r16 & 3)) * 4 + kq) * 8 + (i >> 1) * 4 + ((r16 >> 2) & 1) * 2; };
+        const int m_tile = blockIdx.y;
+        mx_nblk_a = (p.m + 63) >> 6;
+        mx_nblk_b = (p.n + 63) >> 6;
+        mx_a = (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch + (size_t)(m_tile >> 2) * 1024 + lane_off(m_tile & 3);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int nt = min(nt0 + t, n_tiles - 1);
+            mx_b[t] = (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch + (size_t)(nt >> 2) * 1024 + lane_off(nt & 3);
+        }
+    }
 
     // K blocks are consumed in pairs; this wave's share of the pairs
     const int pairs = (k_tiles + 1) >> 1;
@@ -72,17 +91,25 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     struct Frag {
         v4i a[2];
         v4i b[NT][2];
+        int sa, sb[NT];         // MX: the step's E8M0 byte of this lane's row and 32-block
     };
     auto load = [&](int pp, Frag& f) {
         const int kt0 = 2 * pp, kt1 = 2 * pp + 1;
         const bool has1 = kt1 < k_tiles;
         f.a[0] = *(const v4i*)(a_row + kt0 * 64);
         f.a[1] = has1 ? *(const v4i*)(a_row + kt1 * 64) : v4i{0, 0, 0, 0};
+        size_t unit_a = 0, unit_b = 0;
+        if constexpr (MODE == MODE_MXT) {
+            unit_a = ((size_t)(pp >> 2) * mx_nblk_a * 2 + ((pp >> 1) & 1)) * 512 + (pp & 1);
+            unit_b = ((size_t)(pp >> 2) * mx_nblk_b * 2 + ((pp >> 1) & 1)) * 512 + (pp & 1);
+            f.sa = mx_a[unit_a];
+        }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             f.b[t][0] = __builtin_nontemporal_load((const v4i*)(b_tile[t] + (long long)kt0 * 1024));
             f.b[t][1] = has1 ? __builtin_nontemporal_load((const v4i*)(b_tile[t] + (long long)kt1 * 1024))
                              : v4i{0, 0, 0, 0};
+            if constexpr (MODE == MODE_MXT) f.sb[t] = mx_b[t][unit_b];
         }
     };
     auto mma = [&](const Frag& f) {
@@ -97,6 +124,8 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
                                                                  __builtin_bit_cast(v8bf, f.a[0]), acc[t], 0, 0, 0);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, f.b[t][1]),
                                                                  __builtin_bit_cast(v8bf, f.a[1]), acc[t], 0, 0, 0);
+            } else if constexpr (MODE == MODE_MXT) {
+                acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[t], 0, 0, 0, f.sb[t], 0, f.sa);
             } else {
                 acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[t], 0, 0, 0, 0, 0, 0);
             }

@@ -29,3 +29,42 @@ def test_flatmm_exact_integers(orc):
     got = run_flatmm(a, g.preshuffle_b(b), np.ones(1, np.float32), np.ones(1, np.float32), n, mode=g.TENSOR,
                      c_dtype=g.FP32)
     assert (got == want).all()
+
+
+# ---------------------------------------------------------------- MXFP8: E8M0 scales in the tiled layout
+
+def _flat_mx(a, b, ea, eb, c_dtype=g.FP32):
+    import torch
+    from gpu_util import dev
+    bs = g.preshuffle_b_device(dev(b))
+    c = g.flatmm(dev(a), bs, g.mx_tile_scales(dev(ea)), g.mx_tile_scales(dev(eb)), b.shape[0], scale_mode=g.MX_TILED, c_dtype=c_dtype)
+    torch.cuda.synchronize()
+    return c.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("shape", [(16, 256, 512), (16, 1024, 7168), (5, 48, 192), (33, 128, 256), (64, 2048, 1024), (1, 16, 64)])
+def test_flatmm_mx_against_the_oracle(orc, shape):
+    m, n, k = shape
+    a, b, ea, eb = datagen.mx(m, n, k, seed=900 + n)
+    want = orc.gemm_ref(a, b, ea, eb, orc.MX)
+    exact, mag = exact64(orc, a, b, ea, eb, g.MX)
+    assert_fp32_accurate(_flat_mx(a, b, ea, eb), exact, mag)
+    assert_close(_flat_mx(a, b, ea, eb, g.BF16), want, f"flatmm mx {shape}", exact=exact, mag=mag)
+
+
+@pytest.mark.parametrize("case", range(24))
+def test_flatmm_mx_scale_bytes_reach_the_right_lane_and_step(orc, case):
+    """Small integers with a distinct power of two per (row, 32-block): sums are exact in fp32, so any mix-up of
+    row, block or K step changes the result."""
+    r = np.random.default_rng(8100 + case)
+    m = int(r.integers(1, 65))
+    n = 16 * int(r.integers(1, 70))
+    k = 64 * int(r.integers(1, 40))
+    a, b = datagen.small_ints(m, n, k, seed=8200 + case)
+    ea = r.integers(125, 130, (m, k // 32)).astype(np.uint8)
+    eb = r.integers(125, 130, (n, k // 32)).astype(np.uint8)
+    A = orc.decode(a).astype(np.float64) * np.repeat(np.exp2(ea.astype(np.float64) - 127), 32, axis=1)
+    B = orc.decode(b).astype(np.float64) * np.repeat(np.exp2(eb.astype(np.float64) - 127), 32, axis=1)
+    got = _flat_mx(a, b, ea, eb)
+    bad = np.argwhere(got != (A @ B.T).astype(np.float32))
+    assert bad.size == 0, f"{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
