@@ -316,7 +316,8 @@ int validate_flat(const a8w8_gemm_args* g)
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
     if (!g->b_preshuffled) return A8W8_ERR_BAD_MODE;
-    if (g->scale_mode != A8W8_SCALE_ROWCOL && g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_MX_E8M0_TILED)
+    if (g->scale_mode != A8W8_SCALE_ROWCOL && g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_MX_E8M0_TILED &&
+        g->scale_mode != A8W8_SCALE_BLOCK_1x128_128x128)
         return A8W8_ERR_BAD_MODE;
     const int st = validate_common(g);
     if (st != A8W8_OK) return st;
@@ -591,6 +592,8 @@ int a8w8_flatmm(const a8w8_gemm_args* g, void* hip_stream)
     hipStream_t s = (hipStream_t)hip_stream;
     if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED)
         return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_MXT>(p, g->batch, s) : launch_flat<C_FP32, MODE_MXT>(p, g->batch, s);
+    if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128)
+        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_BLOCK>(p, g->batch, s) : launch_flat<C_FP32, MODE_BLOCK>(p, g->batch, s);
     const bool tensor = g->scale_mode == A8W8_SCALE_TENSOR;
     if (g->c_dtype == A8W8_C_BF16)
         return tensor ? launch_flat<C_BF16, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_BF16, MODE_ROWCOL>(p, g->batch, s);

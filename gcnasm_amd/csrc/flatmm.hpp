@@ -44,8 +44,8 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     if (finisher) {
         const float* sfa = (const float*)p.sfa + (long long)batch * p.sfa_batch;
         const float* sfb = (const float*)p.sfb + (long long)batch * p.sfb_batch;
-        if constexpr (MODE == MODE_BF16 || MODE == MODE_MXT) {
-            // bf16 operands carry no scales; MX scales go into the MFMAs
+        if constexpr (MODE == MODE_BF16 || MODE == MODE_MXT || MODE == MODE_BLOCK) {
+            // bf16 operands carry no scales; MX scales go into the MFMAs, block scales into the K loop
         } else if constexpr (MODE == MODE_TENSOR) {
             sa = sfa[0] * sfb[0];
         } else {
@@ -79,6 +79,17 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         }
     }
 
+    // block scales (1x128 for A, 128x128 for B; the reference's layout): a pair of K blocks is one 128-wide scale
+    // group, lane (r16, .) needs sfa[group][row m0 + r16] and, per weight tile, sfb[tile's 128-row block][group]
+    const float* blk_a = nullptr;
+    const float* blk_b[NT];
+    if constexpr (MODE == MODE_BLOCK) {
+        blk_a = (const float*)p.sfa + (long long)batch * p.sfa_batch + min(m0 + r16, p.m - 1);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            blk_b[t] = (const float*)p.sfb + (long long)batch * p.sfb_batch + (long long)(min(nt0 + t, n_tiles - 1) >> 3) * p.stride_sfb;
+    }
+
     // K blocks are consumed in pairs; this wave's share of the pairs
     const int pairs = (k_tiles + 1) >> 1;
     const int pp_begin = wave * pairs / FLAT_WAVES;
@@ -92,6 +103,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         v4i a[2];
         v4i b[NT][2];
         int sa, sb[NT];         // MX: the step's E8M0 byte of this lane's row and 32-block
+        float fs[NT];           // block scales: sfa * sfb of the pair's scale group
     };
     auto load = [&](int pp, Frag& f) {
         const int kt0 = 2 * pp, kt1 = 2 * pp + 1;
@@ -104,12 +116,15 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
             unit_b = ((size_t)(pp >> 2) * mx_nblk_b * 2 + ((pp >> 1) & 1)) * 512 + (pp & 1);
             f.sa = mx_a[unit_a];
         }
+        float blk_sa = 1.f;
+        if constexpr (MODE == MODE_BLOCK) blk_sa = blk_a[(long long)pp * p.stride_sfa];
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             f.b[t][0] = __builtin_nontemporal_load((const v4i*)(b_tile[t] + (long long)kt0 * 1024));
             f.b[t][1] = has1 ? __builtin_nontemporal_load((const v4i*)(b_tile[t] + (long long)kt1 * 1024))
                              : v4i{0, 0, 0, 0};
             if constexpr (MODE == MODE_MXT) f.sb[t] = mx_b[t][unit_b];
+            if constexpr (MODE == MODE_BLOCK) f.fs[t] = blk_sa * blk_b[t][pp];
         }
     };
     auto mma = [&](const Frag& f) {
@@ -124,6 +139,10 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
                                                                  __builtin_bit_cast(v8bf, f.a[0]), acc[t], 0, 0, 0);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, f.b[t][1]),
                                                                  __builtin_bit_cast(v8bf, f.a[1]), acc[t], 0, 0, 0);
+            } else if constexpr (MODE == MODE_BLOCK) {
+                // each 128-wide K group yields a partial tile that is rescaled into the running sum
+                const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                acc[t] += part * f.fs[t];
             } else if constexpr (MODE == MODE_MXT) {
                 acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[t], 0, 0, 0, f.sb[t], 0, f.sa);
             } else {

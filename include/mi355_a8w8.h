@@ -132,7 +132,8 @@ A8W8_API int a8w8_gemm_blockscale(const a8w8_gemm_args* args, void* hip_stream);
 
 /* Skinny-M GEMM over pre-shuffled weights (the flatmm_a8w8_gfx950 program listed at
  * opus_fmm/README.md:9, built by opus_fmm/rebuild.sh:3-13).  Requires b_preshuffled != 0,
- * scale_mode ROWCOL, TENSOR or MX_E8M0_TILED (MXFP8: both scale arrays in the tiled layout, 16-byte aligned),
+ * scale_mode ROWCOL, TENSOR, BLOCK_1x128_128x128 (scale arrays as for a8w8_gemm_blockscale; n, k % 128 == 0) or
+ * MX_E8M0_TILED (MXFP8: both scale arrays in the tiled layout, 16-byte aligned),
  * m <= 64, n % 16 == 0, k % 64 == 0, a, b and the rows of A 16-byte aligned (A8W8_ERR_MISALIGNED otherwise).
  * B is streamed once with 16-byte non-temporal loads. */
 A8W8_API int a8w8_flatmm(const a8w8_gemm_args* args, void* hip_stream);

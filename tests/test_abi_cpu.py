@@ -63,7 +63,7 @@ def test_null_struct_and_mx_group():
 def test_flatmm_preconditions():
     a = _ok_args(mode=g.ROWCOL, m=16, n=256, k=256, b_preshuffled=1)
     assert g.kernel_name(a) == "flatmm_a8w8"
-    for mutate, want in [(lambda x: setattr(x, "b_preshuffled", 0), -6), (lambda x: setattr(x, "scale_mode", g.BLOCK), -6),
+    for mutate, want in [(lambda x: setattr(x, "b_preshuffled", 0), -6), (lambda x: setattr(x, "scale_mode", g.MX), -6),
                          (lambda x: setattr(x, "m", 65), -2), (lambda x: setattr(x, "n", 250), -3),
                          (lambda x: setattr(x, "k", 96), -3), (lambda x: setattr(x, "a", 0x1001), -5)]:
         b = _ok_args(mode=g.ROWCOL, m=16, n=256, k=256, b_preshuffled=1)

@@ -68,3 +68,47 @@ def test_flatmm_mx_scale_bytes_reach_the_right_lane_and_step(orc, case):
     got = _flat_mx(a, b, ea, eb)
     bad = np.argwhere(got != (A @ B.T).astype(np.float32))
     assert bad.size == 0, f"{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
+
+
+# ---------------------------------------------------------------- block scales (1x128 / 128x128), the reference's layout
+
+@pytest.mark.parametrize("shape", [(16, 256, 512), (16, 1024, 7168), (5, 128, 128), (33, 384, 256), (64, 2048, 1024)])
+def test_flatmm_block_scales(orc, shape):
+    import torch
+    from gpu_util import dev
+    m, n, k = shape
+    a, b, sfa, sfb = datagen.block_scaled(m, n, k, seed=950 + n)
+    want = orc.gemm_ref(a, b, sfa, sfb, orc.BLOCK)
+    bs = g.preshuffle_b_device(dev(b))
+    for c_dtype in (g.FP32, g.BF16):
+        c = g.flatmm(dev(a), bs, dev(sfa), dev(sfb), n, scale_mode=g.BLOCK, c_dtype=c_dtype)
+        torch.cuda.synchronize()
+        got = c.float().cpu().numpy()
+        if c_dtype == g.FP32:
+            assert_fp32_accurate(got, *exact64(orc, a, b, sfa, sfb, g.BLOCK))
+        else:
+            assert_close(got, want, f"flatmm block {shape}")
+    # the reference's own inputs and check (host.cc:46-63, 207-210): every element within 1e-3 absolute
+    a, b, sfa, sfb = datagen.reference_style(m, n, k)
+    c = g.flatmm(dev(a), g.preshuffle_b_device(dev(b)), dev(sfa), dev(sfb), n, scale_mode=g.BLOCK, c_dtype=g.FP32)
+    assert orc.count_abs_mismatch(orc.gemm_ref(a, b, sfa, sfb, orc.BLOCK), c.cpu().numpy(), 1e-3) == 0
+
+
+@pytest.mark.parametrize("case", range(16))
+def test_flatmm_block_scales_exact(orc, case):
+    """Small integers, power-of-two scales distinct per (row, K group) and per (128-row block, K group)."""
+    import torch
+    from gpu_util import dev
+    r = np.random.default_rng(8300 + case)
+    m = int(r.integers(1, 65))
+    n = 128 * int(r.integers(1, 9))
+    k = 128 * int(r.integers(1, 20))
+    a, b = datagen.small_ints(m, n, k, seed=8400 + case)
+    sfa = np.exp2(r.integers(-2, 3, (k // 128, m))).astype(np.float32)
+    sfb = np.exp2(r.integers(-2, 3, (n // 128, k // 128))).astype(np.float32)
+    A = orc.decode(a).astype(np.float64) * np.repeat(sfa.T.astype(np.float64), 128, axis=1)
+    B = orc.decode(b).astype(np.float64) * np.repeat(np.repeat(sfb.astype(np.float64), 128, axis=0), 128, axis=1)
+    c = g.flatmm(dev(a), g.preshuffle_b_device(dev(b)), dev(sfa), dev(sfb), n, scale_mode=g.BLOCK, c_dtype=g.FP32)
+    torch.cuda.synchronize()
+    bad = np.argwhere(c.cpu().numpy() != (A @ B.T).astype(np.float32))
+    assert bad.size == 0, f"{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
