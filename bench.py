@@ -290,6 +290,51 @@ def run_reference_program_sizes(torch, g, steps, warmup, seed):
     return out
 
 
+def run_flat_variants(torch, g, steps, warmup, seed):
+    """The decode shape of the flat workload (16 x 16384 x 7168) in the other scale modes and in MXFP4, each with
+    rotating copies of the pre-shuffled weights (larger than the Infinity Cache together), priced against HBM."""
+    import ctypes
+    m, n, k = 16, 16384, 7168
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    xa = torch.randn((m, k), generator=gen, device="cuda")
+    xb = torch.randn((n, k), generator=gen, device="cuda")
+    L = g.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    out = []
+    for name, fp4 in (("flatmm_mx_tiled", False), ("flatmm_block", False), ("flatmm_mxfp4", True)):
+        if fp4:
+            (a, sfa), (b, sfb) = g.quantize_mxfp4(xa, tiled=True), g.quantize_mxfp4(xb, tiled=True)
+            mode, entry, wbytes, sbytes = g.MX_TILED, L.a4w4_flatmm, n * k // 2, n * k // 32 + m * k // 32
+        elif name == "flatmm_mx_tiled":
+            (a, sfa), (b, sfb) = g.quantize(xa, g.MX_TILED), g.quantize(xb, g.MX_TILED)
+            mode, entry, wbytes, sbytes = g.MX_TILED, L.a8w8_flatmm, n * k, n * k // 32 + m * k // 32
+        else:
+            (a, sfa), (b, sfb) = g.quantize(xa, g.BLOCK, 1), g.quantize(xb, g.BLOCK, 128)
+            mode, entry, wbytes, sbytes = g.BLOCK, L.a8w8_flatmm, n * k, 4 * (n // 128) * (k // 128) + 4 * m * (k // 128)
+        bs = g.preshuffle_b_device(b)
+        copies = [bs] + [bs.clone() for _ in range(3 if not fp4 else 7)]
+        args = [g.raw_gemm_args(a.data_ptr(), x.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, mode, g.BF16,
+                                b_preshuffled=1) for x in copies]
+        refs = [ctypes.byref(x) for x in args]
+        mask = len(copies) - 1
+
+        def fn(i, entry=entry, refs=refs, mask=mask):
+            if entry(refs[i & mask], stream) != 0:
+                raise RuntimeError("flat call failed")
+
+        ms, wall = time_best_of(torch, fn, steps, warmup)
+        abytes = wbytes + sbytes + a.numel() + 2 * m * n
+        out.append({"workload": f"{name}_{m}x{n}x{k}", "m": m, "n": n, "k": k, "kernel": "flatmm_a4w4" if fp4 else "flatmm_a8w8",
+                    "ms_per_launch": ms, "wall_ms_per_launch": wall, "algorithmic_bytes": abytes, "gbs": abytes / ms / 1e6,
+                    "frac_hbm_peak": abytes / ms / 1e6 / PEAK_HBM_GBS,
+                    "note": f"{len(copies)} rotating copies of the weights ({len(copies) * wbytes // 10**6} MB)"})
+        del copies, args, refs, bs, a, b, sfa, sfb
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(name, inp, c_gpu, torch, budget_s=15.0):
     """Times the oracle (port of the reference's host GEMM: per-MAC software fp8 decode,
     OpenMP over (i, j), gemm_a8w8_blockscale_host.cc:66-90) on the first rows of the same
@@ -381,6 +426,7 @@ def main():
             torch.cuda.empty_cache()
         others.extend(run_quantizers(torch, g, args.steps, args.warmup, args.seed + 2))
         others.extend(run_reference_program_sizes(torch, g, args.steps, args.warmup, args.seed + 3))
+        others.extend(run_flat_variants(torch, g, args.steps, args.warmup, args.seed + 4))
         line["other_workloads"] = others
     print(json.dumps(line))
 
