@@ -26,6 +26,13 @@ def test_fake_implementations_propagate_shapes():
         assert q.shape == (256, 1024) and q.dtype == torch.uint8 and sc.shape == shape and sc.dtype == dt
     h = torch.empty((64, 128), dtype=torch.bfloat16, device="meta")
     assert torch.ops.mi355_a8w8.gemm_a16w16(h, h, True).shape == (64, 64)
+    q, sc = torch.ops.mi355_a8w8.quantize_mxfp4(x, True)
+    assert q.shape == (256, 512) and sc.shape == (g.mx_tiled_bytes(256, 1024),)
+    q2, sc2 = torch.ops.mi355_a8w8.quantize_mxfp4(x, False)
+    assert sc2.shape == (256, 32)
+    assert torch.ops.mi355_a8w8.gemm_a4w4(q, q[:64], sc, sc, g.MX_TILED, False).shape == (256, 64)
+    c = torch.ops.mi355_a8w8.flatmm_a4w4(q[:16], q.reshape(-1), sc, sc, 256, True)
+    assert c.shape == (16, 256) and c.dtype == torch.float32
 
 
 @pytest.mark.gpu
@@ -44,3 +51,9 @@ def test_operators_run_the_library(orc):
     np.testing.assert_allclose(cf.cpu().numpy(), ref[:16], rtol=1e-3, atol=1e-3 * np.abs(ref).max())
     h = xa.to(torch.bfloat16)
     assert torch.equal(torch.ops.mi355_a8w8.gemm_a16w16(h, h, False), g.gemm_a16w16(h, h))
+    q4a, s4a = torch.ops.mi355_a8w8.quantize_mxfp4(xa[:16].contiguous(), True)
+    q4b, s4b = torch.ops.mi355_a8w8.quantize_mxfp4(xb, True)
+    c4 = torch.ops.mi355_a8w8.gemm_a4w4(q4a, q4b, s4a, s4b, g.MX_TILED, True)
+    f4 = torch.ops.mi355_a8w8.flatmm_a4w4(q4a, g.preshuffle_b_device(q4b), s4a, s4b, 384, True)
+    assert torch.equal(c4, g.gemm_a4w4(q4a, q4b, s4a, s4b, c_dtype=g.FP32))
+    np.testing.assert_allclose(f4.cpu().numpy(), c4.cpu().numpy(), rtol=1e-4, atol=1e-3)
