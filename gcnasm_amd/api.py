@@ -175,9 +175,10 @@ def _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, b_preshuffled, n=
     return g, c
 
 
-def gemm(a, b, sfa, sfb, scale_mode, c=None, c_dtype=BF16):
-    """C = dequant(A) @ dequant(B)^T through a8w8_gemm.  a [.., M, K] u8, b [.., N, K] u8 on the GPU."""
-    g, c = _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, 0)
+def gemm(a, b, sfa, sfb, scale_mode, c=None, c_dtype=BF16, n=None):
+    """C = dequant(A) @ dequant(B)^T through a8w8_gemm.  a [.., M, K] u8, b [.., N, K] u8 on the GPU; with `n` given,
+    b is the flat pre-shuffled weight (preshuffle_b_device) of n rows."""
+    g, c = _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, 0 if n is None else 1, n=n)
     _check(lib().a8w8_gemm(ctypes.byref(g), _stream()), "a8w8_gemm")
     return c
 

@@ -80,7 +80,10 @@ GemmParams make_params(const a8w8_gemm_args* g)
     p.sfa = g->sfa;
     p.sfb = g->sfb;
     p.m = g->m; p.n = g->n; p.k = g->k;
-    p.lda = g->stride_a; p.ldb = g->stride_b; p.ldc = g->stride_c;
+    p.lda = g->stride_a; p.ldc = g->stride_c;
+    // pre-shuffled B: 16 rows span 16 k bytes and a 128-wide K step two 1 KiB blocks
+    p.ldb = g->b_preshuffled ? g->k : g->stride_b;
+    p.b_kshift = g->b_preshuffled ? 11 : 7;
     p.a_batch = g->stride_a_batch; p.b_batch = g->stride_b_batch; p.c_batch = g->stride_c_batch;
     p.sfa_batch = g->stride_sfa_batch; p.sfb_batch = g->stride_sfb_batch;
     p.stride_sfa = g->stride_sfa; p.stride_sfb = g->stride_sfb;
@@ -104,6 +107,17 @@ bool tiled_ok(const a8w8_gemm_args* g)
     return g->k % BK == 0 && g->stride_a % 16 == 0 && g->stride_b % 16 == 0 && aligned16(g->a) && aligned16(g->b) &&
            (g->batch == 1 || (g->stride_a_batch % 16 == 0 && g->stride_b_batch % 16 == 0)) &&
            (long long)((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 31);
+}
+
+// B in the a8w8_preshuffle_b layout is read by the MFMA kernels only (the one-thread-per-element kernel reads
+// row-major B): whole 16-row groups and 128-wide K steps, aligned pointers.
+int validate_shuffled_b(const a8w8_gemm_args* g)
+{
+    if (!g->b_preshuffled) return A8W8_OK;
+    if (g->n % 16 != 0 || g->k % BK != 0) return A8W8_ERR_BAD_GROUP;
+    a8w8_gemm_args rows = *g;
+    rows.stride_b = g->k;           // what the alignment checks of tiled_ok should see for B
+    return tiled_ok(&rows) ? A8W8_OK : A8W8_ERR_MISALIGNED;
 }
 
 // The persistent kernel pipelines two K steps ahead and indexes work items with an int.
@@ -378,11 +392,15 @@ int launch_flat_f4(const GemmParams& p, int batch, hipStream_t stream)
 
 extern "C" {
 
-int a8w8_gemm(const a8w8_gemm_args* g, void* hip_stream)
+int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream)
 {
-    const int st = validate_common(g);
+    const int st = validate_common(args);
     if (st != A8W8_OK) return st;
-    if (g->b_preshuffled) return A8W8_ERR_BAD_MODE;
+    a8w8_gemm_args local = *args;
+    if (local.b_preshuffled) local.stride_b = local.k;      // stride_b is not read for shuffled weights
+    const a8w8_gemm_args* g = &local;
+    const int shuf = validate_shuffled_b(g);
+    if (shuf != A8W8_OK) return shuf;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
     const GemmParams p = make_params(g);
     hipStream_t s = (hipStream_t)hip_stream;
@@ -579,7 +597,6 @@ int a8w8_gemm_blockscale(const a8w8_gemm_args* g, void* hip_stream)
     if (!g) return A8W8_ERR_NULL_POINTER;
     a8w8_gemm_args local = *g;
     local.scale_mode = A8W8_SCALE_BLOCK_1x128_128x128;
-    local.b_preshuffled = 0;
     return a8w8_gemm(&local, hip_stream);
 }
 
@@ -907,8 +924,9 @@ const char* a8w8_status_string(int status)
 const char* a8w8_kernel_name(const a8w8_gemm_args* g)
 {
     if (!g) return nullptr;
-    if (g->b_preshuffled) return validate_flat(g) == A8W8_OK ? "flatmm_a8w8" : nullptr;
-    if (validate_common(g) != A8W8_OK) return nullptr;
+    // pre-shuffled B: the flat GEMM when its preconditions hold (m <= 64, ...), else a8w8_gemm on shuffled weights
+    if (g->b_preshuffled && validate_flat(g) == A8W8_OK) return "flatmm_a8w8";
+    if (validate_common(g) != A8W8_OK || validate_shuffled_b(g) != A8W8_OK) return nullptr;
     if (!tiled_ok(g)) return "gemm_a8w8_general";
     if (small_ok(g)) return "gemm_a8w8_tile128";
     if (wide_ok(g)) return "gemm_a8w8_wide";

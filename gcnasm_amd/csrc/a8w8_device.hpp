@@ -53,6 +53,9 @@ struct GemmParams {
     long long a_batch, b_batch, c_batch, sfa_batch, sfb_batch;
     int stride_sfa, stride_sfb;
     int tiles_m, tiles_n;
+    // log2 of the byte distance between consecutive 128-wide K steps of a row of B: 7 for row-major B, 11 for B in
+    // the a8w8_preshuffle_b layout (two 1 KiB blocks per step; ldb = k there, so that 16 r rows are 16 r * ldb bytes)
+    int b_kshift;
 };
 
 // Raw buffer descriptor over [base, base + bytes): dword 3 = 0x00020000 selects the raw
@@ -60,6 +63,19 @@ struct GemmParams {
 A8W8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes)
 {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+// Byte offset, inside B, of the 16-byte K piece at `piece_bytes` (0, 16, .. 112) of the first K step of row `row`.
+// Pre-shuffled B [n/16][k/64][4][16][16 B]: the piece's 64-wide K block, its quarter of the block, the row's slot.
+A8W8_DEV int b_lane_offset(const GemmParams& p, int row, int piece_bytes)
+{
+    if (p.b_kshift == 7) return __mul24(row, p.ldb) + piece_bytes;
+    return (row >> 4) * (p.k << 4) + ((piece_bytes >> 6) << 10) + (((piece_bytes >> 4) & 3) << 8) + ((row & 15) << 4);
+}
+// Extent of one batch entry of B for its buffer descriptor (rows past n read as zero in both layouts).
+A8W8_DEV uint32_t b_extent_bytes(const GemmParams& p)
+{
+    return p.b_kshift == 7 ? (uint32_t)(p.n - 1) * p.ldb + p.k : (uint32_t)p.n * p.k;
 }
 
 // 16 bytes per lane straight from global memory into LDS.  The hardware places lane i's

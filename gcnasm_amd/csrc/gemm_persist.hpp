@@ -123,9 +123,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         tile_of_block(item - batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
         const int m0 = tm * BM, n0 = tn * BN;
         rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
-        rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, (uint32_t)(p.n - 1) * p.ldb + p.k);
+        rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, b_extent_bytes(p));
         ld_voff_a = __mul24(m0 + ld_row, p.lda) + ld_piece16;
-        ld_voff_b = __mul24(n0 + ld_row, p.ldb) + ld_piece16;
+        ld_voff_b = b_lane_offset(p, n0 + ld_row, ld_piece16);
         if constexpr (MODE == MODE_MX) {
             const bool is_b = wave >= 4;           // waves 0-3 stage A-row scales, 4-7 B-row scales
             const int rows = is_b ? p.n : p.m;
@@ -149,7 +149,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             load_to_lds_16(rsrc_a, s + which * 8192, ld_voff_a, koff + 64 * which * p.lda);
         } else {
             const int j = which == 4 ? 0 : which == 5 ? 2 : which == 6 ? 1 : 3;
-            load_to_lds_16(rsrc_b, s + OPERAND_BYTES + j * 8192, ld_voff_b, koff + 64 * j * p.ldb);
+            load_to_lds_16(rsrc_b, s + OPERAND_BYTES + j * 8192, ld_voff_b, (kstep << p.b_kshift) + 64 * j * p.ldb);
         }
     };
     auto issue_mx_group = [&](int group) __attribute__((always_inline)) {

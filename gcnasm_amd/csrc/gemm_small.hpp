@@ -66,7 +66,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     const float* sfa_f = (const float*)p.sfa + (long long)batch * p.sfa_batch;
     const float* sfb_f = (const float*)p.sfb + (long long)batch * p.sfb_batch;
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(a_base, (uint32_t)(p.m - 1) * p.lda + p.k);
-    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(b_base, (uint32_t)(p.n - 1) * p.ldb + p.k);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(b_base, b_extent_bytes(p));
 
     // ---- global -> LDS.  A stage holds 16 A chunks then 16 B chunks of 1 KiB (8 rows x 128 B); wave w
     // fills chunks w, w+4, w+8, w+12 of each matrix.  Lane i of a load lands on row i/8, slot i%8 of its
@@ -77,7 +77,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         voff_a[j] = min(m0 + ld_row + 32 * j, p.m - 1) * p.lda + ld_piece16;
-        voff_b[j] = min(n0 + ld_row + 32 * j, p.n - 1) * p.ldb + ld_piece16;
+        voff_b[j] = b_lane_offset(p, min(n0 + ld_row + 32 * j, p.n - 1), ld_piece16);
     }
     // block mode: waves 0 and 1 fetch the step's 128 A-row scales (64 each), waves 2 and 3 the B scale
     // of the tile's 128 x 128 block (every lane the same dword: the stage's copy at +512 is the one read)
@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
         for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_a, s + j * 4096, voff_a[j], koff);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_b, s + SM_BM * BK + j * 4096, voff_b[j], koff);
+        for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_b, s + SM_BM * BK + j * 4096, voff_b[j], kstep << p.b_kshift);
         if constexpr (TILED_SCALES) {
             A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 1024;
             // the pair of 128-element K steps this step belongs to (FP8: two byte steps) or is (FP4: 256 elements)

@@ -62,7 +62,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
     const uint8_t* a_base = p.a + (long long)batch * p.a_batch;
     const uint8_t* b_base = p.b + (long long)batch * p.b_batch;
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(a_base, (uint32_t)(p.m - 1) * p.lda + p.k);
-    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(b_base, (uint32_t)(p.n - 1) * p.ldb + p.k);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(b_base, b_extent_bytes(p));
 
     // ---- global -> LDS assignment.  A stage holds 32 A chunks then 32 B chunks of 1 KiB
     // (8 rows x 128 B).  Wave w fills chunks w, w+8, w+16, w+24 of each matrix; lane i of
@@ -74,7 +74,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         voff_a[j] = min(m0 + ld_row + 64 * j, p.m - 1) * p.lda + ld_piece * 16;
-        voff_b[j] = min(n0 + ld_row + 64 * j, p.n - 1) * p.ldb + ld_piece * 16;
+        voff_b[j] = b_lane_offset(p, min(n0 + ld_row + 64 * j, p.n - 1), ld_piece * 16);
     }
     auto issue_stage = [&](int stage, int kstep) {
         A8W8_LDS char* s = (A8W8_LDS char*)smem + stage * STAGE_BYTES + wave * 1024;
@@ -82,7 +82,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_tile256(GemmParams 
 #pragma unroll
         for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_a, s + j * 8192, voff_a[j], koff);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_b, s + BM * BK + j * 8192, voff_b[j], koff);
+        for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_b, s + BM * BK + j * 8192, voff_b[j], kstep << p.b_kshift);
     };
 
     // ---- LDS -> register addresses.  The 16 x 16 x 128 FP8 MFMA takes, from lane

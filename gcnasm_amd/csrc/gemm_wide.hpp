@@ -148,11 +148,11 @@ gemm_a8w8_wide(PersistParams pp)
         int tm, tn;
         tile_of_block(item - batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
         rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
-        rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, (uint32_t)(p.n - 1) * p.ldb + p.k);
+        rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, b_extent_bytes(p));
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             ld_voff_a[h] = __mul24(tm * BM + 128 * h + ld_row, p.lda) + ld_piece16;
-            ld_voff_b[h] = __mul24(tn * BN + 128 * h + ld_row, p.ldb) + ld_piece16;
+            ld_voff_b[h] = b_lane_offset(p, tn * BN + 128 * h + ld_row, ld_piece16);
         }
     };
     // Load l (0..3) of quarter qt (0 aL, 1 aH, 2 bL, 3 bH) of the step at the load position.  A quarter
@@ -165,7 +165,7 @@ gemm_a8w8_wide(PersistParams pp)
         // four scalar offsets per operand and step (K step + 0, 32, 64 or 96 rows), each used twice
         const int rows = 64 * (qt & 1) + 32 * (l & 1);
         if (qt < 2) load_to_lds_16(rsrc_a, s, ld_voff_a[l >> 1], ld_ks * BK + rows * p.lda);
-        else load_to_lds_16(rsrc_b, s, ld_voff_b[l >> 1], ld_ks * BK + rows * p.ldb);
+        else load_to_lds_16(rsrc_b, s, ld_voff_b[l >> 1], (ld_ks << p.b_kshift) + rows * p.ldb);
     };
     auto advance_ld = [&]() __attribute__((always_inline)) {
         if (++ld_ks == nk) {

@@ -89,7 +89,9 @@ typedef struct {
  *   gemm_a8w8_blockscale_kernel<Traits><<<grid, 512>>>(kargs)   (host.cc:14-15, 249-257)
  * and the launches of the absent siblings gemm_a8w8_8wave (opus_gemm/rebuild.sh:3) for the
  * per-tensor and row/column modes.  Needs k % 128 == 0 and 16-byte aligned A/B rows for
- * the tiled kernels; other shapes run on a slower general kernel.  m, n edges are handled. */
+ * the tiled kernels; other shapes run on a slower general kernel.  m, n edges are handled.
+ * b_preshuffled != 0: B is in the a8w8_preshuffle_b layout (the weights a8w8_flatmm streams), so that one copy
+ * of the weights serves prefill and decode; needs n % 16 == 0, k % 128 == 0 and 16-byte aligned pointers. */
 A8W8_API int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream);
 
 /* The bf16 sibling (gemm_a16w16_8wave, the program opus_gemm/rebuild.sh:3-13 builds; its source is

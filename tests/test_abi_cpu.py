@@ -41,7 +41,6 @@ def _ok_args(mode=g.BLOCK, m=256, n=256, k=256, **kw):
     (lambda a: setattr(a, "stride_sfa", 8), -4),
     (lambda a: setattr(a, "scale_mode", 7), -6),
     (lambda a: setattr(a, "c_dtype", 3), -6),
-    (lambda a: setattr(a, "b_preshuffled", 1), -6),
 ])
 def test_gemm_rejects_bad_arguments(mutate, want):
     a = _ok_args()
@@ -71,6 +70,22 @@ def test_flatmm_preconditions():
         if b.k == 96:
             b.stride_a = 96
         assert g.lib().a8w8_flatmm(ctypes.byref(b), None) == want
+
+
+def test_gemm_on_shuffled_weights_preconditions():
+    """a8w8_gemm reads B in the flat GEMM's layout too: whole 16-row groups and 128-wide K steps, aligned pointers."""
+    L = g.lib()
+    ok = _ok_args(mode=g.ROWCOL, m=4096, n=4096, k=512, b_preshuffled=1)
+    ok.stride_b = 0                                           # not read for shuffled weights
+    assert g.kernel_name(ok) == "gemm_a8w8_wide"
+    assert g.kernel_name(_ok_args(mode=g.BLOCK, m=300, n=512, k=512, b_preshuffled=1)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL, m=16, n=256, k=256, b_preshuffled=1)) == "flatmm_a8w8"     # flat when it can
+    for mutate, want in [(lambda x: setattr(x, "n", 4088), -3), (lambda x: setattr(x, "k", 448), -3),
+                         (lambda x: setattr(x, "b", 0x2008), -5), (lambda x: setattr(x, "stride_a", 520), -5)]:
+        b = _ok_args(mode=g.ROWCOL, m=4096, n=4096, k=512, b_preshuffled=1)
+        mutate(b)
+        assert L.a8w8_gemm(ctypes.byref(b), None) == want, want
+        assert g.kernel_name(b) is None
 
 
 def test_kernel_selection():

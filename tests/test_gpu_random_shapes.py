@@ -38,11 +38,16 @@ def _padded(r, x, pad_choices, fill):
     return view, whole
 
 
+@pytest.mark.parametrize("shuffled", [False, True], ids=["row_major_b", "shuffled_b"])
 @pytest.mark.parametrize("case", range(CASES))
-def test_random_case(case):
+def test_random_case(case, shuffled):
+    """shuffled: the same sweep with B in the pre-shuffled layout of the flat GEMM (whole 16-row groups and 128-wide
+    K steps, aligned rows of A), which a8w8_gemm reads directly."""
     r = np.random.default_rng(9000 + case)
     mode = [g.TENSOR, g.ROWCOL, g.BLOCK, g.MX, g.MX_TILED][case % 5]
     m, n, k = _dims(r)
+    if shuffled:
+        n, k = -(-n // 16) * 16, max(128, k // 128 * 128)
     if mode == g.BLOCK:
         n = max(128, n // 128 * 128)            # the reference's block-scale program needs N and K in whole blocks
         k = max(128, k // 128 * 128)
@@ -73,8 +78,10 @@ def test_random_case(case):
         sfa, sfb = ea, eb
     want = np.einsum("bmk,bnk->bmn", A * sA, B * sB)
 
-    da, _ = _padded(r, torch.from_numpy(qa), [0, 0, 16, 48, 5], 0x7F)
+    da, _ = _padded(r, torch.from_numpy(qa), [0, 0, 16, 48] if shuffled else [0, 0, 16, 48, 5], 0x7F)
     db, _ = _padded(r, torch.from_numpy(qb), [0, 0, 16, 128, 3], 0x7F)
+    if shuffled:
+        db = torch.stack([g.preshuffle_b_device(db[i].contiguous()) for i in range(batch)])
     cdt = torch.bfloat16 if c_dtype == g.BF16 else torch.float32
     c_view, c_whole = _padded(r, torch.zeros((batch, m, n), dtype=cdt), [0, 0, 8, 24, 1], 7.0)
     dsa, dsb = torch.from_numpy(sfa).cuda(), torch.from_numpy(sfb).cuda()
@@ -82,12 +89,12 @@ def test_random_case(case):
         tiles = [g.mx_tile_scales_ab(dsa[i], dsb[i]) for i in range(batch)]
         dsa = torch.stack([t[0] for t in tiles])
         dsb = torch.stack([t[1] for t in tiles])
-    what = f"case {case}: mode {mode} {batch}x{m}x{n}x{k} c={c_dtype} lda={da.stride(-2)} ldb={db.stride(-2)} ldc={c_view.stride(-2)}"
+    what = f"case {case}{' (shuffled B)' if shuffled else ''}: mode {mode} {batch}x{m}x{n}x{k} c={c_dtype} lda={da.stride(-2)} ldb={db.stride(-2)} ldc={c_view.stride(-2)}"
     print(what, flush=True)
     if batch == 1:
-        g.gemm(da[0], db[0], dsa[0], dsb[0], mode, c=c_view[0])
+        g.gemm(da[0], db[0], dsa[0], dsb[0], mode, c=c_view[0], n=n if shuffled else None)
     else:
-        g.gemm(da, db, dsa, dsb, mode, c=c_view)
+        g.gemm(da, db, dsa, dsb, mode, c=c_view, n=n if shuffled else None)
     torch.cuda.synchronize()
     got = c_view.float().cpu().numpy()
     ref = torch.from_numpy(want.astype(np.float32)).to(cdt).float().numpy()
