@@ -183,9 +183,10 @@ def gemm(a, b, sfa, sfb, scale_mode, c=None, c_dtype=BF16, n=None):
     return c
 
 
-def gemm_a16w16(a, b, c=None, c_dtype=BF16):
-    """C = A @ B^T for bf16 a [.., M, K] and b [.., N, K] (torch.bfloat16 on the GPU) through a16w16_gemm."""
-    g, c = _args_from_tensors(a, b, a, b, TENSOR, c, c_dtype, 0)
+def gemm_a16w16(a, b, c=None, c_dtype=BF16, n=None):
+    """C = A @ B^T for bf16 a [.., M, K] and b [.., N, K] (torch.bfloat16 on the GPU) through a16w16_gemm; with `n`
+    given, b is the flat pre-shuffled weight of n rows (preshuffle_b_bf16_device)."""
+    g, c = _args_from_tensors(a, b, a, b, TENSOR, c, c_dtype, 0 if n is None else 1, n=n)
     _check(lib().a16w16_gemm(ctypes.byref(g), _stream()), "a16w16_gemm")
     return c
 
@@ -215,12 +216,17 @@ def quantize_mxfp4(x, tiled=False):
     return q, s
 
 
-def gemm_a4w4(a, b, sfa, sfb, scale_mode=MX_TILED, c=None, c_dtype=BF16):
-    """MXFP4 GEMM through a4w4_gemm: a [M, K/2], b [N, K/2] packed E2M1 (uint8 on the GPU)."""
-    m, n, k = a.shape[-2], b.shape[-2], a.shape[-1] * 2
+def gemm_a4w4(a, b, sfa, sfb, scale_mode=MX_TILED, c=None, c_dtype=BF16, n=None):
+    """MXFP4 GEMM through a4w4_gemm: a [M, K/2], b [N, K/2] packed E2M1 (uint8 on the GPU); with `n` given, b is the
+    flat pre-shuffled weight of n rows (preshuffle_b_device on the packed bytes)."""
+    m, k = a.shape[-2], a.shape[-1] * 2
+    shuffled = n is not None
+    if not shuffled:
+        n = b.shape[-2]
     c, c_dtype = _out(c, (m, n), c_dtype, a.device)
     g = raw_gemm_args(a.data_ptr(), b.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, scale_mode, c_dtype,
-                      stride_a=a.stride(-2) * 2, stride_b=b.stride(-2) * 2, stride_c=c.stride(-2))
+                      stride_a=a.stride(-2) * 2, stride_b=(k if shuffled else b.stride(-2) * 2), stride_c=c.stride(-2),
+                      b_preshuffled=int(shuffled))
     _check(lib().a4w4_gemm(ctypes.byref(g), _stream()), "a4w4_gemm")
     return c
 

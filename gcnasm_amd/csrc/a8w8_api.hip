@@ -416,21 +416,22 @@ int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
     if (!g->a || !g->b || !g->c) return A8W8_ERR_NULL_POINTER;
     if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0) return A8W8_ERR_BAD_SHAPE;
     if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
-    if (g->b_preshuffled) return A8W8_ERR_BAD_MODE;
-    if (g->stride_c < g->n || g->stride_a < g->k || g->stride_b < g->k) return A8W8_ERR_BAD_STRIDE;
+    if (g->stride_c < g->n || g->stride_a < g->k || (!g->b_preshuffled && g->stride_b < g->k)) return A8W8_ERR_BAD_STRIDE;
     if (g->batch > 1 && (g->stride_a_batch < 0 || g->stride_b_batch < 0 || g->stride_c_batch < 0)) return A8W8_ERR_BAD_STRIDE;
     const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) * 2;
-    const long long b_span = ((long long)(g->n - 1) * g->stride_b + g->k) * 2;
+    const long long b_span = (g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k) * 2;
     if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
     hipStream_t s = (hipStream_t)hip_stream;
     // the tiled kernel reads bf16 rows as byte rows of 2k columns
     a8w8_gemm_args bytes = *g;
     bytes.k = g->k * 2;
-    bytes.stride_a = g->stride_a * 2; bytes.stride_b = g->stride_b * 2;
+    bytes.stride_a = g->stride_a * 2; bytes.stride_b = g->b_preshuffled ? bytes.k : g->stride_b * 2;
     bytes.stride_a_batch = g->stride_a_batch * 2; bytes.stride_b_batch = g->stride_b_batch * 2;
     bytes.scale_mode = A8W8_SCALE_TENSOR;
     const bool fits = (long long)g->stride_a_batch * 2 < (1ll << 31) && (long long)g->stride_b_batch * 2 < (1ll << 31);
+    // weights shuffled as bytes (a16w16_flatmm's): MFMA kernels only
+    if (g->b_preshuffled && (validate_shuffled_b(&bytes) != A8W8_OK || !fits || !persist_ok(&bytes))) return A8W8_ERR_BAD_GROUP;
     if (fits && tiled_ok(&bytes) && persist_ok(&bytes)) {
         GemmParams p = make_params(&bytes);
         p.sfa = p.sfb = nullptr;
@@ -462,10 +463,9 @@ int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream)
     if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0) return A8W8_ERR_BAD_SHAPE;
     if (g->scale_mode != A8W8_SCALE_MX_E8M0_1x32 && g->scale_mode != A8W8_SCALE_MX_E8M0_TILED) return A8W8_ERR_BAD_MODE;
     if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
-    if (g->b_preshuffled) return A8W8_ERR_BAD_MODE;
     if (g->k % 32 != 0) return A8W8_ERR_BAD_GROUP;
-    if (g->stride_c < g->n || g->stride_a < g->k || g->stride_b < g->k) return A8W8_ERR_BAD_STRIDE;
-    if ((g->stride_a & 1) || (g->stride_b & 1)) return A8W8_ERR_MISALIGNED;      // rows start on a byte
+    if (g->stride_c < g->n || g->stride_a < g->k || (!g->b_preshuffled && g->stride_b < g->k)) return A8W8_ERR_BAD_STRIDE;
+    if ((g->stride_a & 1) || (!g->b_preshuffled && (g->stride_b & 1))) return A8W8_ERR_MISALIGNED;      // rows start on a byte
     const bool tiled = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;
     if (!tiled && (g->stride_sfa < g->k / 32 || g->stride_sfb < g->k / 32)) return A8W8_ERR_BAD_STRIDE;
     if (g->batch > 1 && ((g->stride_a_batch & 1) || (g->stride_b_batch & 1))) return A8W8_ERR_MISALIGNED;
@@ -473,16 +473,20 @@ int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream)
                          g->stride_sfa_batch < 0 || g->stride_sfb_batch < 0))
         return A8W8_ERR_BAD_STRIDE;
     const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) / 2;
-    const long long b_span = ((long long)(g->n - 1) * g->stride_b + g->k) / 2;
+    const long long b_span = (g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k) / 2;
     if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
     hipStream_t s = (hipStream_t)hip_stream;
     // the tiled kernel reads packed rows as byte rows of k/2 columns
     a8w8_gemm_args bytes = *g;
     bytes.k = g->k / 2;
-    bytes.stride_a = g->stride_a / 2; bytes.stride_b = g->stride_b / 2;
+    bytes.stride_a = g->stride_a / 2; bytes.stride_b = g->b_preshuffled ? bytes.k : g->stride_b / 2;
     bytes.stride_a_batch = g->stride_a_batch / 2; bytes.stride_b_batch = g->stride_b_batch / 2;
     bytes.scale_mode = A8W8_SCALE_MX_E8M0_TILED;
+    // weights shuffled as bytes (a4w4_flatmm's): MFMA kernels only
+    if (g->b_preshuffled && (!tiled || g->k % 256 != 0 || validate_shuffled_b(&bytes) != A8W8_OK ||
+                             (!small_ok(&bytes) && !persist_ok(&bytes))))
+        return A8W8_ERR_BAD_GROUP;
     if (tiled && g->k % 256 == 0 && tiled_ok(&bytes)) {
         const GemmParams p = make_params(&bytes);
         if (small_ok(&bytes))       // few tiles, or an odd number of 128-byte K steps

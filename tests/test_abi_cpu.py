@@ -168,7 +168,7 @@ def test_sibling_entry_points_reject_bad_arguments():
     # a16w16_gemm: strides in bf16 elements
     a = _ok_args(mode=g.TENSOR)
     for mutate, want in [(lambda x: setattr(x, "c", None), -1), (lambda x: setattr(x, "k", 0), -2),
-                         (lambda x: setattr(x, "c_dtype", 7), -6), (lambda x: setattr(x, "b_preshuffled", 1), -6),
+                         (lambda x: setattr(x, "c_dtype", 7), -6),
                          (lambda x: setattr(x, "stride_b", 100), -4)]:
         b = _ok_args(mode=g.TENSOR)
         mutate(b)

@@ -90,6 +90,8 @@ def test_bf16_gemm_and_flat(case):
     print(what, flush=True)
     if flat:
         g.flatmm_a16w16(da, g.preshuffle_b_bf16_device(b.cuda()), n, c=c_view)
+    elif n % 16 == 0 and k % 64 == 0 and k >= 128 and da.stride(0) % 8 == 0:
+        g.gemm_a16w16(da, g.preshuffle_b_bf16_device(b.cuda()), c=c_view, n=n)      # the dense kernels on shuffled weights
     else:
         db, _ = _view(r, b, [0, 8, 64, 1], 1.0)
         g.gemm_a16w16(da, db, c=c_view)
@@ -116,7 +118,10 @@ def test_mxfp4_gemm(case):
     c_view, c_whole = _c(r, m, n)
     what = f"mxfp4 case {case}: tiled={tiled} {m}x{n}x{k} lda={da.stride(0) * 2} ldb={db.stride(0) * 2} c={c_view.dtype} ldc={c_view.stride(0)}"
     print(what, flush=True)
-    if tiled:
+    if tiled and n % 16 == 0 and k % 256 == 0 and da.stride(0) % 16 == 0 and case % 4 == 0:
+        g.gemm_a4w4(da, g.preshuffle_b_device(torch.from_numpy(qb).cuda()), g.mx_tile_scales(dea), g.mx_tile_scales(deb), g.MX_TILED,
+                    c=c_view, n=n)                                                     # shuffled weights
+    elif tiled:
         g.gemm_a4w4(da, db, g.mx_tile_scales(dea), g.mx_tile_scales(deb), g.MX_TILED, c=c_view)
     else:
         g.gemm_a4w4(da, db, dea, deb, g.MX, c=c_view)
