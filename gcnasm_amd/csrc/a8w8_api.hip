@@ -388,6 +388,37 @@ int launch_flat_f4(const GemmParams& p, int batch, hipStream_t stream)
     return launch_flat_f4_nt<1, CDT>(p, batch, stream);
 }
 
+// On shuffled weights both the flat GEMM and the MFMA kernels can run a skinny problem.  The flat kernel streams
+// B once per group of 16 activation rows: faster up to two groups, or when the weights are small enough to stay in
+// cache between the passes (measured, 16384 x 7168: 20 / 37 / 54 / 70 us flat at M = 16 / 32 / 48 / 64 against
+// 37-40 us on the 128-tile kernel; 4096 x 4096: 9 us flat at every M <= 64 against 22 us).
+bool prefer_flat(int m, long long weight_bytes)
+{
+    return m <= 32 || weight_bytes <= (32ll << 20);
+}
+
+int launch_flat_fp8(const a8w8_gemm_args* g, hipStream_t s)
+{
+    const GemmParams p = make_params(g);
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED)
+        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_MXT>(p, g->batch, s) : launch_flat<C_FP32, MODE_MXT>(p, g->batch, s);
+    if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128)
+        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_BLOCK>(p, g->batch, s) : launch_flat<C_FP32, MODE_BLOCK>(p, g->batch, s);
+    const bool tensor = g->scale_mode == A8W8_SCALE_TENSOR;
+    if (g->c_dtype == A8W8_C_BF16)
+        return tensor ? launch_flat<C_BF16, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_BF16, MODE_ROWCOL>(p, g->batch, s);
+    return tensor ? launch_flat<C_FP32, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_FP32, MODE_ROWCOL>(p, g->batch, s);
+}
+
+int launch_dense_fp8(const a8w8_gemm_args* g, hipStream_t s)
+{
+    const GemmParams p = make_params(g);
+    if (!tiled_ok(g)) return dispatch_general(g, p, s);
+    if (small_ok(g)) return dispatch_small(g, p, s);
+    if (wide_ok(g)) return dispatch_wide(g, p, s);
+    return persist_ok(g) ? dispatch_persist(g, p, s) : dispatch_tiled(g, p, s);
+}
+
 }  // namespace
 
 extern "C" {
@@ -402,12 +433,10 @@ int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream)
     const int shuf = validate_shuffled_b(g);
     if (shuf != A8W8_OK) return shuf;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-    const GemmParams p = make_params(g);
     hipStream_t s = (hipStream_t)hip_stream;
-    if (!tiled_ok(g)) return dispatch_general(g, p, s);
-    if (small_ok(g)) return dispatch_small(g, p, s);
-    if (wide_ok(g)) return dispatch_wide(g, p, s);
-    return persist_ok(g) ? dispatch_persist(g, p, s) : dispatch_tiled(g, p, s);
+    // a skinny problem on shuffled weights: the flat kernel where it is the faster one
+    if (g->b_preshuffled && validate_flat(g) == A8W8_OK && prefer_flat(g->m, (long long)g->n * g->k)) return launch_flat_fp8(g, s);
+    return launch_dense_fp8(g, s);
 }
 
 int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
@@ -456,9 +485,15 @@ int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
     return launch_status();
 }
 
-int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream)
+static int a4w4_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_dense);
+
+static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_flat)
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
+    // a skinny problem on shuffled weights: the flat kernel where it is the faster one (and can run it)
+    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= 64 && prefer_flat(g->m, (long long)g->n * g->k / 2) &&
+        a4w4_flat_impl(g, hip_stream, false) == A8W8_OK)
+        return A8W8_OK;
     if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
     if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0) return A8W8_ERR_BAD_SHAPE;
     if (g->scale_mode != A8W8_SCALE_MX_E8M0_1x32 && g->scale_mode != A8W8_SCALE_MX_E8M0_TILED) return A8W8_ERR_BAD_MODE;
@@ -509,7 +544,9 @@ int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream)
     return launch_status();
 }
 
-int a4w4_flatmm(const a8w8_gemm_args* g, void* hip_stream)
+int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream) { return a4w4_gemm_impl(g, hip_stream, true); }
+
+static int a4w4_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_dense)
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
     if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
@@ -528,6 +565,9 @@ int a4w4_flatmm(const a8w8_gemm_args* g, void* hip_stream)
         return A8W8_ERR_MISALIGNED;
     if ((long long)g->n * g->k / 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    // more than two groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
+    if (allow_dense && !prefer_flat(g->m, (long long)g->n * g->k / 2) && a4w4_gemm_impl(g, hip_stream, false) == A8W8_OK)
+        return A8W8_OK;
     a8w8_gemm_args bytes = *g;      // packed rows as byte rows of k/2 columns
     bytes.k = g->k / 2;
     bytes.stride_a = g->stride_a / 2; bytes.stride_b = g->k / 2;
@@ -536,6 +576,8 @@ int a4w4_flatmm(const a8w8_gemm_args* g, void* hip_stream)
     hipStream_t s = (hipStream_t)hip_stream;
     return g->c_dtype == A8W8_C_BF16 ? launch_flat_f4<C_BF16>(p, g->batch, s) : launch_flat_f4<C_FP32>(p, g->batch, s);
 }
+
+int a4w4_flatmm(const a8w8_gemm_args* g, void* hip_stream) { return a4w4_flat_impl(g, hip_stream, true); }
 
 // the vectorised quantisers read 16 bytes per lane and write packed words
 static bool quant_vec_ok(const float* src, int rows, int k, int ld, const uint8_t* q, int q_align)
@@ -609,16 +651,14 @@ int a8w8_flatmm(const a8w8_gemm_args* g, void* hip_stream)
     const int st = validate_flat(g);
     if (st != A8W8_OK) return st;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-    const GemmParams p = make_params(g);
     hipStream_t s = (hipStream_t)hip_stream;
-    if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED)
-        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_MXT>(p, g->batch, s) : launch_flat<C_FP32, MODE_MXT>(p, g->batch, s);
-    if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128)
-        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_BLOCK>(p, g->batch, s) : launch_flat<C_FP32, MODE_BLOCK>(p, g->batch, s);
-    const bool tensor = g->scale_mode == A8W8_SCALE_TENSOR;
-    if (g->c_dtype == A8W8_C_BF16)
-        return tensor ? launch_flat<C_BF16, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_BF16, MODE_ROWCOL>(p, g->batch, s);
-    return tensor ? launch_flat<C_FP32, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_FP32, MODE_ROWCOL>(p, g->batch, s);
+    // more than two groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
+    if (!prefer_flat(g->m, (long long)g->n * g->k)) {
+        a8w8_gemm_args local = *g;
+        local.stride_b = local.k;
+        if (validate_shuffled_b(&local) == A8W8_OK) return launch_dense_fp8(&local, s);
+    }
+    return launch_flat_fp8(g, s);
 }
 
 static size_t shuffled_index(int j, int p, int k)
@@ -928,9 +968,13 @@ const char* a8w8_status_string(int status)
 const char* a8w8_kernel_name(const a8w8_gemm_args* g)
 {
     if (!g) return nullptr;
-    // pre-shuffled B: the flat GEMM when its preconditions hold (m <= 64, ...), else a8w8_gemm on shuffled weights
-    if (g->b_preshuffled && validate_flat(g) == A8W8_OK) return "flatmm_a8w8";
-    if (validate_common(g) != A8W8_OK || validate_shuffled_b(g) != A8W8_OK) return nullptr;
+    // shuffled weights: a8w8_gemm and a8w8_flatmm both pick the flat kernel for skinny problems it runs faster
+    a8w8_gemm_args local = *g;
+    if (local.b_preshuffled) local.stride_b = local.k;
+    g = &local;
+    const bool dense_ok = validate_common(g) == A8W8_OK && validate_shuffled_b(g) == A8W8_OK;
+    if (g->b_preshuffled && validate_flat(g) == A8W8_OK && (prefer_flat(g->m, (long long)g->n * g->k) || !dense_ok)) return "flatmm_a8w8";
+    if (!dense_ok) return nullptr;
     if (!tiled_ok(g)) return "gemm_a8w8_general";
     if (small_ok(g)) return "gemm_a8w8_tile128";
     if (wide_ok(g)) return "gemm_a8w8_wide";
