@@ -439,9 +439,15 @@ int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream)
     return launch_dense_fp8(g, s);
 }
 
-int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
+static int a16w16_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_dense);
+
+static int a16w16_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_flat)
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
+    // a skinny problem on shuffled weights: the flat kernel where it is the faster one (and can run it)
+    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= 64 && prefer_flat(g->m, (long long)g->n * g->k * 2) &&
+        a16w16_flat_impl(g, hip_stream, false) == A8W8_OK)
+        return A8W8_OK;
     if (!g->a || !g->b || !g->c) return A8W8_ERR_NULL_POINTER;
     if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0) return A8W8_ERR_BAD_SHAPE;
     if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
@@ -484,6 +490,8 @@ int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream)
                            (long long)g->stride_a_batch, (long long)g->stride_b_batch, (long long)g->stride_c_batch);
     return launch_status();
 }
+
+int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream) { return a16w16_gemm_impl(g, hip_stream, true); }
 
 static int a4w4_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_dense);
 
@@ -614,7 +622,7 @@ int a4w4_quantize_mx(const float* src, int rows, int k, int ld, uint8_t* q, uint
     return launch_status();
 }
 
-int a16w16_flatmm(const a8w8_gemm_args* g, void* hip_stream)
+static int a16w16_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_dense)
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
     if (!g->a || !g->b || !g->c) return A8W8_ERR_NULL_POINTER;
@@ -627,6 +635,9 @@ int a16w16_flatmm(const a8w8_gemm_args* g, void* hip_stream)
     if (g->batch > 1 && (g->stride_a_batch % 8 != 0 || g->stride_b_batch % 8 != 0)) return A8W8_ERR_MISALIGNED;
     if ((long long)g->n * g->k * 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    // more than two groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
+    if (allow_dense && !prefer_flat(g->m, (long long)g->n * g->k * 2) && a16w16_gemm_impl(g, hip_stream, false) == A8W8_OK)
+        return A8W8_OK;
     a8w8_gemm_args bytes = *g;      // bf16 rows as byte rows of 2k columns
     bytes.k = g->k * 2;
     bytes.stride_a = g->stride_a * 2; bytes.stride_b = g->k * 2;
@@ -637,6 +648,8 @@ int a16w16_flatmm(const a8w8_gemm_args* g, void* hip_stream)
     return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_BF16>(p, g->batch, s)
                                      : launch_flat<C_FP32, MODE_BF16>(p, g->batch, s);
 }
+
+int a16w16_flatmm(const a8w8_gemm_args* g, void* hip_stream) { return a16w16_flat_impl(g, hip_stream, true); }
 
 int a8w8_gemm_blockscale(const a8w8_gemm_args* g, void* hip_stream)
 {
