@@ -354,7 +354,7 @@ template <int NT, int CDT, int MODE>
 int launch_flat_nt(const GemmParams& p, int batch, hipStream_t stream)
 {
     const int n_tiles = p.n / 16;
-    dim3 grid((unsigned)((n_tiles + NT - 1) / NT), (unsigned)((p.m + 15) / 16), (unsigned)batch);
+    dim3 grid((unsigned)(((n_tiles + NT - 1) / NT) * ((p.m + 15) / 16)), 1, (unsigned)batch);
     hipLaunchKernelGGL((flatmm_a8w8<NT, CDT, MODE>), grid, dim3(FLAT_THREADS), 0, stream, p);
     return launch_status();
 }
@@ -373,7 +373,7 @@ template <int NT, int CDT>
 int launch_flat_f4_nt(const GemmParams& p, int batch, hipStream_t stream)
 {
     const int n_tiles = p.n / 16;
-    dim3 grid((unsigned)((n_tiles + NT - 1) / NT), (unsigned)((p.m + 15) / 16), (unsigned)batch);
+    dim3 grid((unsigned)(((n_tiles + NT - 1) / NT) * ((p.m + 15) / 16)), 1, (unsigned)batch);
     hipLaunchKernelGGL((flatmm_a4w4<NT, CDT>), grid, dim3(FLAT_THREADS), 0, stream, p);
     return launch_status();
 }
@@ -389,12 +389,13 @@ int launch_flat_f4(const GemmParams& p, int batch, hipStream_t stream)
 }
 
 // On shuffled weights both the flat GEMM and the MFMA kernels can run a skinny problem.  The flat kernel streams
-// B once per group of 16 activation rows: faster up to two groups, or when the weights are small enough to stay in
-// cache between the passes (measured, 16384 x 7168: 20 / 37 / 54 / 70 us flat at M = 16 / 32 / 48 / 64 against
-// 37-40 us on the 128-tile kernel; 4096 x 4096: 9 us flat at every M <= 64 against 22 us).
+// B once per group of 16 activation rows (the groups of one weight tile run side by side on one XCD, so only the
+// first pass comes from memory): faster up to three groups, or when the weights are small enough to stay in cache
+// anyway (measured, 16384 x 7168: 20 / 27 / 38 / 47 us flat at M = 16 / 32 / 48 / 64 against 37-40 us on the
+// 128-tile kernel; 4096 x 4096: 9 us flat at every M <= 64 against 22 us).
 bool prefer_flat(int m, long long weight_bytes)
 {
-    return m <= 32 || weight_bytes <= (32ll << 20);
+    return m <= 48 || weight_bytes <= (32ll << 20);
 }
 
 int launch_flat_fp8(const a8w8_gemm_args* g, hipStream_t s)
@@ -573,7 +574,7 @@ static int a4w4_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
         return A8W8_ERR_MISALIGNED;
     if ((long long)g->n * g->k / 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-    // more than two groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
+    // more than three groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
     if (allow_dense && !prefer_flat(g->m, (long long)g->n * g->k / 2) && a4w4_gemm_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     a8w8_gemm_args bytes = *g;      // packed rows as byte rows of k/2 columns
@@ -635,7 +636,7 @@ static int a16w16_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     if (g->batch > 1 && (g->stride_a_batch % 8 != 0 || g->stride_b_batch % 8 != 0)) return A8W8_ERR_MISALIGNED;
     if ((long long)g->n * g->k * 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-    // more than two groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
+    // more than three groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
     if (allow_dense && !prefer_flat(g->m, (long long)g->n * g->k * 2) && a16w16_gemm_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     a8w8_gemm_args bytes = *g;      // bf16 rows as byte rows of 2k columns
@@ -665,7 +666,7 @@ int a8w8_flatmm(const a8w8_gemm_args* g, void* hip_stream)
     if (st != A8W8_OK) return st;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
     hipStream_t s = (hipStream_t)hip_stream;
-    // more than two groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
+    // more than three groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
     if (!prefer_flat(g->m, (long long)g->n * g->k)) {
         a8w8_gemm_args local = *g;
         local.stride_b = local.k;

@@ -18,6 +18,21 @@ namespace a8w8 {
 constexpr int FLAT_WAVES = 8;
 constexpr int FLAT_THREADS = FLAT_WAVES * 64;
 
+// Workgroup id -> (group of NT weight tiles, group of 16 activation rows).  The workgroups that stream the same weight
+// tiles for different row groups get ids 8 apart and next to each other in that stride: the hardware deals consecutive
+// ids to the 8 XCDs in turn, so they run on one XCD at the same time and all but the first find the weights in its L2.
+A8W8_DEV void flat_work_of_block(int bid, int n_groups, int m_tiles, int& n_group, int& m_tile)
+{
+    if ((n_groups & 7) == 0) {
+        const int rest = bid >> 3;
+        m_tile = rest % m_tiles;
+        n_group = (rest / m_tiles) * 8 + (bid & 7);
+    } else {
+        m_tile = bid % m_tiles;
+        n_group = bid / m_tiles;
+    }
+}
+
 template <int NT, int CDT, int MODE>
 __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 {
@@ -31,8 +46,10 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 
     const int n_tiles = p.n >> 4;
     const int k_tiles = p.k >> 6;
-    const int nt0 = blockIdx.x * NT;
-    const int m0 = blockIdx.y * 16;
+    int n_group, m_tile_;
+    flat_work_of_block(blockIdx.x, (n_tiles + NT - 1) / NT, (p.m + 15) >> 4, n_group, m_tile_);
+    const int nt0 = n_group * NT;
+    const int m0 = m_tile_ * 16;
 
     // Wave t < NT writes tile t at the end: its lane holds C[m = r16][n = tile*16 + 4*kq .. +3].
     // Its scales are fetched now, so that the tail of the kernel is only reduce + store.
@@ -68,7 +85,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     int mx_nblk_a = 1, mx_nblk_b = 1;
     if constexpr (MODE == MODE_MXT) {
         auto lane_off = [&](int i) { return ((4 * ((2 * i + (r16 >> 3)) & 3) + (r16 & 3)) * 4 + kq) * 8 + (i >> 1) * 4 + ((r16 >> 2) & 1) * 2; };
-        const int m_tile = blockIdx.y;
+        const int m_tile = m_tile_;
         mx_nblk_a = (p.m + 63) >> 6;
         mx_nblk_b = (p.n + 63) >> 6;
         mx_a = (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch + (size_t)(m_tile >> 2) * 1024 + lane_off(m_tile & 3);
@@ -212,8 +229,9 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a4w4(GemmParams p)
 
     const int n_tiles = p.n >> 4;
     const int k_tiles = p.k >> 6;                  // blocks of 64 bytes = 128 elements = one MFMA
-    const int nt0 = blockIdx.x * NT;
-    const int m_tile = blockIdx.y;
+    int n_group, m_tile;
+    flat_work_of_block(blockIdx.x, (n_tiles + NT - 1) / NT, (p.m + 15) >> 4, n_group, m_tile);
+    const int nt0 = n_group * NT;
     const int m0 = m_tile * 16;
     const int cm = m0 + r16;
     const int cn = (nt0 + wave) * 16 + 4 * kq;
