@@ -326,7 +326,7 @@ def run_flat_variants(torch, g, steps, warmup, seed):
 
         ms, wall = time_best_of(torch, fn, steps, warmup)
         abytes = wbytes + sbytes + a.numel() + 2 * m * n
-        out.append({"workload": f"{name}_{m}x{n}x{k}", "m": m, "n": n, "k": k, "kernel": "flatmm_a4w4" if fp4 else "flatmm_a8w8",
+        out.append({"workload": f"{name}_{m}x{n}x{k}", "m": m, "n": n, "k": k, "kernel": "flatmm_a8w8 (FP4 mode)" if fp4 else "flatmm_a8w8",
                     "ms_per_launch": ms, "wall_ms_per_launch": wall, "algorithmic_bytes": abytes, "gbs": abytes / ms / 1e6,
                     "frac_hbm_peak": abytes / ms / 1e6 / PEAK_HBM_GBS,
                     "note": f"{len(copies)} rotating copies of the weights ({len(copies) * wbytes // 10**6} MB)"})

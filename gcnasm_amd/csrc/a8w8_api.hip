@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <string.h>
+#include <algorithm>
 
 #include "cvt.hpp"
 #include "flatmm.hpp"
@@ -348,54 +349,74 @@ int validate_flat(const a8w8_gemm_args* g)
 // Weight tiles (16 rows of B) per workgroup: the activation fragment of a K block is re-used by all of them, but
 // the grid shrinks by the same factor: the largest of 4, 2, 1 that still gives every compute unit a workgroup
 // (16 x 4096 x 4096: 8.6 us with 4 tiles per workgroup on 64 compute units, 5.4 us with 1 on 256).
-// Several groups of 16 activation rows per workgroup (one pass over B for m > 16) were measured slower: the
-// activation gather (16 cache lines per load instruction) then costs more than re-reading B from cache.
-template <int NT, int CDT, int MODE>
+template <int NT, int MT, int CDT, int MODE>
 int launch_flat_nt(const GemmParams& p, int batch, hipStream_t stream)
 {
     const int n_tiles = p.n / 16;
-    dim3 grid((unsigned)(((n_tiles + NT - 1) / NT) * ((p.m + 15) / 16)), 1, (unsigned)batch);
-    hipLaunchKernelGGL((flatmm_a8w8<NT, CDT, MODE>), grid, dim3(FLAT_THREADS), 0, stream, p);
+    dim3 grid((unsigned)(((n_tiles + NT - 1) / NT) * ((p.m + 16 * MT - 1) / (16 * MT))), 1, (unsigned)batch);
+    hipLaunchKernelGGL((flatmm_a8w8<NT, MT, CDT, MODE>), grid, dim3(FLAT_THREADS), 0, stream, p);
     return launch_status();
 }
 
+// Up to four groups of 16 activation rows share one pass over the weights; as many weight tiles per workgroup as
+// still leave every compute unit a workgroup (every workgroup reads all rows of A once, so more weight tiles per
+// workgroup also means fewer reads of A: 16384 x 7168 at M = 48, 30 us with two tiles, 24 us with four).
 template <int CDT, int MODE>
 int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 {
-    const long long tiles = (long long)(p.n / 16) * ((p.m + 15) / 16) * batch;
+    const long long tiles = (long long)(p.n / 16) * batch;
     const int cus = num_cus();
-    if (tiles >= 4ll * cus) return launch_flat_nt<4, CDT, MODE>(p, batch, stream);
-    if (tiles >= 2ll * cus) return launch_flat_nt<2, CDT, MODE>(p, batch, stream);
-    return launch_flat_nt<1, CDT, MODE>(p, batch, stream);
+    if (p.m > 48) {
+        // four weight tiles x four row groups fill the register file; MX or block scales on top would spill
+        if constexpr (MODE != MODE_BLOCK && MODE != MODE_MXT && MODE != MODE_F4T) {
+            if (tiles >= 4ll * cus) return launch_flat_nt<4, 4, CDT, MODE>(p, batch, stream);
+        }
+        return launch_flat_nt<2, 4, CDT, MODE>(p, batch, stream);
+    }
+    if (p.m > 32) {
+        if (tiles >= 4ll * cus) return launch_flat_nt<4, 3, CDT, MODE>(p, batch, stream);
+        return launch_flat_nt<2, 3, CDT, MODE>(p, batch, stream);
+    }
+    if (p.m > 16) {
+        if (tiles >= 4ll * cus) return launch_flat_nt<4, 2, CDT, MODE>(p, batch, stream);
+        return launch_flat_nt<2, 2, CDT, MODE>(p, batch, stream);
+    }
+    if (tiles >= 4ll * cus) return launch_flat_nt<4, 1, CDT, MODE>(p, batch, stream);
+    if (tiles >= 2ll * cus) return launch_flat_nt<2, 1, CDT, MODE>(p, batch, stream);
+    return launch_flat_nt<1, 1, CDT, MODE>(p, batch, stream);
 }
 
-template <int NT, int CDT>
-int launch_flat_f4_nt(const GemmParams& p, int batch, hipStream_t stream)
+// On shuffled weights both the flat GEMM and the MFMA kernels can run a skinny problem; the entry points take the
+// one a small cost model calls faster.  Times in microseconds, W = weight bytes, row_bytes = bytes of one weight row:
+//   flat:  one pass over the weights at ~6.3 TB/s; every further group of 16 activation rows adds ~2 us of
+//          activation traffic and MFMA work.  With MX or block scales, four groups only fit the registers with two
+//          weight tiles per workgroup, which costs another ~30%.
+//   dense: the 128-tile kernel has only n/128 workgroups to pull the weights with, ~28 GB/s each (128 rows a
+//          workgroup), and ~5 TB/s at best over the chip.
+// Weights of at most 32 MiB always go flat.  Measured on MI355X, M = 16 / 32 / 48 / 64, flat against dense:
+//   16384 x 7168   FP8 21 / 21 / 23 / 24 against 37-40, MXFP8 20 / 22 / 24 / 35 against 38-41,
+//                  MXFP4 12 / 13 / 14 / 20 against 21-22, bf16 37 / 38 / 41 / 45 against 66-72
+//   8192 x 8192    FP8 13 / 14 / 16 / 18 against 40-41 (64 workgroups on the dense side)
+//   28672 x 4096   FP8 21 / 23 / 26 / 28 against 26-27, MXFP8 22 / 25 / 28 / 40 against 26-28,
+//                  MXFP4 13 / 16 / 17 / 25 against 15-16, bf16 43 / 43 / 48 / 52 against 47-48
+// The model takes the faster side in these except where the two are within ~8% of each other.
+bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop)
 {
-    const int n_tiles = p.n / 16;
-    dim3 grid((unsigned)(((n_tiles + NT - 1) / NT) * ((p.m + 15) / 16)), 1, (unsigned)batch);
-    hipLaunchKernelGGL((flatmm_a4w4<NT, CDT>), grid, dim3(FLAT_THREADS), 0, stream, p);
-    return launch_status();
-}
-
-template <int CDT>
-int launch_flat_f4(const GemmParams& p, int batch, hipStream_t stream)
-{
-    const long long tiles = (long long)(p.n / 16) * ((p.m + 15) / 16) * batch;
+    const double w = (double)n * (double)row_bytes;
+    if (w <= (double)(32ll << 20)) return true;
+    const int groups = (m + 15) / 16;
     const int cus = num_cus();
-    if (tiles >= 4ll * cus) return launch_flat_f4_nt<4, CDT>(p, batch, stream);
-    if (tiles >= 2ll * cus) return launch_flat_f4_nt<2, CDT>(p, batch, stream);
-    return launch_flat_f4_nt<1, CDT>(p, batch, stream);
+    const int rounds = ((n + 127) / 128 + cus - 1) / cus;
+    double flat = 3.5 + w / 6.3e6 + 2.0 * (groups - 1);
+    if (groups == 4 && scaled_in_loop) flat *= 1.3;
+    const double dense = 4.0 + std::max(rounds * 128.0 * (double)row_bytes / 28.0e3, w / 5.0e6);
+    return flat <= dense;
 }
 
-// On shuffled weights both the flat GEMM and the MFMA kernels can run a skinny problem.  The flat kernel streams
-// B once per group of 16 activation rows (the groups of one weight tile run side by side on one XCD, so only the
-// first pass comes from memory): faster up to three groups, or when the weights are small enough to stay in cache
-// anyway (measured, 16384 x 7168: 20 / 27 / 38 / 47 us flat at M = 16 / 32 / 48 / 64 against 37-40 us on the
-// 128-tile kernel; 4096 x 4096: 9 us flat at every M <= 64 against 22 us).
-bool prefer_flat(int m, long long weight_bytes)
+bool prefer_flat_fp8(const a8w8_gemm_args* g)
 {
-    return m <= 48 || weight_bytes <= (32ll << 20);
+    const bool scaled_in_loop = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED || g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128;
+    return prefer_flat(g->m, g->n, g->k, scaled_in_loop);
 }
 
 int launch_flat_fp8(const a8w8_gemm_args* g, hipStream_t s)
@@ -436,7 +457,7 @@ int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream)
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
     hipStream_t s = (hipStream_t)hip_stream;
     // a skinny problem on shuffled weights: the flat kernel where it is the faster one
-    if (g->b_preshuffled && validate_flat(g) == A8W8_OK && prefer_flat(g->m, (long long)g->n * g->k)) return launch_flat_fp8(g, s);
+    if (g->b_preshuffled && validate_flat(g) == A8W8_OK && prefer_flat_fp8(g)) return launch_flat_fp8(g, s);
     return launch_dense_fp8(g, s);
 }
 
@@ -446,7 +467,7 @@ static int a16w16_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
     // a skinny problem on shuffled weights: the flat kernel where it is the faster one (and can run it)
-    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= 64 && prefer_flat(g->m, (long long)g->n * g->k * 2) &&
+    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= 64 && prefer_flat(g->m, g->n, 2ll * g->k, false) &&
         a16w16_flat_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     if (!g->a || !g->b || !g->c) return A8W8_ERR_NULL_POINTER;
@@ -500,7 +521,7 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
     // a skinny problem on shuffled weights: the flat kernel where it is the faster one (and can run it)
-    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= 64 && prefer_flat(g->m, (long long)g->n * g->k / 2) &&
+    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= 64 && prefer_flat(g->m, g->n, g->k / 2, true) &&
         a4w4_flat_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
@@ -574,8 +595,8 @@ static int a4w4_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
         return A8W8_ERR_MISALIGNED;
     if ((long long)g->n * g->k / 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-    // more than three groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
-    if (allow_dense && !prefer_flat(g->m, (long long)g->n * g->k / 2) && a4w4_gemm_impl(g, hip_stream, false) == A8W8_OK)
+    // several groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
+    if (allow_dense && !prefer_flat(g->m, g->n, g->k / 2, true) && a4w4_gemm_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     a8w8_gemm_args bytes = *g;      // packed rows as byte rows of k/2 columns
     bytes.k = g->k / 2;
@@ -583,7 +604,7 @@ static int a4w4_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
     bytes.stride_a_batch = g->stride_a_batch / 2; bytes.stride_b_batch = g->stride_b_batch / 2;
     const GemmParams p = make_params(&bytes);
     hipStream_t s = (hipStream_t)hip_stream;
-    return g->c_dtype == A8W8_C_BF16 ? launch_flat_f4<C_BF16>(p, g->batch, s) : launch_flat_f4<C_FP32>(p, g->batch, s);
+    return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_F4T>(p, g->batch, s) : launch_flat<C_FP32, MODE_F4T>(p, g->batch, s);
 }
 
 int a4w4_flatmm(const a8w8_gemm_args* g, void* hip_stream) { return a4w4_flat_impl(g, hip_stream, true); }
@@ -636,8 +657,8 @@ static int a16w16_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     if (g->batch > 1 && (g->stride_a_batch % 8 != 0 || g->stride_b_batch % 8 != 0)) return A8W8_ERR_MISALIGNED;
     if ((long long)g->n * g->k * 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-    // more than three groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
-    if (allow_dense && !prefer_flat(g->m, (long long)g->n * g->k * 2) && a16w16_gemm_impl(g, hip_stream, false) == A8W8_OK)
+    // several groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
+    if (allow_dense && !prefer_flat(g->m, g->n, 2ll * g->k, false) && a16w16_gemm_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     a8w8_gemm_args bytes = *g;      // bf16 rows as byte rows of 2k columns
     bytes.k = g->k * 2;
@@ -666,8 +687,8 @@ int a8w8_flatmm(const a8w8_gemm_args* g, void* hip_stream)
     if (st != A8W8_OK) return st;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
     hipStream_t s = (hipStream_t)hip_stream;
-    // more than three groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
-    if (!prefer_flat(g->m, (long long)g->n * g->k)) {
+    // several groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
+    if (!prefer_flat_fp8(g)) {
         a8w8_gemm_args local = *g;
         local.stride_b = local.k;
         if (validate_shuffled_b(&local) == A8W8_OK) return launch_dense_fp8(&local, s);
@@ -987,7 +1008,7 @@ const char* a8w8_kernel_name(const a8w8_gemm_args* g)
     if (local.b_preshuffled) local.stride_b = local.k;
     g = &local;
     const bool dense_ok = validate_common(g) == A8W8_OK && validate_shuffled_b(g) == A8W8_OK;
-    if (g->b_preshuffled && validate_flat(g) == A8W8_OK && (prefer_flat(g->m, (long long)g->n * g->k) || !dense_ok)) return "flatmm_a8w8";
+    if (g->b_preshuffled && validate_flat(g) == A8W8_OK && (prefer_flat_fp8(g) || !dense_ok)) return "flatmm_a8w8";
     if (!dense_ok) return nullptr;
     if (!tiled_ok(g)) return "gemm_a8w8_general";
     if (small_ok(g)) return "gemm_a8w8_tile128";

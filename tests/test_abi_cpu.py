@@ -80,10 +80,15 @@ def test_gemm_on_shuffled_weights_preconditions():
     assert g.kernel_name(ok) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(mode=g.BLOCK, m=300, n=512, k=512, b_preshuffled=1)) == "gemm_a8w8_tile128"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, m=16, n=256, k=256, b_preshuffled=1)) == "flatmm_a8w8"     # flat when it can
-    # skinny problems: flat up to three groups of 16 rows, or on weights small enough to stay in cache
-    big = dict(mode=g.ROWCOL, n=16384, k=7168, b_preshuffled=1)
-    assert g.kernel_name(_ok_args(m=48, **big)) == "flatmm_a8w8"
-    assert g.kernel_name(_ok_args(m=49, **big)) == "gemm_a8w8_tile128"
+    # skinny problems: the side a cost model of the two kernels calls faster (the measured winners)
+    big = dict(n=16384, k=7168, b_preshuffled=1)
+    assert g.kernel_name(_ok_args(m=64, mode=g.ROWCOL, **big)) == "flatmm_a8w8"
+    assert g.kernel_name(_ok_args(m=64, mode=g.MX_TILED, **big)) == "flatmm_a8w8"
+    wide = dict(n=28672, k=4096, b_preshuffled=1)                # 224 workgroups on the 128-tile kernel, short rows
+    assert g.kernel_name(_ok_args(m=48, mode=g.ROWCOL, **wide)) == "flatmm_a8w8"
+    assert g.kernel_name(_ok_args(m=64, mode=g.ROWCOL, **wide)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(m=48, mode=g.MX_TILED, **wide)) == "flatmm_a8w8"
+    assert g.kernel_name(_ok_args(m=64, mode=g.MX_TILED, **wide)) == "gemm_a8w8_tile128"
     assert g.kernel_name(_ok_args(m=64, n=4096, k=4096, mode=g.ROWCOL, b_preshuffled=1)) == "flatmm_a8w8"
     assert g.kernel_name(_ok_args(m=64, n=16384, k=7104, mode=g.ROWCOL, b_preshuffled=1)) == "flatmm_a8w8"   # K % 128 != 0: flat only
     for mutate, want in [(lambda x: setattr(x, "n", 4088), -3), (lambda x: setattr(x, "k", 448), -3),

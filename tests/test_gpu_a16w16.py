@@ -98,3 +98,16 @@ def test_flat_gemm_exact_integers_and_decode_shape(orc):
     b = torch.randint(-4, 5, (n, k), generator=gen, device="cuda").to(torch.bfloat16)
     want = a.float() @ b.float().T
     assert torch.equal(g.flatmm_a16w16(a, g.preshuffle_b_bf16_device(b), n, c_dtype=g.FP32), want)
+
+
+@pytest.mark.parametrize("m", [17, 33, 48, 49, 64])
+@pytest.mark.parametrize("n,batch", [(144, 2), (288, 57)])      # two / four weight tiles per workgroup
+def test_flat_gemm_row_groups_exact(m, n, batch):
+    """M > 16: up to four groups of 16 rows share one pass over the weights (rows staged through LDS)."""
+    k = 160                                                      # 320 bytes a row: an odd number of 64-byte K blocks
+    gen = torch.Generator(device="cuda"); gen.manual_seed(900 + m + n)
+    a = torch.randint(-4, 5, (batch, m, k), generator=gen, device="cuda").to(torch.bfloat16)
+    b = torch.randint(-4, 5, (batch, n, k), generator=gen, device="cuda").to(torch.bfloat16)
+    bs = torch.stack([g.preshuffle_b_bf16_device(b[i]) for i in range(batch)])
+    got = g.flatmm_a16w16(a, bs, n, c_dtype=g.FP32)
+    assert torch.equal(got, torch.einsum("bmk,bnk->bmn", a.float(), b.float()))

@@ -146,6 +146,22 @@ def test_flat_scale_bytes_reach_the_right_lane_and_block(orc, case):
     assert (_flat(qa, qb, ea, eb, g.BF16) == torch.from_numpy(exact.astype(np.float32)).to(torch.bfloat16).float().numpy()).all()
 
 
+@pytest.mark.parametrize("m", [17, 32, 33, 48, 49, 64])
+def test_flat_row_groups_four_weight_tiles(orc, m):
+    """Enough weight tiles for four per workgroup (two past 48 rows), 1025 of them so that the last workgroup holds
+    one; 2 / 3 / 4 groups of 16 rows share the pass over the weights."""
+    r = np.random.default_rng(8700 + m)
+    n, k = 16400, 384
+    qa = r.integers(0, 256, (m, k // 2)).astype(np.uint8)
+    qb = r.integers(0, 256, (n, k // 2)).astype(np.uint8)
+    ea = r.integers(126, 129, (m, k // 32)).astype(np.uint8)
+    eb = r.integers(126, 129, (n, k // 32)).astype(np.uint8)
+    exact, _ = _exact(orc, qa, qb, ea, eb)
+    got = _flat(qa, qb, ea, eb)
+    bad = np.argwhere(got != exact.astype(np.float32))
+    assert bad.size == 0, f"{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
+
+
 def test_flat_rejects_what_it_cannot_run():
     qa = torch.zeros((16, 64), dtype=torch.uint8, device="cuda")
     bs = torch.zeros(16 * 64, dtype=torch.uint8, device="cuda")

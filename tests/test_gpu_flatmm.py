@@ -1,4 +1,6 @@
 """GPU parity of the skinny-M flatmm over pre-shuffled weights."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -112,3 +114,69 @@ def test_flatmm_block_scales_exact(orc, case):
     torch.cuda.synchronize()
     bad = np.argwhere(c.cpu().numpy() != (A @ B.T).astype(np.float32))
     assert bad.size == 0, f"{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
+
+
+# ---------------------------------------------------------------- several row groups per workgroup (M > 16)
+
+def _row_group_case(orc, mode, m, n, k, batch, seed):
+    """Exact small-integer problem, batched so that the launch picks the variant wanted; power-of-two scales
+    distinct per row / group, so that a row group, weight tile, K block or scale taken from the wrong place
+    changes the result."""
+    import torch
+    from gpu_util import dev
+    r = np.random.default_rng(seed)
+    a = np.stack([datagen.small_ints(m, n, k, seed=seed + 7 * i)[0] for i in range(batch)])
+    b = np.stack([datagen.small_ints(m, n, k, seed=seed + 7 * i)[1] for i in range(batch)])
+    A = orc.decode(a).astype(np.float64)
+    B = orc.decode(b).astype(np.float64)
+    if mode == g.ROWCOL:
+        sfa = np.exp2(r.integers(-3, 4, (batch, m))).astype(np.float32)
+        sfb = np.exp2(r.integers(-3, 4, (batch, n))).astype(np.float32)
+        A, B = A * sfa[:, :, None], B * sfb[:, :, None]
+        da, db = dev(sfa), dev(sfb)
+    elif mode == g.TENSOR:
+        sfa = np.exp2(r.integers(-3, 4, batch)).astype(np.float32)
+        sfb = np.exp2(r.integers(-3, 4, batch)).astype(np.float32)
+        A = A * (sfa * sfb).astype(np.float64)[:, None, None]
+        da, db = dev(sfa), dev(sfb)
+    elif mode == g.BLOCK:
+        sfa = np.exp2(r.integers(-2, 3, (batch, k // 128, m))).astype(np.float32)
+        sfb = np.exp2(r.integers(-2, 3, (batch, n // 128, k // 128))).astype(np.float32)
+        A = A * np.repeat(np.swapaxes(sfa, 1, 2).astype(np.float64), 128, axis=2)
+        B = B * np.repeat(np.repeat(sfb.astype(np.float64), 128, axis=1), 128, axis=2)
+        da, db = dev(sfa), dev(sfb)
+    else:
+        ea = r.integers(125, 130, (batch, m, k // 32)).astype(np.uint8)
+        eb = r.integers(125, 130, (batch, n, k // 32)).astype(np.uint8)
+        A = A * np.repeat(np.exp2(ea.astype(np.float64) - 127), 32, axis=2)
+        B = B * np.repeat(np.exp2(eb.astype(np.float64) - 127), 32, axis=2)
+        da = torch.stack([g.mx_tile_scales(dev(ea[i])) for i in range(batch)])
+        db = torch.stack([g.mx_tile_scales(dev(eb[i])) for i in range(batch)])
+    bs = torch.stack([g.preshuffle_b_device(dev(b[i])) for i in range(batch)])
+    args, c = g.api._args_from_tensors(dev(a), bs, da, db, mode, None, g.FP32, 1, n=n)
+    assert (args.stride_sfa_batch, args.stride_sfb_batch) == (da[0].numel(), db[0].numel())      # scales of their own per entry
+    assert g.kernel_name(args) == "flatmm_a8w8"
+    assert g.lib().a8w8_flatmm(ctypes.byref(args), g.api._stream()) == 0
+    torch.cuda.synchronize()
+    want = np.einsum("bmk,bnk->bmn", A, B).astype(np.float32)
+    bad = np.argwhere(c.cpu().numpy() != want)
+    assert bad.size == 0, f"mode {mode} {batch}x{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
+
+
+@pytest.mark.parametrize("m", [17, 32, 33, 47, 48, 49, 63, 64])
+@pytest.mark.parametrize("mode", [g.ROWCOL, g.TENSOR, g.MX_TILED, g.BLOCK])
+def test_row_groups_two_weight_tiles(orc, mode, m):
+    """Few weight tiles: two per workgroup, 2 / 3 / 4 row groups; 9 tiles leave the last workgroup half empty."""
+    n, k = (144, 320) if mode in (g.ROWCOL, g.TENSOR) else (256, 384)      # 320 = an odd number of 64-wide K blocks
+    _row_group_case(orc, mode, m, n, k, 2, 8500 + m)
+
+
+@pytest.mark.parametrize("m", [17, 32, 33, 48, 49, 64])
+@pytest.mark.parametrize("mode", [g.ROWCOL, g.TENSOR, g.MX_TILED, g.BLOCK])
+def test_row_groups_four_weight_tiles(orc, mode, m):
+    """At least four weight tiles per compute unit over all batch entries: four per workgroup (two for MX and block
+    scales past 48 rows); 18 or 24 tiles per entry are not a multiple of four or leave the id remap without its
+    multiple of eight."""
+    n, k = (288, 192) if mode in (g.ROWCOL, g.TENSOR) else (384, 256)
+    batch = (1024 * 16 + n - 1) // n
+    _row_group_case(orc, mode, m, n, k, batch, 8600 + m)
