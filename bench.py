@@ -291,20 +291,26 @@ def run_reference_program_sizes(torch, g, steps, warmup, seed):
 
 
 def run_flat_variants(torch, g, steps, warmup, seed):
-    """The decode shape of the flat workload (16 x 16384 x 7168) in the other scale modes and in MXFP4, each with
-    rotating copies of the pre-shuffled weights (larger than the Infinity Cache together), priced against HBM."""
+    """The decode shape of the flat workload (16 x 16384 x 7168) in the other scale modes and in MXFP4, and with 32
+    and 64 activation rows (one pass over the weights for all of them), each with rotating copies of the pre-shuffled
+    weights (larger than the Infinity Cache together), priced against HBM."""
     import ctypes
-    m, n, k = 16, 16384, 7168
+    n, k = 16384, 7168
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
-    xa = torch.randn((m, k), generator=gen, device="cuda")
+    xa64 = torch.randn((64, k), generator=gen, device="cuda")
     xb = torch.randn((n, k), generator=gen, device="cuda")
     L = g.lib()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     out = []
-    for name, fp4 in (("flatmm_mx_tiled", False), ("flatmm_block", False), ("flatmm_mxfp4", True)):
-        if fp4:
+    for name, fp4, m in (("flatmm_mx_tiled", False, 16), ("flatmm_block", False, 16), ("flatmm_mxfp4", True, 16),
+                         ("flatmm_rowcol", False, 32), ("flatmm_rowcol", False, 64), ("flatmm_mx_tiled", False, 64)):
+        xa = xa64[:m].contiguous()
+        c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+        if name == "flatmm_rowcol":
+            (a, sfa), (b, sfb) = g.quantize(xa, g.ROWCOL), g.quantize(xb, g.ROWCOL)
+            mode, entry, wbytes, sbytes = g.ROWCOL, L.a8w8_flatmm, n * k, 4 * (n + m)
+        elif fp4:
             (a, sfa), (b, sfb) = g.quantize_mxfp4(xa, tiled=True), g.quantize_mxfp4(xb, tiled=True)
             mode, entry, wbytes, sbytes = g.MX_TILED, L.a4w4_flatmm, n * k // 2, n * k // 32 + m * k // 32
         elif name == "flatmm_mx_tiled":

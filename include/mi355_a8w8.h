@@ -138,9 +138,10 @@ A8W8_API int a8w8_gemm_blockscale(const a8w8_gemm_args* args, void* hip_stream);
  * scale_mode ROWCOL, TENSOR, BLOCK_1x128_128x128 (scale arrays as for a8w8_gemm_blockscale; n, k % 128 == 0) or
  * MX_E8M0_TILED (MXFP8: both scale arrays in the tiled layout, 16-byte aligned),
  * m <= 64, n % 16 == 0, k % 64 == 0, a, b and the rows of A 16-byte aligned (A8W8_ERR_MISALIGNED otherwise).
- * B is streamed once per 16 rows of A with 16-byte non-temporal loads; for more than 48 rows over weights larger
- * than 32 MiB the call runs a8w8_gemm's kernels on the same shuffled weights (k % 128 == 0 permitting), and
- * a8w8_gemm with b_preshuffled takes this kernel for the skinny problems it runs faster. */
+ * B is streamed once, with 16-byte non-temporal loads, for all rows of A.  Where a8w8_gemm's kernels are the
+ * faster ones on the same shuffled weights (several groups of 16 rows over many short weight rows; k % 128 == 0
+ * permitting) the call runs those, and a8w8_gemm with b_preshuffled takes this kernel for the skinny problems it
+ * runs faster: either entry point gives the same kernel for the same problem. */
 A8W8_API int a8w8_flatmm(const a8w8_gemm_args* args, void* hip_stream);
 
 /* Host-side weight pre-shuffle, row-major b[n][k] -> Bshuf[n/16][k/64][4][16][16 bytes]:
