@@ -42,6 +42,17 @@ A8W8_DEV void flat_work_of_block(int bid, int n_groups, int m_tiles, int& n_grou
     }
 }
 
+// 16 bytes per lane through a buffer descriptor: lane offset in a register, the rest of the address scalar.
+A8W8_DEV v4i ld16(__amdgpu_buffer_rsrc_t rs, uint32_t voffset, int soffset)
+{
+    return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rs, voffset, soffset, 0));
+}
+// The same marked non-temporal (streamed once: no reason to keep it in cache).
+A8W8_DEV v4i ld16_nt(__amdgpu_buffer_rsrc_t rs, uint32_t voffset, int soffset)
+{
+    return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rs, voffset, soffset, 2));
+}
+
 // Activation rows of one pair of K blocks, staged per wave for MT > 1: 8 pieces of 16 bytes per row (piece c of
 // a 128-byte line), piece-major with a stride of 18 slots so that both the row-wise writes and the piece-wise reads
 // touch every LDS bank once.
@@ -110,7 +121,8 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     const int ld_c = lane & 3;
     // addresses are a wave-uniform base plus a 32-bit lane offset (operand extents are below 2 GiB): one register
     // per row group and weight tile instead of a 64-bit pointer each
-    const uint8_t* a_base = p.a + (long long)batch * p.a_batch;
+    // (buffer loads: descriptor + 32-bit lane offset + scalar offset, so no load needs a 64-bit address in registers)
+    const auto rs_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * (uint32_t)p.lda + (uint32_t)p.k);
     uint32_t a_off[MT];
 #pragma unroll
     for (int g = 0; g < MT; ++g)
@@ -119,7 +131,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     const int st_write = (2 * ld_c) * 18 + ld_row;      // piece 2c, the next piece is 18 slots on
     const int st_read = kq * 18 + r16;                   // piece kq, the second K block's is 4 * 18 slots on
 
-    const uint8_t* b_base = p.b + (long long)batch * p.b_batch;
+    const auto rs_b = make_rsrc(p.b + (long long)batch * p.b_batch, (uint32_t)p.n * (uint32_t)p.k);
     const uint32_t lane16 = lane * 16;
     uint32_t b_off[NT];                                 // wave-uniform
 #pragma unroll
@@ -128,8 +140,9 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     // step ks; lane (r16, kq) scales 32-block kq of its row, whose byte for step ks sits at
     // ((ks / 4 * nblk + blk) * 2 + (ks / 2) % 2) * 512 + ((4x + y) * 4 + kq) * 8 + jp * 4 + par * 2 + ks % 2
     // with, for row 16 i + r16 of a 64-row block, x = (2 i + r16 / 8) % 4, y = r16 % 4, jp = i / 2, par = (r16 / 4) % 2
-    const uint8_t* mx_a[MT];
-    const uint8_t* mx_b[NT];
+    const auto rs_sa = make_rsrc((const uint8_t*)p.sfa + (long long)batch * p.sfa_batch, 0x7fffffffu);
+    const auto rs_sb = make_rsrc((const uint8_t*)p.sfb + (long long)batch * p.sfb_batch, 0x7fffffffu);
+    uint32_t mx_a[MT], mx_b[NT];
     int mx_nblk_a = 1, mx_nblk_b = 1;
     if constexpr (MODE == MODE_MXT || MODE == MODE_F4T) {
         auto lane_off = [&](int i) { return ((4 * ((2 * i + (r16 >> 3)) & 3) + (r16 & 3)) * 4 + kq) * 8 + (i >> 1) * 4 + ((r16 >> 2) & 1) * 2; };
@@ -138,12 +151,12 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 #pragma unroll
         for (int g = 0; g < MT; ++g) {
             const int mt = min(m_tile_ * MT + g, ((p.m + 15) >> 4) - 1);
-            mx_a[g] = (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch + (size_t)(mt >> 2) * 1024 + lane_off(mt & 3);
+            mx_a[g] = (uint32_t)(mt >> 2) * 1024u + lane_off(mt & 3);
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const int nt = min(nt0 + t, n_tiles - 1);
-            mx_b[t] = (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch + (size_t)(nt >> 2) * 1024 + lane_off(nt & 3);
+            mx_b[t] = (uint32_t)(nt >> 2) * 1024u + lane_off(nt & 3);
         }
     }
 
@@ -185,8 +198,8 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         const bool there = 2 * pp + 1 < k_tiles || ld_c < 2;
 #pragma unroll
         for (int g = 0; g < MT; ++g) {
-            raw[g][0] = there ? *(const v4i*)(a_base + (size_t)pp * 128 + a_off[g]) : v4i{0, 0, 0, 0};
-            raw[g][1] = there ? *(const v4i*)(a_base + (size_t)pp * 128 + 16 + a_off[g]) : v4i{0, 0, 0, 0};
+            raw[g][0] = there ? ld16(rs_a, a_off[g], pp * 128) : v4i{0, 0, 0, 0};
+            raw[g][1] = there ? ld16(rs_a, a_off[g], pp * 128 + 16) : v4i{0, 0, 0, 0};
         }
     };
     // rows -> this wave's own LDS.  A wave's LDS operations complete in order, so the fragment reads that follow
@@ -207,22 +220,22 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         const int kt0 = 2 * pp, kt1 = 2 * pp + 1;
         const bool has1 = kt1 < k_tiles;
         if constexpr (MT == 1) {
-            f.a[0] = *(const v4i*)(a_base + (size_t)kt0 * 64 + a_off[0]);
-            f.a[1] = has1 ? *(const v4i*)(a_base + (size_t)kt1 * 64 + a_off[0]) : v4i{0, 0, 0, 0};
+            f.a[0] = ld16(rs_a, a_off[0], kt0 * 64);
+            f.a[1] = has1 ? ld16(rs_a, a_off[0], kt1 * 64) : v4i{0, 0, 0, 0};
         }
-        size_t unit_a = 0, unit_b = 0;
+        int unit_a = 0, unit_b = 0;
         if constexpr (MODE == MODE_MXT) {
-            unit_a = ((size_t)(pp >> 2) * mx_nblk_a * 2 + ((pp >> 1) & 1)) * 512 + (pp & 1);
-            unit_b = ((size_t)(pp >> 2) * mx_nblk_b * 2 + ((pp >> 1) & 1)) * 512 + (pp & 1);
+            unit_a = ((pp >> 2) * mx_nblk_a * 2 + ((pp >> 1) & 1)) * 512 + (pp & 1);
+            unit_b = ((pp >> 2) * mx_nblk_b * 2 + ((pp >> 1) & 1)) * 512 + (pp & 1);
 #pragma unroll
-            for (int g = 0; g < MT; ++g) f.sa[g] = mx_a[g][unit_a];
+            for (int g = 0; g < MT; ++g) f.sa[g] = __builtin_amdgcn_raw_buffer_load_b8(rs_sa, mx_a[g], unit_a, 0);
         }
         if constexpr (MODE == MODE_F4T) {
             // FP4: a pair of 64-byte blocks is two 128-element K steps, whose two scale bytes sit side by side
-            unit_a = ((size_t)(pp >> 1) * mx_nblk_a * 2 + (pp & 1)) * 512;
-            unit_b = ((size_t)(pp >> 1) * mx_nblk_b * 2 + (pp & 1)) * 512;
+            unit_a = ((pp >> 1) * mx_nblk_a * 2 + (pp & 1)) * 512;
+            unit_b = ((pp >> 1) * mx_nblk_b * 2 + (pp & 1)) * 512;
 #pragma unroll
-            for (int g = 0; g < MT; ++g) f.sa[g] = *(const unsigned short*)(mx_a[g] + unit_a);
+            for (int g = 0; g < MT; ++g) f.sa[g] = __builtin_amdgcn_raw_buffer_load_b16(rs_sa, mx_a[g], unit_a, 0);
         }
         if constexpr (MODE == MODE_BLOCK) {
 #pragma unroll
@@ -230,11 +243,11 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            f.b[t][0] = __builtin_nontemporal_load((const v4i*)(b_base + ((size_t)b_off[t] + (size_t)kt0 * 1024) + lane16));
-            f.b[t][1] = has1 ? __builtin_nontemporal_load((const v4i*)(b_base + ((size_t)b_off[t] + (size_t)kt1 * 1024) + lane16))
+            f.b[t][0] = ld16_nt(rs_b, lane16, b_off[t] + kt0 * 1024);
+            f.b[t][1] = has1 ? ld16_nt(rs_b, lane16, b_off[t] + kt1 * 1024)
                              : v4i{0, 0, 0, 0};
-            if constexpr (MODE == MODE_MXT) f.sb[t] = mx_b[t][unit_b];
-            if constexpr (MODE == MODE_F4T) f.sb[t] = *(const unsigned short*)(mx_b[t] + unit_b);
+            if constexpr (MODE == MODE_MXT) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b8(rs_sb, mx_b[t], unit_b, 0);
+            if constexpr (MODE == MODE_F4T) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b16(rs_sb, mx_b[t], unit_b, 0);
             if constexpr (MODE == MODE_BLOCK) f.fsb[t] = blk_b[t][pp];
         }
     };
