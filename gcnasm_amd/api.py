@@ -232,7 +232,7 @@ def gemm_a4w4(a, b, sfa, sfb, scale_mode=MX_TILED, c=None, c_dtype=BF16, n=None)
 
 
 def flatmm_a4w4(a, b_shuffled, sfa_tiled, sfb_tiled, n, c=None, c_dtype=BF16):
-    """MXFP4 skinny-M GEMM through a4w4_flatmm: a [M, K/2] packed E2M1 with M <= 64, b_shuffled from
+    """MXFP4 skinny-M GEMM through a4w4_flatmm: a [M, K/2] packed E2M1 with M <= 128, b_shuffled from
     preshuffle_b_device on the packed weight bytes [N, K/2], both scale arrays in the MX_TILED layout."""
     m, k = a.shape[-2], a.shape[-1] * 2
     c, c_dtype = _out(c, (m, n), c_dtype, a.device)

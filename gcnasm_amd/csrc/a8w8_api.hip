@@ -327,6 +327,10 @@ int dispatch_general(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s
     A8W8_DISPATCH(launch_general, g->scale_mode, g->c_dtype, p, g->batch, s)
 }
 
+// The flat kernels take up to 128 activation rows: up to four groups of 16 share one pass over the weights, past
+// 64 rows two workgroups per group of weight tiles make two passes (the second one from L2).
+constexpr int FLAT_MAX_M = 128;
+
 int validate_flat(const a8w8_gemm_args* g)
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
@@ -336,7 +340,7 @@ int validate_flat(const a8w8_gemm_args* g)
         return A8W8_ERR_BAD_MODE;
     const int st = validate_common(g);
     if (st != A8W8_OK) return st;
-    if (g->m > 64) return A8W8_ERR_BAD_SHAPE;
+    if (g->m > FLAT_MAX_M) return A8W8_ERR_BAD_SHAPE;
     if (g->n % 16 != 0 || g->k % 64 != 0) return A8W8_ERR_BAD_GROUP;
     if (!aligned16(g->a) || !aligned16(g->b) || g->stride_a % 16 != 0) return A8W8_ERR_MISALIGNED;
     if (g->batch > 1 && (g->stride_a_batch % 16 != 0 || g->stride_b_batch % 16 != 0)) return A8W8_ERR_MISALIGNED;
@@ -366,18 +370,21 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 {
     const long long tiles = (long long)(p.n / 16) * batch;
     const int cus = num_cus();
-    if (p.m > 48) {
+    // row groups per workgroup: all of them up to four, an even split over two passes beyond
+    const int groups = (p.m + 15) / 16, passes = (groups + 3) / 4;
+    const int mt = (groups + passes - 1) / passes;
+    if (mt == 4) {
         // four weight tiles x four row groups fill the register file; MX or block scales on top would spill
         if constexpr (MODE != MODE_BLOCK && MODE != MODE_MXT && MODE != MODE_F4T) {
             if (tiles >= 4ll * cus) return launch_flat_nt<4, 4, CDT, MODE>(p, batch, stream);
         }
         return launch_flat_nt<2, 4, CDT, MODE>(p, batch, stream);
     }
-    if (p.m > 32) {
+    if (mt == 3) {
         if (tiles >= 4ll * cus) return launch_flat_nt<4, 3, CDT, MODE>(p, batch, stream);
         return launch_flat_nt<2, 3, CDT, MODE>(p, batch, stream);
     }
-    if (p.m > 16) {
+    if (mt == 2) {
         if (tiles >= 4ll * cus) return launch_flat_nt<4, 2, CDT, MODE>(p, batch, stream);
         return launch_flat_nt<2, 2, CDT, MODE>(p, batch, stream);
     }
@@ -400,16 +407,21 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 //   28672 x 4096   FP8 21 / 23 / 26 / 28 against 26-27, MXFP8 22 / 25 / 28 / 40 against 26-28,
 //                  MXFP4 13 / 16 / 17 / 25 against 15-16, bf16 43 / 43 / 48 / 52 against 47-48
 // The model takes the faster side in these except where the two are within ~8% of each other.
+// 64 < M <= 128 (two flat passes, FP8, M = 80 / 96 / 128): 16384 x 7168 flat 42 / 40 / 41 against 41 / 43 / 47,
+// 8192 x 8192 flat 29 / 29 / 30 against 42 / 43 / 45, 28672 x 4096 flat 46 / 46 / 48 against 28 / 29 / 31.
 bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop)
 {
     const double w = (double)n * (double)row_bytes;
     if (w <= (double)(32ll << 20)) return true;
-    const int groups = (m + 15) / 16;
+    const int groups = (m + 15) / 16, passes = (groups + 3) / 4;
+    const int mt = (groups + passes - 1) / passes;
     const int cus = num_cus();
     const int rounds = ((n + 127) / 128 + cus - 1) / cus;
-    double flat = 3.5 + w / 6.3e6 + 2.0 * (groups - 1);
-    if (groups == 4 && scaled_in_loop) flat *= 1.3;
-    const double dense = 4.0 + std::max(rounds * 128.0 * (double)row_bytes / 28.0e3, w / 5.0e6);
+    double flat = 3.5 + w / 6.3e6 + 2.0 * (mt - 1);
+    if (mt == 4 && scaled_in_loop) flat *= 1.3;
+    if (passes == 2) flat *= 1.55;      // the second pass reads the weights from L2
+    double dense = 4.0 + std::max(rounds * 128.0 * (double)row_bytes / 28.0e3, w / 5.0e6);
+    if (m > 64) dense *= 1.0 + 0.25 * (m - 64) / 64.0;
     return flat <= dense;
 }
 
@@ -467,7 +479,7 @@ static int a16w16_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
     // a skinny problem on shuffled weights: the flat kernel where it is the faster one (and can run it)
-    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= 64 && prefer_flat(g->m, g->n, 2ll * g->k, false) &&
+    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= FLAT_MAX_M && prefer_flat(g->m, g->n, 2ll * g->k, false) &&
         a16w16_flat_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     if (!g->a || !g->b || !g->c) return A8W8_ERR_NULL_POINTER;
@@ -521,7 +533,7 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
     // a skinny problem on shuffled weights: the flat kernel where it is the faster one (and can run it)
-    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= 64 && prefer_flat(g->m, g->n, g->k / 2, true) &&
+    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= FLAT_MAX_M && prefer_flat(g->m, g->n, g->k / 2, true) &&
         a4w4_flat_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
@@ -581,7 +593,7 @@ static int a4w4_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
     if (!g) return A8W8_ERR_NULL_POINTER;
     if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
     if (!g->b_preshuffled || g->scale_mode != A8W8_SCALE_MX_E8M0_TILED) return A8W8_ERR_BAD_MODE;
-    if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0 || g->m > 64) return A8W8_ERR_BAD_SHAPE;
+    if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0 || g->m > FLAT_MAX_M) return A8W8_ERR_BAD_SHAPE;
     if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
     if (g->n % 16 != 0 || g->k % 128 != 0) return A8W8_ERR_BAD_GROUP;
     if (g->stride_c < g->n || g->stride_a < g->k) return A8W8_ERR_BAD_STRIDE;
@@ -649,7 +661,7 @@ static int a16w16_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     if (!g) return A8W8_ERR_NULL_POINTER;
     if (!g->a || !g->b || !g->c) return A8W8_ERR_NULL_POINTER;
     if (!g->b_preshuffled) return A8W8_ERR_BAD_MODE;
-    if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0 || g->m > 64) return A8W8_ERR_BAD_SHAPE;
+    if (g->m <= 0 || g->n <= 0 || g->k <= 0 || g->batch <= 0 || g->m > FLAT_MAX_M) return A8W8_ERR_BAD_SHAPE;
     if (g->c_dtype != A8W8_C_BF16 && g->c_dtype != A8W8_C_FP32) return A8W8_ERR_BAD_MODE;
     if (g->n % 16 != 0 || g->k % 32 != 0) return A8W8_ERR_BAD_GROUP;
     if (g->stride_c < g->n || g->stride_a < g->k) return A8W8_ERR_BAD_STRIDE;
@@ -986,7 +998,7 @@ const char* a8w8_status_string(int status)
     switch (status) {
         case A8W8_OK: return "ok";
         case A8W8_ERR_NULL_POINTER: return "null pointer";
-        case A8W8_ERR_BAD_SHAPE: return "m, n, k and batch must be positive (and m <= 64 for flatmm)";
+        case A8W8_ERR_BAD_SHAPE: return "m, n, k and batch must be positive (and m <= 128 for the flat GEMMs)";
         case A8W8_ERR_BAD_GROUP: return "m/n/k must be multiples of the scale group (or of the shuffle tile)";
         case A8W8_ERR_BAD_STRIDE: return "a stride is smaller than the extent it spans";
         case A8W8_ERR_MISALIGNED: return "pointer or stride not 16-byte aligned";

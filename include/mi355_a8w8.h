@@ -103,7 +103,7 @@ A8W8_API int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream);
 A8W8_API int a16w16_gemm(const a8w8_gemm_args* args, void* hip_stream);
 
 /* The bf16 flat GEMM (flatmm_a16w16_gfx950, opus_fmm/README.md:10,51-57; source absent): A [batch, m, k]
- * bf16 with m <= 64, B bf16 pre-shuffled as a byte matrix -- a8w8_preshuffle_b[_device](b, out, n, 2*k) --
+ * bf16 with m <= 128, B bf16 pre-shuffled as a byte matrix -- a8w8_preshuffle_b[_device](b, out, n, 2*k) --
  * n % 16 == 0, k % 32 == 0, a, b and the rows of A 16-byte aligned, no scales, bf16 or fp32 C.  Same
  * streaming kernel as a8w8_flatmm. */
 A8W8_API int a16w16_flatmm(const a8w8_gemm_args* args, void* hip_stream);
@@ -117,7 +117,7 @@ A8W8_API int a16w16_flatmm(const a8w8_gemm_args* args, void* hip_stream);
 A8W8_API int a4w4_gemm(const a8w8_gemm_args* args, void* hip_stream);
 /* MXFP4 skinny-M GEMM over pre-shuffled weights (no counterpart in the reference, which has neither an FP4
  * program nor a flat one for it; it is a8w8_flatmm for the FP4 form of the same instruction).  A [batch, m, k/2
- * bytes] with m <= 64; B pre-shuffled as the byte matrix it is -- a8w8_preshuffle_b[_device](b, out, n, k/2) --
+ * bytes] with m <= 128; B pre-shuffled as the byte matrix it is -- a8w8_preshuffle_b[_device](b, out, n, k/2) --
  * with b_preshuffled != 0; sfa, sfb E8M0 in the MX_E8M0_TILED layout (a4w4_quantize_mx(tiled) or
  * a8w8_mx_tile_scales), scale_mode = MX_E8M0_TILED; n % 16 == 0, k % 128 == 0; m, n, k and the strides count
  * elements; a, b, sfa, sfb and the rows of A 16-byte aligned.  B is streamed once with 16-byte non-temporal loads. */
@@ -137,8 +137,9 @@ A8W8_API int a8w8_gemm_blockscale(const a8w8_gemm_args* args, void* hip_stream);
  * opus_fmm/README.md:9, built by opus_fmm/rebuild.sh:3-13).  Requires b_preshuffled != 0,
  * scale_mode ROWCOL, TENSOR, BLOCK_1x128_128x128 (scale arrays as for a8w8_gemm_blockscale; n, k % 128 == 0) or
  * MX_E8M0_TILED (MXFP8: both scale arrays in the tiled layout, 16-byte aligned),
- * m <= 64, n % 16 == 0, k % 64 == 0, a, b and the rows of A 16-byte aligned (A8W8_ERR_MISALIGNED otherwise).
- * B is streamed once, with 16-byte non-temporal loads, for all rows of A.  Where a8w8_gemm's kernels are the
+ * m <= 128, n % 16 == 0, k % 64 == 0, a, b and the rows of A 16-byte aligned (A8W8_ERR_MISALIGNED otherwise).
+ * B is streamed once, with 16-byte non-temporal loads, for up to 64 rows of A (twice, the second time from
+ * cache, beyond).  Where a8w8_gemm's kernels are the
  * faster ones on the same shuffled weights (several groups of 16 rows over many short weight rows; k % 128 == 0
  * permitting) the call runs those, and a8w8_gemm with b_preshuffled takes this kernel for the skinny problems it
  * runs faster: either entry point gives the same kernel for the same problem. */

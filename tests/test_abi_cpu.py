@@ -63,7 +63,7 @@ def test_flatmm_preconditions():
     a = _ok_args(mode=g.ROWCOL, m=16, n=256, k=256, b_preshuffled=1)
     assert g.kernel_name(a) == "flatmm_a8w8"
     for mutate, want in [(lambda x: setattr(x, "b_preshuffled", 0), -6), (lambda x: setattr(x, "scale_mode", g.MX), -6),
-                         (lambda x: setattr(x, "m", 65), -2), (lambda x: setattr(x, "n", 250), -3),
+                         (lambda x: setattr(x, "m", 129), -2), (lambda x: setattr(x, "n", 250), -3),
                          (lambda x: setattr(x, "k", 96), -3), (lambda x: setattr(x, "a", 0x1001), -5)]:
         b = _ok_args(mode=g.ROWCOL, m=16, n=256, k=256, b_preshuffled=1)
         mutate(b)
@@ -186,7 +186,7 @@ def test_sibling_entry_points_reject_bad_arguments():
         assert L.a16w16_gemm(ref(b), None) == want
     assert L.a16w16_gemm(None, None) == -1
     # a16w16_flatmm
-    for mutate, want in [(lambda x: setattr(x, "b_preshuffled", 0), -6), (lambda x: setattr(x, "m", 65), -2),
+    for mutate, want in [(lambda x: setattr(x, "b_preshuffled", 0), -6), (lambda x: setattr(x, "m", 129), -2),
                          (lambda x: setattr(x, "n", 250), -3), (lambda x: setattr(x, "k", 48), -3),
                          (lambda x: setattr(x, "stride_a", 260), -5), (lambda x: setattr(x, "a", 0x1008), -5)]:
         b = _ok_args(mode=g.TENSOR, m=16, n=256, k=256, b_preshuffled=1)
@@ -202,7 +202,7 @@ def test_sibling_entry_points_reject_bad_arguments():
         assert L.a4w4_gemm(ref(b), None) == want, want
     # a4w4_flatmm: pre-shuffled packed weights, tiled scales only
     for mutate, want in [(lambda x: setattr(x, "b_preshuffled", 0), -6), (lambda x: setattr(x, "scale_mode", g.MX), -6),
-                         (lambda x: setattr(x, "m", 65), -2), (lambda x: setattr(x, "n", 250), -3),
+                         (lambda x: setattr(x, "m", 129), -2), (lambda x: setattr(x, "n", 250), -3),
                          (lambda x: setattr(x, "k", 192), -3), (lambda x: setattr(x, "stride_a", 272), -5),
                          (lambda x: setattr(x, "sfb", 0x5004), -5), (lambda x: setattr(x, "sfa", None), -1)]:
         b = _ok_args(mode=g.MX_TILED, m=16, n=256, k=256, b_preshuffled=1)

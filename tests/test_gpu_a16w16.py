@@ -100,7 +100,7 @@ def test_flat_gemm_exact_integers_and_decode_shape(orc):
     assert torch.equal(g.flatmm_a16w16(a, g.preshuffle_b_bf16_device(b), n, c_dtype=g.FP32), want)
 
 
-@pytest.mark.parametrize("m", [17, 33, 48, 49, 64])
+@pytest.mark.parametrize("m", [17, 33, 48, 49, 64, 80, 128])
 @pytest.mark.parametrize("n,batch", [(144, 2), (288, 57)])      # two / four weight tiles per workgroup
 def test_flat_gemm_row_groups_exact(m, n, batch):
     """M > 16: up to four groups of 16 rows share one pass over the weights (rows staged through LDS)."""

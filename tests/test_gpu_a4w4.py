@@ -132,7 +132,7 @@ def test_flat_scale_bytes_reach_the_right_lane_and_block(orc, case):
     magnitude <= 6 and the scales are 2^-1..2^1, so sums are exact in fp32 and any mix-up of row, block or the
     pair's byte changes the result."""
     r = np.random.default_rng(8000 + case)
-    m = int(r.integers(1, 65))
+    m = int(r.integers(1, 129))
     n = 16 * int(r.integers(1, 70))
     k = 128 * int(r.integers(1, 24))
     qa = r.integers(0, 256, (m, k // 2)).astype(np.uint8)
@@ -146,7 +146,7 @@ def test_flat_scale_bytes_reach_the_right_lane_and_block(orc, case):
     assert (_flat(qa, qb, ea, eb, g.BF16) == torch.from_numpy(exact.astype(np.float32)).to(torch.bfloat16).float().numpy()).all()
 
 
-@pytest.mark.parametrize("m", [17, 32, 33, 48, 49, 64])
+@pytest.mark.parametrize("m", [17, 32, 33, 48, 49, 64, 80, 128])
 def test_flat_row_groups_four_weight_tiles(orc, m):
     """Enough weight tiles for four per workgroup (two past 48 rows), 1025 of them so that the last workgroup holds
     one; 2 / 3 / 4 groups of 16 rows share the pass over the weights."""
@@ -170,6 +170,6 @@ def test_flat_rejects_what_it_cannot_run():
     with pytest.raises(g.A8W8Error, match="aligned"):
         g.flatmm_a4w4(torch.zeros((16, 64 + 8), dtype=torch.uint8, device="cuda")[:, :64], bs, t, t, 16)
     with pytest.raises(g.A8W8Error):
-        g.flatmm_a4w4(torch.zeros((65, 64), dtype=torch.uint8, device="cuda"), bs, t, t, 16)
+        g.flatmm_a4w4(torch.zeros((129, 64), dtype=torch.uint8, device="cuda"), bs, t, t, 16)
     with pytest.raises(g.A8W8Error):
         g.flatmm_a4w4(torch.zeros((16, 32), dtype=torch.uint8, device="cuda"), bs, t, t, 16)      # k = 64: not a whole block

@@ -59,7 +59,7 @@ def test_flatmm_mx_scale_bytes_reach_the_right_lane_and_step(orc, case):
     """Small integers with a distinct power of two per (row, 32-block): sums are exact in fp32, so any mix-up of
     row, block or K step changes the result."""
     r = np.random.default_rng(8100 + case)
-    m = int(r.integers(1, 65))
+    m = int(r.integers(1, 129))
     n = 16 * int(r.integers(1, 70))
     k = 64 * int(r.integers(1, 40))
     a, b = datagen.small_ints(m, n, k, seed=8200 + case)
@@ -102,7 +102,7 @@ def test_flatmm_block_scales_exact(orc, case):
     import torch
     from gpu_util import dev
     r = np.random.default_rng(8300 + case)
-    m = int(r.integers(1, 65))
+    m = int(r.integers(1, 129))
     n = 128 * int(r.integers(1, 9))
     k = 128 * int(r.integers(1, 20))
     a, b = datagen.small_ints(m, n, k, seed=8400 + case)
@@ -163,7 +163,7 @@ def _row_group_case(orc, mode, m, n, k, batch, seed):
     assert bad.size == 0, f"mode {mode} {batch}x{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
 
 
-@pytest.mark.parametrize("m", [17, 32, 33, 47, 48, 49, 63, 64])
+@pytest.mark.parametrize("m", [17, 32, 33, 47, 48, 49, 63, 64, 65, 80, 97, 128])
 @pytest.mark.parametrize("mode", [g.ROWCOL, g.TENSOR, g.MX_TILED, g.BLOCK])
 def test_row_groups_two_weight_tiles(orc, mode, m):
     """Few weight tiles: two per workgroup, 2 / 3 / 4 row groups; 9 tiles leave the last workgroup half empty."""
@@ -171,7 +171,7 @@ def test_row_groups_two_weight_tiles(orc, mode, m):
     _row_group_case(orc, mode, m, n, k, 2, 8500 + m)
 
 
-@pytest.mark.parametrize("m", [17, 32, 33, 48, 49, 64])
+@pytest.mark.parametrize("m", [17, 32, 33, 48, 49, 64, 81, 96, 113, 128])
 @pytest.mark.parametrize("mode", [g.ROWCOL, g.TENSOR, g.MX_TILED, g.BLOCK])
 def test_row_groups_four_weight_tiles(orc, mode, m):
     """At least four weight tiles per compute unit over all batch entries: four per workgroup (two for MX and block

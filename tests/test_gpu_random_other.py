@@ -43,7 +43,7 @@ def _c(r, m, n):
 @pytest.mark.parametrize("case", range(CASES))
 def test_flatmm_fp8(case):
     r = np.random.default_rng(7000 + case)
-    m = int(r.integers(1, 65))
+    m = int(r.integers(1, 129))
     n = 16 * int(r.integers(1, 80))
     k = 64 * int(r.integers(1, 40))
     mode = [g.ROWCOL, g.TENSOR][case % 2]
@@ -78,7 +78,7 @@ def test_flat_gemms_reject_misaligned_rows():
 def test_bf16_gemm_and_flat(case):
     r = np.random.default_rng(7100 + case)
     flat = case % 3 == 0
-    m = int(r.integers(1, 65)) if flat else int(r.choice([1, 17, 64, 200, 256, 300, 513]))
+    m = int(r.integers(1, 129)) if flat else int(r.choice([1, 17, 64, 200, 256, 300, 513]))
     n = 16 * int(r.integers(1, 40)) if flat else int(r.choice([1, 24, 64, 255, 256, 384, 520]))
     k = 32 * int(r.integers(1, 40)) if flat else int(r.choice([8, 40, 64, 128, 192, 256, 448, 512, 1024]))
     a = torch.from_numpy(r.integers(-8, 9, (m, k)).astype(np.float32)).to(torch.bfloat16)
