@@ -373,6 +373,13 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
     // row groups per workgroup: all of them up to four, an even split over two passes beyond
     const int groups = (p.m + 15) / 16, passes = (groups + 3) / 4;
     const int mt = (groups + passes - 1) / passes;
+    if (groups > 4 && tiles < 4ll * cus) {
+        // too few weight tiles for four per workgroup: two passes would run two tiles per workgroup anyway, and one
+        // pass with six or eight row groups on two tiles reads the weights once (8192 x 8192, M = 128: 30 -> 25 us)
+        if (groups <= 6) return launch_flat_nt<2, 6, CDT, MODE>(p, batch, stream);
+        if constexpr (MODE != MODE_BLOCK && MODE != MODE_MXT && MODE != MODE_F4T)      // eight groups + scales would spill
+            return launch_flat_nt<2, 8, CDT, MODE>(p, batch, stream);
+    }
     if (mt == 4) {
         // four weight tiles x four row groups fill the register file; MX or block scales on top would spill
         if constexpr (MODE != MODE_BLOCK && MODE != MODE_MXT && MODE != MODE_F4T) {
@@ -408,7 +415,7 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 //                  MXFP4 13 / 16 / 17 / 25 against 15-16, bf16 43 / 43 / 48 / 52 against 47-48
 // The model takes the faster side in these except where the two are within ~8% of each other.
 // 64 < M <= 128 (two flat passes, FP8, M = 80 / 96 / 128): 16384 x 7168 flat 42 / 40 / 41 against 41 / 43 / 47,
-// 8192 x 8192 flat 29 / 29 / 30 against 42 / 43 / 45, 28672 x 4096 flat 46 / 46 / 48 against 28 / 29 / 31.
+// 8192 x 8192 flat 29 / 29 / 30 (20 / 22 / 25 in one pass on two weight tiles, which is what runs there) against 42 / 43 / 45, 28672 x 4096 flat 46 / 46 / 48 against 28 / 29 / 31.
 bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop)
 {
     const double w = (double)n * (double)row_bytes;
@@ -417,9 +424,14 @@ bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop)
     const int mt = (groups + passes - 1) / passes;
     const int cus = num_cus();
     const int rounds = ((n + 127) / 128 + cus - 1) / cus;
-    double flat = 3.5 + w / 6.3e6 + 2.0 * (mt - 1);
-    if (mt == 4 && scaled_in_loop) flat *= 1.3;
-    if (passes == 2) flat *= 1.55;      // the second pass reads the weights from L2
+    double flat;
+    if (groups > 4 && n / 16 < 4 * cus && (groups <= 6 || !scaled_in_loop)) {
+        flat = 3.5 + w / 6.3e6 + 2.0 * (groups - 1);      // one pass with six or eight row groups (see launch_flat)
+    } else {
+        flat = 3.5 + w / 6.3e6 + 2.0 * (mt - 1);
+        if (mt == 4 && scaled_in_loop) flat *= 1.3;
+        if (passes == 2) flat *= 1.55;      // the second pass reads the weights from L2
+    }
     double dense = 4.0 + std::max(rounds * 128.0 * (double)row_bytes / 28.0e3, w / 5.0e6);
     if (m > 64) dense *= 1.0 + 0.25 * (m - 64) / 64.0;
     return flat <= dense;
