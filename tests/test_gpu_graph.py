@@ -85,3 +85,40 @@ def test_per_tensor_quantiser_replays():
         torch.cuda.synchronize()
         assert torch.equal(got_q, q) and torch.equal(got_s, s)
         assert np.isclose(float(got_s[0]), float(x.abs().max()) / 448.0, rtol=1e-6)
+
+
+@pytest.mark.parametrize("m", [16, 48, 128])      # fragments gathered from memory / rows staged through LDS / two row-group sets
+def test_flat_gemm_replays(m):
+    """Decode step under capture: quantise the activations, flat GEMM over shuffled weights."""
+    n, k = 2048, 1024
+    xa, xb = _fresh((m, k), 5), _fresh((n, k), 6)
+    qb, sb = g.quantize(xb, g.ROWCOL)
+    bs = g.preshuffle_b_device(qb)
+    qa = torch.empty((m, k), dtype=torch.uint8, device="cuda")
+    sa = torch.empty(m, dtype=torch.float32, device="cuda")
+    c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    L = g.lib()
+
+    def step():
+        assert L.a8w8_quantize(xa.data_ptr(), m, k, k, qa.data_ptr(), sa.data_ptr(), g.ROWCOL, 1, g.api._stream()) == 0
+        g.flatmm(qa, bs, sa, sb, n, c=c)
+
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        xa.copy_(_fresh((m, k), 40 + rep))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = c.clone()
+        c.zero_()
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(got, c), f"replay {rep} differs from the eager result"
+        ref = xa @ xb.T
+        assert (got.float() - ref).abs().max() <= 0.08 * ref.abs().max()      # FP8 quantisation error, not a parity bound
