@@ -353,19 +353,19 @@ int validate_flat(const a8w8_gemm_args* g)
 // Weight tiles (16 rows of B) per workgroup: the activation fragment of a K block is re-used by all of them, but
 // the grid shrinks by the same factor: the largest of 4, 2, 1 that still gives every compute unit a workgroup
 // (16 x 4096 x 4096: 8.6 us with 4 tiles per workgroup on 64 compute units, 5.4 us with 1 on 256).
-template <int NT, int MT, int CDT, int MODE>
+template <int NT, int MT, int CDT, int MODE, bool BROW>
 int launch_flat_nt(const GemmParams& p, int batch, hipStream_t stream)
 {
     const int n_tiles = p.n / 16;
     dim3 grid((unsigned)(((n_tiles + NT - 1) / NT) * ((p.m + 16 * MT - 1) / (16 * MT))), 1, (unsigned)batch);
-    hipLaunchKernelGGL((flatmm_a8w8<NT, MT, CDT, MODE>), grid, dim3(FLAT_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((flatmm_a8w8<NT, MT, CDT, MODE, BROW>), grid, dim3(FLAT_THREADS), 0, stream, p);
     return launch_status();
 }
 
 // Up to four groups of 16 activation rows share one pass over the weights; as many weight tiles per workgroup as
 // still leave every compute unit a workgroup (every workgroup reads all rows of A once, so more weight tiles per
 // workgroup also means fewer reads of A: 16384 x 7168 at M = 48, 30 us with two tiles, 24 us with four).
-template <int CDT, int MODE>
+template <int CDT, int MODE, bool BROW = false>
 int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 {
     const long long tiles = (long long)(p.n / 16) * batch;
@@ -376,28 +376,29 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
     if (groups > 4 && tiles < 4ll * cus) {
         // too few weight tiles for four per workgroup: two passes would run two tiles per workgroup anyway, and one
         // pass with six or eight row groups on two tiles reads the weights once (8192 x 8192, M = 128: 30 -> 25 us)
-        if (groups <= 6) return launch_flat_nt<2, 6, CDT, MODE>(p, batch, stream);
-        if constexpr (MODE != MODE_BLOCK && MODE != MODE_MXT && MODE != MODE_F4T)      // eight groups + scales would spill
-            return launch_flat_nt<2, 8, CDT, MODE>(p, batch, stream);
+        if (groups <= 6) return launch_flat_nt<2, 6, CDT, MODE, BROW>(p, batch, stream);
+        // eight groups + scales would spill; with row-major weights their staging does not fit LDS
+        if constexpr (MODE != MODE_BLOCK && MODE != MODE_MXT && MODE != MODE_F4T && !BROW)
+            return launch_flat_nt<2, 8, CDT, MODE, BROW>(p, batch, stream);
     }
     if (mt == 4) {
         // four weight tiles x four row groups fill the register file; MX or block scales on top would spill
         if constexpr (MODE != MODE_BLOCK && MODE != MODE_MXT && MODE != MODE_F4T) {
-            if (tiles >= 4ll * cus) return launch_flat_nt<4, 4, CDT, MODE>(p, batch, stream);
+            if (tiles >= 4ll * cus) return launch_flat_nt<4, 4, CDT, MODE, BROW>(p, batch, stream);
         }
-        return launch_flat_nt<2, 4, CDT, MODE>(p, batch, stream);
+        return launch_flat_nt<2, 4, CDT, MODE, BROW>(p, batch, stream);
     }
     if (mt == 3) {
-        if (tiles >= 4ll * cus) return launch_flat_nt<4, 3, CDT, MODE>(p, batch, stream);
-        return launch_flat_nt<2, 3, CDT, MODE>(p, batch, stream);
+        if (tiles >= 4ll * cus) return launch_flat_nt<4, 3, CDT, MODE, BROW>(p, batch, stream);
+        return launch_flat_nt<2, 3, CDT, MODE, BROW>(p, batch, stream);
     }
     if (mt == 2) {
-        if (tiles >= 4ll * cus) return launch_flat_nt<4, 2, CDT, MODE>(p, batch, stream);
-        return launch_flat_nt<2, 2, CDT, MODE>(p, batch, stream);
+        if (tiles >= 4ll * cus) return launch_flat_nt<4, 2, CDT, MODE, BROW>(p, batch, stream);
+        return launch_flat_nt<2, 2, CDT, MODE, BROW>(p, batch, stream);
     }
-    if (tiles >= 4ll * cus) return launch_flat_nt<4, 1, CDT, MODE>(p, batch, stream);
-    if (tiles >= 2ll * cus) return launch_flat_nt<2, 1, CDT, MODE>(p, batch, stream);
-    return launch_flat_nt<1, 1, CDT, MODE>(p, batch, stream);
+    if (tiles >= 4ll * cus) return launch_flat_nt<4, 1, CDT, MODE, BROW>(p, batch, stream);
+    if (tiles >= 2ll * cus) return launch_flat_nt<2, 1, CDT, MODE, BROW>(p, batch, stream);
+    return launch_flat_nt<1, 1, CDT, MODE, BROW>(p, batch, stream);
 }
 
 // On shuffled weights both the flat GEMM and the MFMA kernels can run a skinny problem; the entry points take the
@@ -414,9 +415,11 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 //   28672 x 4096   FP8 21 / 23 / 26 / 28 against 26-27, MXFP8 22 / 25 / 28 / 40 against 26-28,
 //                  MXFP4 13 / 16 / 17 / 25 against 15-16, bf16 43 / 43 / 48 / 52 against 47-48
 // The model takes the faster side in these except where the two are within ~8% of each other.
+// Row-major weights (a8w8_gemm without b_preshuffled; the flat kernel stages the weight rows through LDS): ~1.3x the
+// shuffled flat times -- 16384 x 7168 FP8 25 / 27 / 31 / 55, 8192 x 8192 20 / 20 / 22 / 37, 28672 x 4096 27 / 31 / - / -.
 // 64 < M <= 128 (two flat passes, FP8, M = 80 / 96 / 128): 16384 x 7168 flat 42 / 40 / 41 against 41 / 43 / 47,
 // 8192 x 8192 flat 29 / 29 / 30 (20 / 22 / 25 in one pass on two weight tiles, which is what runs there) against 42 / 43 / 45, 28672 x 4096 flat 46 / 46 / 48 against 28 / 29 / 31.
-bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop)
+bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, bool rowmajor = false)
 {
     const double w = (double)n * (double)row_bytes;
     if (w <= (double)(32ll << 20)) return true;
@@ -432,6 +435,7 @@ bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop)
         if (mt == 4 && scaled_in_loop) flat *= 1.3;
         if (passes == 2) flat *= 1.55;      // the second pass reads the weights from L2
     }
+    if (rowmajor) flat *= 1.3;      // weight rows staged through LDS, two half-line reads per row and pair
     double dense = 4.0 + std::max(rounds * 128.0 * (double)row_bytes / 28.0e3, w / 5.0e6);
     if (m > 64) dense *= 1.0 + 0.25 * (m - 64) / 64.0;
     return flat <= dense;
@@ -440,20 +444,42 @@ bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop)
 bool prefer_flat_fp8(const a8w8_gemm_args* g)
 {
     const bool scaled_in_loop = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED || g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128;
-    return prefer_flat(g->m, g->n, g->k, scaled_in_loop);
+    return prefer_flat(g->m, g->n, g->k, scaled_in_loop, !g->b_preshuffled);
+}
+
+template <bool BROW>
+int launch_flat_fp8_layout(const a8w8_gemm_args* g, hipStream_t s)
+{
+    const GemmParams p = make_params(g);
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED)
+        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_MXT, BROW>(p, g->batch, s) : launch_flat<C_FP32, MODE_MXT, BROW>(p, g->batch, s);
+    if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128)
+        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_BLOCK, BROW>(p, g->batch, s) : launch_flat<C_FP32, MODE_BLOCK, BROW>(p, g->batch, s);
+    const bool tensor = g->scale_mode == A8W8_SCALE_TENSOR;
+    if (g->c_dtype == A8W8_C_BF16)
+        return tensor ? launch_flat<C_BF16, MODE_TENSOR, BROW>(p, g->batch, s) : launch_flat<C_BF16, MODE_ROWCOL, BROW>(p, g->batch, s);
+    return tensor ? launch_flat<C_FP32, MODE_TENSOR, BROW>(p, g->batch, s) : launch_flat<C_FP32, MODE_ROWCOL, BROW>(p, g->batch, s);
 }
 
 int launch_flat_fp8(const a8w8_gemm_args* g, hipStream_t s)
 {
-    const GemmParams p = make_params(g);
-    if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED)
-        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_MXT>(p, g->batch, s) : launch_flat<C_FP32, MODE_MXT>(p, g->batch, s);
-    if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128)
-        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_BLOCK>(p, g->batch, s) : launch_flat<C_FP32, MODE_BLOCK>(p, g->batch, s);
-    const bool tensor = g->scale_mode == A8W8_SCALE_TENSOR;
-    if (g->c_dtype == A8W8_C_BF16)
-        return tensor ? launch_flat<C_BF16, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_BF16, MODE_ROWCOL>(p, g->batch, s);
-    return tensor ? launch_flat<C_FP32, MODE_TENSOR>(p, g->batch, s) : launch_flat<C_FP32, MODE_ROWCOL>(p, g->batch, s);
+    return g->b_preshuffled ? launch_flat_fp8_layout<false>(g, s) : launch_flat_fp8_layout<true>(g, s);
+}
+
+// A skinny problem on row-major weights that the flat kernel can run (it stages the weight rows through LDS).
+bool flat_rowmajor_ok(const a8w8_gemm_args* g)
+{
+    if (g->b_preshuffled || g->m > FLAT_MAX_M) return false;
+    if (g->scale_mode != A8W8_SCALE_ROWCOL && g->scale_mode != A8W8_SCALE_TENSOR && g->scale_mode != A8W8_SCALE_MX_E8M0_TILED &&
+        g->scale_mode != A8W8_SCALE_BLOCK_1x128_128x128)
+        return false;
+    if (g->n % 16 != 0 || g->k % 64 != 0) return false;
+    if (!aligned16(g->a) || !aligned16(g->b) || g->stride_a % 16 != 0 || g->stride_b % 16 != 0) return false;
+    if (g->batch > 1 && (g->stride_a_batch % 16 != 0 || g->stride_b_batch % 16 != 0)) return false;
+    if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED &&
+        (!aligned16(g->sfa) || !aligned16(g->sfb) || (g->batch > 1 && (g->stride_sfa_batch % 16 != 0 || g->stride_sfb_batch % 16 != 0))))
+        return false;
+    return (long long)(g->n - 1) * g->stride_b + g->k < (1ll << 31);
 }
 
 int launch_dense_fp8(const a8w8_gemm_args* g, hipStream_t s)
@@ -482,6 +508,7 @@ int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream)
     hipStream_t s = (hipStream_t)hip_stream;
     // a skinny problem on shuffled weights: the flat kernel where it is the faster one
     if (g->b_preshuffled && validate_flat(g) == A8W8_OK && prefer_flat_fp8(g)) return launch_flat_fp8(g, s);
+    if (flat_rowmajor_ok(g) && prefer_flat_fp8(g)) return launch_flat_fp8(g, s);
     return launch_dense_fp8(g, s);
 }
 
@@ -1033,6 +1060,7 @@ const char* a8w8_kernel_name(const a8w8_gemm_args* g)
     g = &local;
     const bool dense_ok = validate_common(g) == A8W8_OK && validate_shuffled_b(g) == A8W8_OK;
     if (g->b_preshuffled && validate_flat(g) == A8W8_OK && (prefer_flat_fp8(g) || !dense_ok)) return "flatmm_a8w8";
+    if (dense_ok && flat_rowmajor_ok(g) && prefer_flat_fp8(g)) return "flatmm_a8w8";
     if (!dense_ok) return nullptr;
     if (!tiled_ok(g)) return "gemm_a8w8_general";
     if (small_ok(g)) return "gemm_a8w8_tile128";

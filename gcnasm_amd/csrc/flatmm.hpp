@@ -63,14 +63,19 @@ constexpr int FLAT_STAGE_SLOTS = 8 * 18;
 // once per pair of K blocks).  With MT > 1 that gather would cost more than the weight stream, so the wave reads
 // the rows the coalesced way (four lanes per 128-byte line) and turns them into fragments through a private
 // piece of LDS; nothing is shared between waves, so the K loop still has no barrier.
-template <int NT, int MT, int CDT, int MODE>
+//
+// BROW: the weights are row-major ([n][ldb], not pre-shuffled).  Their 16-row tiles then take the road of the
+// activation rows of MT > 1: read the coalesced way, one register set in flight, through the wave's LDS into fragments.
+template <int NT, int MT, int CDT, int MODE, bool BROW = false>
 __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 {
     // the NT * MT output tiles are finished in rounds of up to eight, wave w taking tile 8 * round + w of the round
     constexpr int TILES = NT * MT;
     constexpr int ROUNDS = (TILES + FLAT_WAVES - 1) / FLAT_WAVES;
     constexpr int RED_SLOTS = FLAT_WAVES * (TILES < FLAT_WAVES ? TILES : FLAT_WAVES) * 64;
-    constexpr int STAGE_SLOTS = MT > 1 ? FLAT_WAVES * MT * FLAT_STAGE_SLOTS : 0;
+    constexpr int A_GROUPS = MT > 1 ? MT : 0;                 // staged row groups of A, then NT of row-major B
+    constexpr int STAGED = A_GROUPS + (BROW ? NT : 0);
+    constexpr int STAGE_SLOTS = FLAT_WAVES * STAGED * FLAT_STAGE_SLOTS;
     __shared__ v4i smem[RED_SLOTS > STAGE_SLOTS ? RED_SLOTS : STAGE_SLOTS];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -127,15 +132,21 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 #pragma unroll
     for (int g = 0; g < MT; ++g)
         a_off[g] = (uint32_t)min(m0 + g * 16 + ld_row, p.m - 1) * (uint32_t)p.lda + (MT == 1 ? kq * 16 : ld_c * 32);
-    v4i* stage = smem + wave * (MT * FLAT_STAGE_SLOTS);
-    const int st_write = (2 * ld_c) * 18 + ld_row;      // piece 2c, the next piece is 18 slots on
+    v4i* stage = smem + wave * (STAGED * FLAT_STAGE_SLOTS);
+    const int st_write = (2 * ld_c) * 18 + (lane >> 2);  // piece 2c of row lane / 4, the next piece is 18 slots on
     const int st_read = kq * 18 + r16;                   // piece kq, the second K block's is 4 * 18 slots on
 
-    const auto rs_b = make_rsrc(p.b + (long long)batch * p.b_batch, (uint32_t)p.n * (uint32_t)p.k);
+    const auto rs_b = make_rsrc(p.b + (long long)batch * p.b_batch, BROW ? (uint32_t)(p.n - 1) * (uint32_t)p.ldb + (uint32_t)p.k
+                                                                         : (uint32_t)p.n * (uint32_t)p.k);
     const uint32_t lane16 = lane * 16;
-    uint32_t b_off[NT];                                 // wave-uniform
+    uint32_t b_off[NT];                                 // shuffled B: wave-uniform; row-major B: the lane's row and piece
 #pragma unroll
-    for (int t = 0; t < NT; ++t) b_off[t] = (uint32_t)min(nt0 + t, n_tiles - 1) * (uint32_t)k_tiles * 1024u;
+    for (int t = 0; t < NT; ++t) {
+        if constexpr (BROW)
+            b_off[t] = (uint32_t)min((nt0 + t) * 16 + (lane >> 2), p.n - 1) * (uint32_t)p.ldb + ld_c * 32;
+        else
+            b_off[t] = (uint32_t)min(nt0 + t, n_tiles - 1) * (uint32_t)k_tiles * 1024u;
+    }
     // MX scales in the tiled layout of the dense kernels (mx_tiled_index): a pair of K blocks is one 128-wide K
     // step ks; lane (r16, kq) scales 32-block kq of its row, whose byte for step ks sits at
     // ((ks / 4 * nblk + blk) * 2 + (ks / 2) % 2) * 512 + ((4x + y) * 4 + kq) * 8 + jp * 4 + par * 2 + ks % 2
@@ -193,6 +204,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     };
     // MT > 1: the rows of one pair in flight (one register set: a pair's rows go to LDS before the next is asked for)
     v4i raw[MT][2];
+    v4i raw_b[NT][2];          // BROW: the same for the rows of the weight tiles
     auto load_rows = [&](int pp) {
         // lanes c = 2, 3 hold the second K block of the pair
         const bool there = 2 * pp + 1 < k_tiles || ld_c < 2;
@@ -202,15 +214,30 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
             raw[g][1] = there ? ld16(rs_a, a_off[g], pp * 128 + 16) : v4i{0, 0, 0, 0};
         }
     };
+    auto load_weight_rows = [&](int pp) {
+        const bool there = 2 * pp + 1 < k_tiles || ld_c < 2;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            raw_b[t][0] = there ? ld16_nt(rs_b, b_off[t], pp * 128) : v4i{0, 0, 0, 0};
+            raw_b[t][1] = there ? ld16_nt(rs_b, b_off[t], pp * 128 + 16) : v4i{0, 0, 0, 0};
+        }
+    };
     // rows -> this wave's own LDS.  A wave's LDS operations complete in order, so the fragment reads that follow
     // see these writes, and these writes cannot pass the fragment reads of the pair before.
     auto stage_rows = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int g = 0; g < MT; ++g) {
+        for (int g = 0; g < A_GROUPS; ++g) {
             stage[g * FLAT_STAGE_SLOTS + st_write] = raw[g][0];
             stage[g * FLAT_STAGE_SLOTS + st_write + 18] = raw[g][1];
+        }
+        if constexpr (BROW) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                stage[(A_GROUPS + t) * FLAT_STAGE_SLOTS + st_write] = raw_b[t][0];
+                stage[(A_GROUPS + t) * FLAT_STAGE_SLOTS + st_write + 18] = raw_b[t][1];
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -243,15 +270,27 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            f.b[t][0] = ld16_nt(rs_b, lane16, b_off[t] + kt0 * 1024);
-            f.b[t][1] = has1 ? ld16_nt(rs_b, lane16, b_off[t] + kt1 * 1024)
-                             : v4i{0, 0, 0, 0};
+            if constexpr (!BROW) {
+                f.b[t][0] = ld16_nt(rs_b, lane16, b_off[t] + kt0 * 1024);
+                f.b[t][1] = has1 ? ld16_nt(rs_b, lane16, b_off[t] + kt1 * 1024) : v4i{0, 0, 0, 0};
+            }
             if constexpr (MODE == MODE_MXT) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b8(rs_sb, mx_b[t], unit_b, 0);
             if constexpr (MODE == MODE_F4T) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b16(rs_sb, mx_b[t], unit_b, 0);
             if constexpr (MODE == MODE_BLOCK) f.fsb[t] = blk_b[t][pp];
         }
     };
     auto mma = [&](const Frag& f) {
+        v4i blo[NT], bhi[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if constexpr (BROW) {
+                blo[t] = stage[(A_GROUPS + t) * FLAT_STAGE_SLOTS + st_read];
+                bhi[t] = stage[(A_GROUPS + t) * FLAT_STAGE_SLOTS + st_read + 4 * 18];
+            } else {
+                blo[t] = f.b[t][0];
+                bhi[t] = f.b[t][1];
+            }
+        }
 #pragma unroll
         for (int g = 0; g < MT; ++g) {
             v4i alo, ahi;
@@ -265,13 +304,12 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
             const v8i fa = v8i{alo.x, alo.y, alo.z, alo.w, ahi.x, ahi.y, ahi.z, ahi.w};
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                const v8i fb = v8i{f.b[t][0].x, f.b[t][0].y, f.b[t][0].z, f.b[t][0].w,
-                                   f.b[t][1].x, f.b[t][1].y, f.b[t][1].z, f.b[t][1].w};
+                const v8i fb = v8i{blo[t].x, blo[t].y, blo[t].z, blo[t].w, bhi[t].x, bhi[t].y, bhi[t].z, bhi[t].w};
                 if constexpr (MODE == MODE_BF16) {
                     // bf16 weights: a 1 KiB block is 16 rows x 32 bf16, one 16x16x32 MFMA operand
-                    acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, f.b[t][0]),
+                    acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, blo[t]),
                                                                         __builtin_bit_cast(v8bf, alo), acc[g][t], 0, 0, 0);
-                    acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, f.b[t][1]),
+                    acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, bhi[t]),
                                                                         __builtin_bit_cast(v8bf, ahi), acc[g][t], 0, 0, 0);
                 } else if constexpr (MODE == MODE_BLOCK) {
                     // each 128-wide K group yields a partial tile that is rescaled into the running sum
@@ -280,10 +318,10 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
                 } else if constexpr (MODE == MODE_F4T) {
                     // packed E2M1: a 64-byte block is 128 elements, one FP4 MFMA; op_sel picks the block's scale byte
                     acc[g][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        (v8i{f.b[t][0].x, f.b[t][0].y, f.b[t][0].z, f.b[t][0].w, 0, 0, 0, 0}), (v8i{alo.x, alo.y, alo.z, alo.w, 0, 0, 0, 0}),
+                        (v8i{blo[t].x, blo[t].y, blo[t].z, blo[t].w, 0, 0, 0, 0}), (v8i{alo.x, alo.y, alo.z, alo.w, 0, 0, 0, 0}),
                         acc[g][t], 4, 4, 0, f.sb[t], 0, f.sa[g]);
                     acc[g][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        (v8i{f.b[t][1].x, f.b[t][1].y, f.b[t][1].z, f.b[t][1].w, 0, 0, 0, 0}), (v8i{ahi.x, ahi.y, ahi.z, ahi.w, 0, 0, 0, 0}),
+                        (v8i{bhi[t].x, bhi[t].y, bhi[t].z, bhi[t].w, 0, 0, 0, 0}), (v8i{ahi.x, ahi.y, ahi.z, ahi.w, 0, 0, 0, 0}),
                         acc[g][t], 4, 4, 1, f.sb[t], 1, f.sa[g]);
                 } else if constexpr (MODE == MODE_MXT) {
                     acc[g][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[g][t], 0, 0, 0, f.sb[t], 0, f.sa[g]);
@@ -297,20 +335,25 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     if (wave < pairs) {
         Frag f0, f1;
         int pp = wave;
-        if constexpr (MT > 1) load_rows(pp);
+        constexpr bool STAGING = MT > 1 || BROW;
+        auto load_staged = [&](int q) {
+            if constexpr (MT > 1) load_rows(q);
+            if constexpr (BROW) load_weight_rows(q);
+        };
+        load_staged(pp);
         load(pp, f0);
         // two register stages, loads of the next pair in flight while the current one is used
         while (true) {
-            if constexpr (MT > 1) stage_rows();
+            if constexpr (STAGING) stage_rows();
             if (pp + PSTEP < pairs) {
-                if constexpr (MT > 1) load_rows(pp + PSTEP);
+                load_staged(pp + PSTEP);
                 load(pp + PSTEP, f1);
             }
             mma(f0);
             if ((pp += PSTEP) >= pairs) break;
-            if constexpr (MT > 1) stage_rows();
+            if constexpr (STAGING) stage_rows();
             if (pp + PSTEP < pairs) {
-                if constexpr (MT > 1) load_rows(pp + PSTEP);
+                load_staged(pp + PSTEP);
                 load(pp + PSTEP, f0);
             }
             mma(f1);
@@ -325,7 +368,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     constexpr int PER_ROUND = TILES < FLAT_WAVES ? TILES : FLAT_WAVES;
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
-        if (MT > 1 || r > 0) __syncthreads();
+        if (MT > 1 || BROW || r > 0) __syncthreads();
 #pragma unroll
         for (int j = 0; j < PER_ROUND; ++j) {
             const int c = r * FLAT_WAVES + j;

@@ -92,7 +92,10 @@ typedef struct {
  * the tiled kernels; other shapes run on a slower general kernel.  m, n edges are handled.
  * b_preshuffled != 0: B is in the a8w8_preshuffle_b layout (the weights a8w8_flatmm streams), so that one copy
  * of the weights serves prefill and decode; needs n % 16 == 0, k % 128 == 0 and 16-byte aligned pointers.
- * a16w16_gemm and a4w4_gemm accept it likewise for the weights their flat siblings stream (shuffled as bytes). */
+ * a16w16_gemm and a4w4_gemm accept it likewise for the weights their flat siblings stream (shuffled as bytes).
+ * Skinny problems (m <= 128, n % 16 == 0, k % 64 == 0, 16-byte aligned rows; per-tensor, row/column, block or
+ * tiled MX scales) run on the flat kernel of a8w8_flatmm where that is the faster one, on shuffled and on
+ * row-major weights alike. */
 A8W8_API int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream);
 
 /* The bf16 sibling (gemm_a16w16_8wave, the program opus_gemm/rebuild.sh:3-13 builds; its source is

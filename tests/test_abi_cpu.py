@@ -80,6 +80,14 @@ def test_gemm_on_shuffled_weights_preconditions():
     assert g.kernel_name(ok) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(mode=g.BLOCK, m=300, n=512, k=512, b_preshuffled=1)) == "gemm_a8w8_tile128"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, m=16, n=256, k=256, b_preshuffled=1)) == "flatmm_a8w8"     # flat when it can
+    # row-major weights, at most 128 rows: the flat kernel where it can run and the model calls it faster
+    rm = dict(mode=g.ROWCOL, n=16384, k=7168)
+    assert g.kernel_name(_ok_args(m=64, **rm)) == "flatmm_a8w8"
+    assert g.kernel_name(_ok_args(m=128, **rm)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(m=129, **rm)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(m=64, mode=g.ROWCOL, n=16384 + 8, k=7168)) == "gemm_a8w8_tile128"      # n % 16 != 0
+    assert g.kernel_name(_ok_args(m=16, mode=g.MX, n=4096, k=4096)) == "gemm_a8w8_tile128"              # row-major MX scales
+    assert g.kernel_name(_ok_args(m=16, mode=g.BLOCK, n=4096, k=4096)) == "flatmm_a8w8"
     # skinny problems: the side a cost model of the two kernels calls faster (the measured winners)
     big = dict(n=16384, k=7168, b_preshuffled=1)
     assert g.kernel_name(_ok_args(m=64, mode=g.ROWCOL, **big)) == "flatmm_a8w8"

@@ -118,7 +118,7 @@ def test_flatmm_block_scales_exact(orc, case):
 
 # ---------------------------------------------------------------- several row groups per workgroup (M > 16)
 
-def _row_group_case(orc, mode, m, n, k, batch, seed):
+def _row_group_case(orc, mode, m, n, k, batch, seed, rowmajor=False):
     """Exact small-integer problem, batched so that the launch picks the variant wanted; power-of-two scales
     distinct per row / group, so that a row group, weight tile, K block or scale taken from the wrong place
     changes the result."""
@@ -152,11 +152,17 @@ def _row_group_case(orc, mode, m, n, k, batch, seed):
         B = B * np.repeat(np.exp2(eb.astype(np.float64) - 127), 32, axis=2)
         da = torch.stack([g.mx_tile_scales(dev(ea[i])) for i in range(batch)])
         db = torch.stack([g.mx_tile_scales(dev(eb[i])) for i in range(batch)])
-    bs = torch.stack([g.preshuffle_b_device(dev(b[i])) for i in range(batch)])
-    args, c = g.api._args_from_tensors(dev(a), bs, da, db, mode, None, g.FP32, 1, n=n)
+    if rowmajor:                                            # a8w8_gemm on row-major weights takes the flat kernel too
+        bs = dev(b)
+        args, c = g.api._args_from_tensors(dev(a), bs, da, db, mode, None, g.FP32, 0)
+        entry = g.lib().a8w8_gemm
+    else:
+        bs = torch.stack([g.preshuffle_b_device(dev(b[i])) for i in range(batch)])
+        args, c = g.api._args_from_tensors(dev(a), bs, da, db, mode, None, g.FP32, 1, n=n)
+        entry = g.lib().a8w8_flatmm
     assert (args.stride_sfa_batch, args.stride_sfb_batch) == (da[0].numel(), db[0].numel())      # scales of their own per entry
     assert g.kernel_name(args) == "flatmm_a8w8"
-    assert g.lib().a8w8_flatmm(ctypes.byref(args), g.api._stream()) == 0
+    assert entry(ctypes.byref(args), g.api._stream()) == 0
     torch.cuda.synchronize()
     want = np.einsum("bmk,bnk->bmn", A, B).astype(np.float32)
     bad = np.argwhere(c.cpu().numpy() != want)
@@ -180,3 +186,14 @@ def test_row_groups_four_weight_tiles(orc, mode, m):
     n, k = (288, 192) if mode in (g.ROWCOL, g.TENSOR) else (384, 256)
     batch = (1024 * 16 + n - 1) // n
     _row_group_case(orc, mode, m, n, k, batch, 8600 + m)
+
+
+@pytest.mark.parametrize("m", [1, 16, 17, 48, 64, 65, 96, 128])
+@pytest.mark.parametrize("mode", [g.ROWCOL, g.TENSOR, g.MX_TILED, g.BLOCK])
+@pytest.mark.parametrize("many_tiles", [False, True])
+def test_row_major_weights_on_the_flat_kernel(orc, mode, m, many_tiles):
+    """a8w8_gemm with row-major B and at most 128 rows: the flat kernel stages the weight rows through LDS.  Two or
+    four weight tiles per workgroup, every count of row groups, ragged tile counts, an odd number of K blocks."""
+    n, k = (144, 320) if mode in (g.ROWCOL, g.TENSOR) else (384, 256)
+    batch = (1024 * 16 + n - 1) // n if many_tiles else 2
+    _row_group_case(orc, mode, m, n, k, batch, 8800 + m, rowmajor=True)

@@ -56,12 +56,14 @@ def test_quantize_writes_the_tiled_layout(orc, rows, k):
 @pytest.mark.parametrize("shape", [(256, 256, 256), (512, 256, 1024), (130, 270, 768), (256, 512, 2048), (64, 64, 512),
                                    (70, 40, 384), (64, 64, 128), (2304, 2048, 256), (1300, 4000, 512), (2100, 2300, 384), (2304, 4096, 256), (2100, 4500, 384)])
 def test_gemm_with_tiled_scales(orc, shape):
-    """At most 512 tiles of 128 x 128, or an odd number of K steps: the 128-tile kernel; otherwise the four-wave kernel."""
+    """Up to 128 rows: the flat kernel.  At most 512 tiles of 128 x 128, or an odd number of K steps: the 128-tile kernel;
+    otherwise the four-wave kernel."""
     m, n, k = shape
     a, b, ea, eb = datagen.mx(m, n, k, seed=1500 + m + k)
     args = g.raw_gemm_args(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, m, n, k, g.MX_TILED)
     workgroups128 = -(-m // 128) * -(-n // 128)
-    assert g.kernel_name(args) == ("gemm_a8w8_wide" if workgroups128 > 512 and k % 256 == 0 else "gemm_a8w8_tile128")
+    flat = m <= 128 and n % 16 == 0 and k % 64 == 0          # skinny: the flat kernel, also on row-major weights
+    assert g.kernel_name(args) == ("flatmm_a8w8" if flat else "gemm_a8w8_wide" if workgroups128 > 512 and k % 256 == 0 else "gemm_a8w8_tile128")
     want = orc.gemm_ref(a, b, ea, eb, orc.MX)
     exact, mag = exact64(orc, a, b, ea, eb, g.MX)
     assert_close(_tiled_gemm(a, b, ea, eb), want, f"mx tiled {shape}", exact=exact, mag=mag)
