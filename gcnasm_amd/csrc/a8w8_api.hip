@@ -415,11 +415,11 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 //   28672 x 4096   FP8 21 / 23 / 26 / 28 against 26-27, MXFP8 22 / 25 / 28 / 40 against 26-28,
 //                  MXFP4 13 / 16 / 17 / 25 against 15-16, bf16 43 / 43 / 48 / 52 against 47-48
 // The model takes the faster side in these except where the two are within ~8% of each other.
-// Row-major weights (a8w8_gemm without b_preshuffled; the flat kernel stages the weight rows through LDS): ~1.3x the
-// shuffled flat times -- 16384 x 7168 FP8 25 / 27 / 31 / 55, 8192 x 8192 20 / 20 / 22 / 37, 28672 x 4096 27 / 31 / - / -.
-// 64 < M <= 128 (two flat passes, FP8, M = 80 / 96 / 128): 16384 x 7168 flat 42 / 40 / 41 against 41 / 43 / 47,
-// 8192 x 8192 flat 29 / 29 / 30 (20 / 22 / 25 in one pass on two weight tiles, which is what runs there) against 42 / 43 / 45, 28672 x 4096 flat 46 / 46 / 48 against 28 / 29 / 31.
-bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, bool rowmajor = false)
+// Row-major weights (a8w8_gemm without b_preshuffled; the flat kernel stages the weight rows through LDS, whole lines
+// per load): as fast as shuffled ones unless the rows are a large power of two apart, where the 16 rows of a tile fall
+// on the same memory channels -- 16384 x 7168 FP8 M = 16 / 32 / 64: 20 / 21 / 25 us, 8192 x 8192: 19 / 20 / 21 us
+// (13 / 14 / 18 shuffled).
+bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, double layout_factor = 1.0)
 {
     const double w = (double)n * (double)row_bytes;
     if (w <= (double)(32ll << 20)) return true;
@@ -435,7 +435,7 @@ bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, bool ro
         if (mt == 4 && scaled_in_loop) flat *= 1.3;
         if (passes == 2) flat *= 1.55;      // the second pass reads the weights from L2
     }
-    if (rowmajor) flat *= 1.3;      // weight rows staged through LDS, two half-line reads per row and pair
+    flat *= layout_factor;      // row-major weights: rows staged through LDS, rows a power of two apart share channels
     double dense = 4.0 + std::max(rounds * 128.0 * (double)row_bytes / 28.0e3, w / 5.0e6);
     if (m > 64) dense *= 1.0 + 0.25 * (m - 64) / 64.0;
     return flat <= dense;
@@ -444,7 +444,8 @@ bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, bool ro
 bool prefer_flat_fp8(const a8w8_gemm_args* g)
 {
     const bool scaled_in_loop = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED || g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128;
-    return prefer_flat(g->m, g->n, g->k, scaled_in_loop, !g->b_preshuffled);
+    const double layout_factor = g->b_preshuffled ? 1.0 : g->stride_b % 4096 == 0 ? 1.4 : 1.05;
+    return prefer_flat(g->m, g->n, g->k, scaled_in_loop, layout_factor);
 }
 
 template <bool BROW>

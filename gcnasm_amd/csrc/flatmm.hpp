@@ -61,7 +61,7 @@ constexpr int FLAT_STAGE_SLOTS = 8 * 18;
 // MT groups of 16 activation rows per workgroup share one pass over the weights.  With MT = 1 a lane gathers its
 // MFMA fragment straight from memory (16 bytes of one row per lane: 16 cache lines per quarter wave, affordable
 // once per pair of K blocks).  With MT > 1 that gather would cost more than the weight stream, so the wave reads
-// the rows the coalesced way (four lanes per 128-byte line) and turns them into fragments through a private
+// the rows the coalesced way (eight lanes per 128-byte line) and turns them into fragments through a private
 // piece of LDS; nothing is shared between waves, so the K loop still has no barrier.
 //
 // BROW: the weights are row-major ([n][ldb], not pre-shuffled).  Their 16-row tiles then take the road of the
@@ -122,8 +122,10 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 
     // MT = 1: lane (r16, kq) reads bytes [16 kq, 16 kq + 16) of row r16 in each K block.
     // MT > 1: lane (row = lane / 4, c = lane % 4) reads bytes [32 c, 32 c + 32) of the pair's 128-byte line.
-    const int ld_row = MT == 1 ? r16 : lane >> 2;
-    const int ld_c = lane & 3;
+    // Staged rows (A for MT > 1, row-major B): lane (row = lane / 8, piece = lane % 8) reads 16-byte piece `piece` of
+    // the pair's 128-byte line of row `row`, and of row + 8 with a second load: eight whole lines per instruction.
+    const int ld_row = lane >> 3;
+    const int ld_piece = lane & 7;
     // addresses are a wave-uniform base plus a 32-bit lane offset (operand extents are below 2 GiB): one register
     // per row group and weight tile instead of a 64-bit pointer each
     // (buffer loads: descriptor + 32-bit lane offset + scalar offset, so no load needs a 64-bit address in registers)
@@ -131,9 +133,11 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     uint32_t a_off[MT];
 #pragma unroll
     for (int g = 0; g < MT; ++g)
-        a_off[g] = (uint32_t)min(m0 + g * 16 + ld_row, p.m - 1) * (uint32_t)p.lda + (MT == 1 ? kq * 16 : ld_c * 32);
+        a_off[g] = MT == 1 ? (uint32_t)min(m0 + r16, p.m - 1) * (uint32_t)p.lda + kq * 16
+                           // rows past m lie beyond the descriptor's extent and read as zero: no clamp
+                           : (uint32_t)(m0 + g * 16 + ld_row) * (uint32_t)p.lda + ld_piece * 16;
     v4i* stage = smem + wave * (STAGED * FLAT_STAGE_SLOTS);
-    const int st_write = (2 * ld_c) * 18 + (lane >> 2);  // piece 2c of row lane / 4, the next piece is 18 slots on
+    const int st_write = ld_piece * 18 + ld_row;         // row + 8 is 8 slots on
     const int st_read = kq * 18 + r16;                   // piece kq, the second K block's is 4 * 18 slots on
 
     const auto rs_b = make_rsrc(p.b + (long long)batch * p.b_batch, BROW ? (uint32_t)(p.n - 1) * (uint32_t)p.ldb + (uint32_t)p.k
@@ -143,7 +147,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         if constexpr (BROW)
-            b_off[t] = (uint32_t)min((nt0 + t) * 16 + (lane >> 2), p.n - 1) * (uint32_t)p.ldb + ld_c * 32;
+            b_off[t] = (uint32_t)((nt0 + t) * 16 + ld_row) * (uint32_t)p.ldb + ld_piece * 16;      // rows past n read as zero
         else
             b_off[t] = (uint32_t)min(nt0 + t, n_tiles - 1) * (uint32_t)k_tiles * 1024u;
     }
@@ -206,20 +210,20 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     v4i raw[MT][2];
     v4i raw_b[NT][2];          // BROW: the same for the rows of the weight tiles
     auto load_rows = [&](int pp) {
-        // lanes c = 2, 3 hold the second K block of the pair
-        const bool there = 2 * pp + 1 < k_tiles || ld_c < 2;
+        // pieces 4 .. 7 are the second K block of the pair
+        const bool there = 2 * pp + 1 < k_tiles || ld_piece < 4;
 #pragma unroll
         for (int g = 0; g < MT; ++g) {
             raw[g][0] = there ? ld16(rs_a, a_off[g], pp * 128) : v4i{0, 0, 0, 0};
-            raw[g][1] = there ? ld16(rs_a, a_off[g], pp * 128 + 16) : v4i{0, 0, 0, 0};
+            raw[g][1] = there ? ld16(rs_a, a_off[g], pp * 128 + 8 * p.lda) : v4i{0, 0, 0, 0};
         }
     };
     auto load_weight_rows = [&](int pp) {
-        const bool there = 2 * pp + 1 < k_tiles || ld_c < 2;
+        const bool there = 2 * pp + 1 < k_tiles || ld_piece < 4;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             raw_b[t][0] = there ? ld16_nt(rs_b, b_off[t], pp * 128) : v4i{0, 0, 0, 0};
-            raw_b[t][1] = there ? ld16_nt(rs_b, b_off[t], pp * 128 + 16) : v4i{0, 0, 0, 0};
+            raw_b[t][1] = there ? ld16_nt(rs_b, b_off[t], pp * 128 + 8 * p.ldb) : v4i{0, 0, 0, 0};
         }
     };
     // rows -> this wave's own LDS.  A wave's LDS operations complete in order, so the fragment reads that follow
@@ -230,13 +234,13 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 #pragma unroll
         for (int g = 0; g < A_GROUPS; ++g) {
             stage[g * FLAT_STAGE_SLOTS + st_write] = raw[g][0];
-            stage[g * FLAT_STAGE_SLOTS + st_write + 18] = raw[g][1];
+            stage[g * FLAT_STAGE_SLOTS + st_write + 8] = raw[g][1];
         }
         if constexpr (BROW) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 stage[(A_GROUPS + t) * FLAT_STAGE_SLOTS + st_write] = raw_b[t][0];
-                stage[(A_GROUPS + t) * FLAT_STAGE_SLOTS + st_write + 18] = raw_b[t][1];
+                stage[(A_GROUPS + t) * FLAT_STAGE_SLOTS + st_write + 8] = raw_b[t][1];
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -83,7 +83,7 @@ def test_gemm_on_shuffled_weights_preconditions():
     # row-major weights, at most 128 rows: the flat kernel where it can run and the model calls it faster
     rm = dict(mode=g.ROWCOL, n=16384, k=7168)
     assert g.kernel_name(_ok_args(m=64, **rm)) == "flatmm_a8w8"
-    assert g.kernel_name(_ok_args(m=128, **rm)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(m=128, mode=g.ROWCOL, n=16384, k=8192)) == "gemm_a8w8_tile128"       # two passes, rows 8192 apart
     assert g.kernel_name(_ok_args(m=129, **rm)) == "gemm_a8w8_tile128"
     assert g.kernel_name(_ok_args(m=64, mode=g.ROWCOL, n=16384 + 8, k=7168)) == "gemm_a8w8_tile128"      # n % 16 != 0
     assert g.kernel_name(_ok_args(m=16, mode=g.MX, n=4096, k=4096)) == "gemm_a8w8_tile128"              # row-major MX scales
