@@ -417,7 +417,7 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 // The model takes the faster side in these except where the two are within ~8% of each other.
 // Row-major weights (a8w8_gemm without b_preshuffled; the flat kernel stages the weight rows through LDS, whole lines
 // per load): as fast as shuffled ones unless the rows are a large power of two apart, where the 16 rows of a tile fall
-// on the same memory channels -- 16384 x 7168 FP8 M = 16 / 32 / 64: 20 / 21 / 25 us, 8192 x 8192: 19 / 20 / 21 us
+// on the same memory channels -- 16384 x 7168 FP8 M = 16 / 32 / 64: 20 / 21 / 25 us, 8192 x 8192: 17 / 17 / 20 us
 // (13 / 14 / 18 shuffled).
 bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, double layout_factor = 1.0)
 {
@@ -444,7 +444,7 @@ bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, double 
 bool prefer_flat_fp8(const a8w8_gemm_args* g)
 {
     const bool scaled_in_loop = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED || g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128;
-    const double layout_factor = g->b_preshuffled ? 1.0 : g->stride_b % 4096 == 0 ? 1.4 : 1.05;
+    const double layout_factor = g->b_preshuffled ? 1.0 : g->stride_b % 4096 == 0 ? 1.3 : 1.05;
     return prefer_flat(g->m, g->n, g->k, scaled_in_loop, layout_factor);
 }
 

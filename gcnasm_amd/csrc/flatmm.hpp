@@ -338,30 +338,39 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 
     if (wave < pairs) {
         Frag f0, f1;
-        int pp = wave;
         constexpr bool STAGING = MT > 1 || BROW;
         auto load_staged = [&](int q) {
             if constexpr (MT > 1) load_rows(q);
             if constexpr (BROW) load_weight_rows(q);
         };
-        load_staged(pp);
-        load(pp, f0);
+        // This wave's pairs are wave, wave + 8, ...; it starts at one that depends on the workgroup and wraps around,
+        // so that workgroups running side by side are at different K offsets: with rows (or weight tiles) a power of
+        // two apart they would otherwise all sit on the same memory channels at any moment.
+        const int count = (pairs - wave + PSTEP - 1) / PSTEP;
+        // (the same for the workgroups of one group of weight tiles: those read the weights together, through L2)
+        int at = (n_group * 5) % count;
+        auto next_of = [&](int j) { return j + 1 == count ? 0 : j + 1; };
+        int left = count;
+        load_staged(wave + PSTEP * at);
+        load(wave + PSTEP * at, f0);
         // two register stages, loads of the next pair in flight while the current one is used
         while (true) {
             if constexpr (STAGING) stage_rows();
-            if (pp + PSTEP < pairs) {
-                load_staged(pp + PSTEP);
-                load(pp + PSTEP, f1);
+            at = next_of(at);
+            if (left > 1) {
+                load_staged(wave + PSTEP * at);
+                load(wave + PSTEP * at, f1);
             }
             mma(f0);
-            if ((pp += PSTEP) >= pairs) break;
+            if (--left == 0) break;
             if constexpr (STAGING) stage_rows();
-            if (pp + PSTEP < pairs) {
-                load_staged(pp + PSTEP);
-                load(pp + PSTEP, f0);
+            at = next_of(at);
+            if (left > 1) {
+                load_staged(wave + PSTEP * at);
+                load(wave + PSTEP * at, f0);
             }
             mma(f1);
-            if ((pp += PSTEP) >= pairs) break;
+            if (--left == 0) break;
         }
     }
 
