@@ -539,6 +539,13 @@ static int a16w16_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     bytes.stride_a_batch = g->stride_a_batch * 2; bytes.stride_b_batch = g->stride_b_batch * 2;
     bytes.scale_mode = A8W8_SCALE_TENSOR;
     const bool fits = (long long)g->stride_a_batch * 2 < (1ll << 31) && (long long)g->stride_b_batch * 2 < (1ll << 31);
+    // a skinny problem on row-major weights: the flat kernel (weight rows staged through LDS) where it is the faster one
+    if (fits && flat_rowmajor_ok(&bytes) && prefer_flat(g->m, g->n, bytes.k, false, bytes.stride_b % 4096 == 0 ? 1.3 : 1.05)) {
+        GemmParams p = make_params(&bytes);
+        p.sfa = p.sfb = nullptr;
+        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_BF16, true>(p, g->batch, s)
+                                         : launch_flat<C_FP32, MODE_BF16, true>(p, g->batch, s);
+    }
     // weights shuffled as bytes (a16w16_flatmm's): MFMA kernels only
     if (g->b_preshuffled && (validate_shuffled_b(&bytes) != A8W8_OK || !fits || !persist_ok(&bytes))) return A8W8_ERR_BAD_GROUP;
     if (fits && tiled_ok(&bytes) && persist_ok(&bytes)) {
@@ -600,6 +607,12 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
     bytes.stride_a = g->stride_a / 2; bytes.stride_b = g->b_preshuffled ? bytes.k : g->stride_b / 2;
     bytes.stride_a_batch = g->stride_a_batch / 2; bytes.stride_b_batch = g->stride_b_batch / 2;
     bytes.scale_mode = A8W8_SCALE_MX_E8M0_TILED;
+    // a skinny problem on row-major weights: the flat kernel where it is the faster one
+    if (tiled && flat_rowmajor_ok(&bytes) && prefer_flat(g->m, g->n, bytes.k, true, bytes.stride_b % 4096 == 0 ? 1.3 : 1.05)) {
+        const GemmParams p = make_params(&bytes);
+        return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_F4T, true>(p, g->batch, s)
+                                         : launch_flat<C_FP32, MODE_F4T, true>(p, g->batch, s);
+    }
     // weights shuffled as bytes (a4w4_flatmm's): MFMA kernels only
     if (g->b_preshuffled && (!tiled || g->k % 256 != 0 || validate_shuffled_b(&bytes) != A8W8_OK ||
                              (!small_ok(&bytes) && !persist_ok(&bytes))))

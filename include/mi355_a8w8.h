@@ -95,7 +95,7 @@ typedef struct {
  * a16w16_gemm and a4w4_gemm accept it likewise for the weights their flat siblings stream (shuffled as bytes).
  * Skinny problems (m <= 128, n % 16 == 0, k % 64 == 0, 16-byte aligned rows; per-tensor, row/column, block or
  * tiled MX scales) run on the flat kernel of a8w8_flatmm where that is the faster one, on shuffled and on
- * row-major weights alike. */
+ * row-major weights alike (a16w16_gemm and a4w4_gemm with tiled scales likewise). */
 A8W8_API int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream);
 
 /* The bf16 sibling (gemm_a16w16_8wave, the program opus_gemm/rebuild.sh:3-13 builds; its source is

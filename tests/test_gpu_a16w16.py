@@ -111,3 +111,18 @@ def test_flat_gemm_row_groups_exact(m, n, batch):
     bs = torch.stack([g.preshuffle_b_bf16_device(b[i]) for i in range(batch)])
     got = g.flatmm_a16w16(a, bs, n, c_dtype=g.FP32)
     assert torch.equal(got, torch.einsum("bmk,bnk->bmn", a.float(), b.float()))
+
+
+@pytest.mark.parametrize("m", [1, 16, 40, 64, 100, 128])
+@pytest.mark.parametrize("n,batch", [(144, 2), (288, 57)])
+def test_skinny_gemm_on_row_major_weights_exact(m, n, batch):
+    """a16w16_gemm with at most 128 rows on row-major weights runs the flat kernel (weight rows staged through LDS)."""
+    k = 160
+    gen = torch.Generator(device="cuda"); gen.manual_seed(950 + m + n)
+    a = torch.randint(-4, 5, (batch, m, k), generator=gen, device="cuda").to(torch.bfloat16)
+    b = torch.randint(-4, 5, (batch, n, k), generator=gen, device="cuda").to(torch.bfloat16)
+    got = g.gemm_a16w16(a, b, c_dtype=g.FP32)
+    assert torch.equal(got, torch.einsum("bmk,bnk->bmn", a.float(), b.float()))
+    # the same bits as the flat entry point on shuffled weights
+    bs = torch.stack([g.preshuffle_b_bf16_device(b[i]) for i in range(batch)])
+    assert torch.equal(got, g.flatmm_a16w16(a, bs, n, c_dtype=g.FP32))

@@ -162,6 +162,26 @@ def test_flat_row_groups_four_weight_tiles(orc, m):
     assert bad.size == 0, f"{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
 
 
+@pytest.mark.parametrize("m", [1, 16, 33, 64, 100, 128])
+@pytest.mark.parametrize("n", [144, 16400])
+def test_skinny_gemm_on_row_major_weights(orc, m, n):
+    """a4w4_gemm with at most 128 rows on row-major packed weights runs the flat kernel: exact, and the same bits
+    as a4w4_flatmm on the shuffled weights."""
+    r = np.random.default_rng(8900 + m + n)
+    k = 384
+    qa = r.integers(0, 256, (m, k // 2)).astype(np.uint8)
+    qb = r.integers(0, 256, (n, k // 2)).astype(np.uint8)
+    ea = r.integers(126, 129, (m, k // 32)).astype(np.uint8)
+    eb = r.integers(126, 129, (n, k // 32)).astype(np.uint8)
+    exact, _ = _exact(orc, qa, qb, ea, eb)
+    ta, tb = g.mx_tile_scales(dev(ea)), g.mx_tile_scales(dev(eb))
+    got = g.gemm_a4w4(dev(qa), dev(qb), ta, tb, c_dtype=g.FP32)
+    torch.cuda.synchronize()
+    bad = np.argwhere(got.cpu().numpy() != exact.astype(np.float32))
+    assert bad.size == 0, f"{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
+    assert torch.equal(got, g.flatmm_a4w4(dev(qa), g.preshuffle_b_device(dev(qb)), ta, tb, n, c_dtype=g.FP32))
+
+
 def test_flat_rejects_what_it_cannot_run():
     qa = torch.zeros((16, 64), dtype=torch.uint8, device="cuda")
     bs = torch.zeros(16 * 64, dtype=torch.uint8, device="cuda")
