@@ -382,8 +382,8 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
             return launch_flat_nt<2, 8, CDT, MODE, BROW>(p, batch, stream);
     }
     if (mt == 4) {
-        // four weight tiles x four row groups fill the register file; MX or block scales on top would spill
-        if constexpr (MODE != MODE_BLOCK && MODE != MODE_MXT && MODE != MODE_F4T) {
+        // four weight tiles x four row groups fill the register file; MX scales on top would spill
+        if constexpr (MODE != MODE_MXT && MODE != MODE_F4T) {
             if (tiles >= 4ll * cus) return launch_flat_nt<4, 4, CDT, MODE, BROW>(p, batch, stream);
         }
         return launch_flat_nt<2, 4, CDT, MODE, BROW>(p, batch, stream);
@@ -404,7 +404,7 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 // On shuffled weights both the flat GEMM and the MFMA kernels can run a skinny problem; the entry points take the
 // one a small cost model calls faster.  Times in microseconds, W = weight bytes, row_bytes = bytes of one weight row:
 //   flat:  one pass over the weights at ~6.3 TB/s; every further group of 16 activation rows adds ~2 us of
-//          activation traffic and MFMA work.  With MX or block scales, four groups only fit the registers with two
+//          activation traffic and MFMA work.  With MX scales, four groups only fit the registers with two
 //          weight tiles per workgroup, which costs another ~30%.
 //   dense: the 128-tile kernel has only n/128 workgroups to pull the weights with, ~28 GB/s each (128 rows a
 //          workgroup), and ~5 TB/s at best over the chip.
@@ -443,7 +443,7 @@ bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, double 
 
 bool prefer_flat_fp8(const a8w8_gemm_args* g)
 {
-    const bool scaled_in_loop = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED || g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128;
+    const bool scaled_in_loop = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;      // four row groups: two weight tiles per workgroup
     const double layout_factor = g->b_preshuffled ? 1.0 : g->stride_b % 4096 == 0 ? 1.3 : 1.05;
     return prefer_flat(g->m, g->n, g->k, scaled_in_loop, layout_factor);
 }

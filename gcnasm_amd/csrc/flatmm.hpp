@@ -157,6 +157,8 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     // with, for row 16 i + r16 of a 64-row block, x = (2 i + r16 / 8) % 4, y = r16 % 4, jp = i / 2, par = (r16 / 4) % 2
     const auto rs_sa = make_rsrc((const uint8_t*)p.sfa + (long long)batch * p.sfa_batch, 0x7fffffffu);
     const auto rs_sb = make_rsrc((const uint8_t*)p.sfb + (long long)batch * p.sfb_batch, 0x7fffffffu);
+    // offsets of row groups / weight tiles 1, 2, 3 of a 64-row block from group 0's, for a lane (see lane_off below)
+    constexpr uint32_t MX_DELTA[4] = {0u, 256u, 4u, 260u};
     uint32_t mx_a[MT], mx_b[NT];
     int mx_nblk_a = 1, mx_nblk_b = 1;
     if constexpr (MODE == MODE_MXT || MODE == MODE_F4T) {
@@ -166,26 +168,28 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 #pragma unroll
         for (int g = 0; g < MT; ++g) {
             const int mt = min(m_tile_ * MT + g, ((p.m + 15) >> 4) - 1);
-            mx_a[g] = (uint32_t)(mt >> 2) * 1024u + lane_off(mt & 3);
+            // four groups are one 64-row block: constant distances from group 0 (rows past m stay inside the block)
+            mx_a[g] = MT == 4 ? (uint32_t)m_tile_ * 1024u + lane_off(0) + MX_DELTA[g & 3] : (uint32_t)(mt >> 2) * 1024u + lane_off(mt & 3);
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const int nt = min(nt0 + t, n_tiles - 1);
-            mx_b[t] = (uint32_t)(nt >> 2) * 1024u + lane_off(nt & 3);
+            mx_b[t] = NT == 4 ? (uint32_t)n_group * 1024u + lane_off(0) + MX_DELTA[t & 3] : (uint32_t)(nt >> 2) * 1024u + lane_off(nt & 3);
         }
     }
 
     // block scales (1x128 for A, 128x128 for B; the reference's layout): a pair of K blocks is one 128-wide scale
     // group, lane (r16, .) needs sfa[group][its row] and, per weight tile, sfb[tile's 128-row block][group]
-    const float* blk_a[MT];
-    const float* blk_b[NT];
+    uint32_t blk_a_off = 0;
+    const auto rs_blk_a = make_rsrc((const float*)p.sfa + (long long)batch * p.sfa_batch,
+                                    MODE == MODE_BLOCK ? ((uint32_t)(p.k / 128 - 1) * (uint32_t)p.stride_sfa + (uint32_t)p.m) * 4u : 0u);
+    const float* blk_b;      // NT divides 8 and the tile groups start at multiples of NT: one 128-row block per workgroup
     if constexpr (MODE == MODE_BLOCK) {
-#pragma unroll
-        for (int g = 0; g < MT; ++g)
-            blk_a[g] = (const float*)p.sfa + (long long)batch * p.sfa_batch + min(m0 + g * 16 + r16, p.m - 1);
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-            blk_b[t] = (const float*)p.sfb + (long long)batch * p.sfb_batch + (long long)(min(nt0 + t, n_tiles - 1) >> 3) * p.stride_sfb;
+        // sfa[group][row] through a descriptor over the whole array: one lane offset (the row), the row groups 64 bytes
+        // apart, the K group scalar; rows past m read a neighbour's scale or zero and feed rows that are not stored
+        blk_a_off = (uint32_t)(m0 + r16) * 4u;
+        static_assert(MODE != MODE_BLOCK || 8 % NT == 0, "the weight tiles of a workgroup share their block scale");
+        blk_b = (const float*)p.sfb + (long long)batch * p.sfb_batch + (long long)(nt0 >> 3) * p.stride_sfb;
     }
 
     // K blocks are consumed in pairs; wave w takes pairs w, w + 8, ...: at any moment the eight waves read 16 KiB in
@@ -204,7 +208,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         v4i a[2];               // MT = 1: the activation fragment itself
         v4i b[NT][2];
         int sa[MT], sb[NT];     // MX: the step's E8M0 byte of this lane's row and 32-block
-        float fsa[MT], fsb[NT]; // block scales of the pair's scale group
+        float fsa[MT], fsb;     // block scales of the pair's scale group
     };
     // MT > 1: the rows of one pair in flight (one register set: a pair's rows go to LDS before the next is asked for)
     v4i raw[MT][2];
@@ -214,16 +218,18 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         const bool there = 2 * pp + 1 < k_tiles || ld_piece < 4;
 #pragma unroll
         for (int g = 0; g < MT; ++g) {
-            raw[g][0] = there ? ld16(rs_a, a_off[g], pp * 128) : v4i{0, 0, 0, 0};
-            raw[g][1] = there ? ld16(rs_a, a_off[g], pp * 128 + 8 * p.lda) : v4i{0, 0, 0, 0};
+            // (group g is 16 g rows on: a scalar offset, so that one lane offset serves every group)
+            raw[g][0] = there ? ld16(rs_a, a_off[0], pp * 128 + 16 * g * p.lda) : v4i{0, 0, 0, 0};
+            raw[g][1] = there ? ld16(rs_a, a_off[0], pp * 128 + (16 * g + 8) * p.lda) : v4i{0, 0, 0, 0};
         }
     };
     auto load_weight_rows = [&](int pp) {
         const bool there = 2 * pp + 1 < k_tiles || ld_piece < 4;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            raw_b[t][0] = there ? ld16_nt(rs_b, b_off[t], pp * 128) : v4i{0, 0, 0, 0};
-            raw_b[t][1] = there ? ld16_nt(rs_b, b_off[t], pp * 128 + 8 * p.ldb) : v4i{0, 0, 0, 0};
+            // (tile t is 16 t rows on: a scalar offset, one lane offset for every tile)
+            raw_b[t][0] = there ? ld16_nt(rs_b, b_off[0], pp * 128 + 16 * t * p.ldb) : v4i{0, 0, 0, 0};
+            raw_b[t][1] = there ? ld16_nt(rs_b, b_off[0], pp * 128 + (16 * t + 8) * p.ldb) : v4i{0, 0, 0, 0};
         }
     };
     // rows -> this wave's own LDS.  A wave's LDS operations complete in order, so the fragment reads that follow
@@ -270,7 +276,9 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         }
         if constexpr (MODE == MODE_BLOCK) {
 #pragma unroll
-            for (int g = 0; g < MT; ++g) f.fsa[g] = blk_a[g][(long long)pp * p.stride_sfa];
+            for (int g = 0; g < MT; ++g)
+                f.fsa[g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_blk_a, blk_a_off + 64u * g, pp * p.stride_sfa * 4, 0));
+            f.fsb = blk_b[pp];
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
@@ -280,7 +288,6 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
             }
             if constexpr (MODE == MODE_MXT) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b8(rs_sb, mx_b[t], unit_b, 0);
             if constexpr (MODE == MODE_F4T) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b16(rs_sb, mx_b[t], unit_b, 0);
-            if constexpr (MODE == MODE_BLOCK) f.fsb[t] = blk_b[t][pp];
         }
     };
     auto mma = [&](const Frag& f) {
@@ -318,7 +325,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
                 } else if constexpr (MODE == MODE_BLOCK) {
                     // each 128-wide K group yields a partial tile that is rescaled into the running sum
                     const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                    acc[g][t] += part * (f.fsa[g] * f.fsb[t]);
+                    acc[g][t] += part * (f.fsa[g] * f.fsb);
                 } else if constexpr (MODE == MODE_F4T) {
                     // packed E2M1: a 64-byte block is 128 elements, one FP4 MFMA; op_sel picks the block's scale byte
                     acc[g][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
