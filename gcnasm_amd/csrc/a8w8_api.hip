@@ -382,8 +382,8 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
             return launch_flat_nt<2, 8, CDT, MODE, BROW>(p, batch, stream);
     }
     if (mt == 4) {
-        // four weight tiles x four row groups fill the register file; MX scales on top would spill
-        if constexpr (MODE != MODE_MXT && MODE != MODE_F4T) {
+        // four weight tiles x four row groups fill the register file; the scale bytes of MXFP8 on top would spill
+        if constexpr (MODE != MODE_MXT) {
             if (tiles >= 4ll * cus) return launch_flat_nt<4, 4, CDT, MODE, BROW>(p, batch, stream);
         }
         return launch_flat_nt<2, 4, CDT, MODE, BROW>(p, batch, stream);
@@ -404,7 +404,7 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 // On shuffled weights both the flat GEMM and the MFMA kernels can run a skinny problem; the entry points take the
 // one a small cost model calls faster.  Times in microseconds, W = weight bytes, row_bytes = bytes of one weight row:
 //   flat:  one pass over the weights at ~6.3 TB/s; every further group of 16 activation rows adds ~2 us of
-//          activation traffic and MFMA work.  With MX scales, four groups only fit the registers with two
+//          activation traffic and MFMA work.  With the scale bytes of MXFP8, four groups only fit the registers with two
 //          weight tiles per workgroup, which costs another ~30%.
 //   dense: the 128-tile kernel has only n/128 workgroups to pull the weights with, ~28 GB/s each (128 rows a
 //          workgroup), and ~5 TB/s at best over the chip.
@@ -580,7 +580,7 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
 {
     if (!g) return A8W8_ERR_NULL_POINTER;
     // a skinny problem on shuffled weights: the flat kernel where it is the faster one (and can run it)
-    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= FLAT_MAX_M && prefer_flat(g->m, g->n, g->k / 2, true) &&
+    if (allow_flat && g->b_preshuffled && g->m > 0 && g->m <= FLAT_MAX_M && prefer_flat(g->m, g->n, g->k / 2, false) &&
         a4w4_flat_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     if (!g->a || !g->b || !g->c || !g->sfa || !g->sfb) return A8W8_ERR_NULL_POINTER;
@@ -608,7 +608,7 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
     bytes.stride_a_batch = g->stride_a_batch / 2; bytes.stride_b_batch = g->stride_b_batch / 2;
     bytes.scale_mode = A8W8_SCALE_MX_E8M0_TILED;
     // a skinny problem on row-major weights: the flat kernel where it is the faster one
-    if (tiled && flat_rowmajor_ok(&bytes) && prefer_flat(g->m, g->n, bytes.k, true, bytes.stride_b % 4096 == 0 ? 1.3 : 1.05)) {
+    if (tiled && flat_rowmajor_ok(&bytes) && prefer_flat(g->m, g->n, bytes.k, false, bytes.stride_b % 4096 == 0 ? 1.3 : 1.05)) {
         const GemmParams p = make_params(&bytes);
         return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_F4T, true>(p, g->batch, s)
                                          : launch_flat<C_FP32, MODE_F4T, true>(p, g->batch, s);
@@ -661,7 +661,7 @@ static int a4w4_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
     if ((long long)g->n * g->k / 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
     // several groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
-    if (allow_dense && !prefer_flat(g->m, g->n, g->k / 2, true) && a4w4_gemm_impl(g, hip_stream, false) == A8W8_OK)
+    if (allow_dense && !prefer_flat(g->m, g->n, g->k / 2, false) && a4w4_gemm_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
     a8w8_gemm_args bytes = *g;      // packed rows as byte rows of k/2 columns
     bytes.k = g->k / 2;

@@ -137,6 +137,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
                            // rows past m lie beyond the descriptor's extent and read as zero: no clamp
                            : (uint32_t)(m0 + g * 16 + ld_row) * (uint32_t)p.lda + ld_piece * 16;
     v4i* stage = smem + wave * (STAGED * FLAT_STAGE_SLOTS);
+    const uint32_t kill_second = ld_piece >= 4 ? 0x80000000u : 0u;
     const int st_write = ld_piece * 18 + ld_row;         // row + 8 is 8 slots on
     const int st_read = kq * 18 + r16;                   // piece kq, the second K block's is 4 * 18 slots on
 
@@ -169,12 +170,13 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         for (int g = 0; g < MT; ++g) {
             const int mt = min(m_tile_ * MT + g, ((p.m + 15) >> 4) - 1);
             // four groups are one 64-row block: constant distances from group 0 (rows past m stay inside the block)
-            mx_a[g] = MT == 4 ? (uint32_t)m_tile_ * 1024u + lane_off(0) + MX_DELTA[g & 3] : (uint32_t)(mt >> 2) * 1024u + lane_off(mt & 3);
+            // (the distance goes into the scalar offset of the load: one lane offset for the four groups)
+            mx_a[g] = MT == 4 ? (uint32_t)m_tile_ * 1024u + lane_off(0) : (uint32_t)(mt >> 2) * 1024u + lane_off(mt & 3);
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const int nt = min(nt0 + t, n_tiles - 1);
-            mx_b[t] = NT == 4 ? (uint32_t)n_group * 1024u + lane_off(0) + MX_DELTA[t & 3] : (uint32_t)(nt >> 2) * 1024u + lane_off(nt & 3);
+            mx_b[t] = NT == 4 ? (uint32_t)n_group * 1024u + lane_off(0) : (uint32_t)(nt >> 2) * 1024u + lane_off(nt & 3);
         }
     }
 
@@ -214,22 +216,23 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     v4i raw[MT][2];
     v4i raw_b[NT][2];          // BROW: the same for the rows of the weight tiles
     auto load_rows = [&](int pp) {
-        // pieces 4 .. 7 are the second K block of the pair
-        const bool there = 2 * pp + 1 < k_tiles || ld_piece < 4;
+        // pieces 4 .. 7 are the second K block of the pair: past the end of K (an odd number of blocks) they get an
+        // offset beyond the descriptor's extent instead of a branch, which reads as zero and touches no memory
+        const uint32_t off = a_off[0] | (2 * pp + 1 < k_tiles ? 0u : kill_second);
 #pragma unroll
         for (int g = 0; g < MT; ++g) {
             // (group g is 16 g rows on: a scalar offset, so that one lane offset serves every group)
-            raw[g][0] = there ? ld16(rs_a, a_off[0], pp * 128 + 16 * g * p.lda) : v4i{0, 0, 0, 0};
-            raw[g][1] = there ? ld16(rs_a, a_off[0], pp * 128 + (16 * g + 8) * p.lda) : v4i{0, 0, 0, 0};
+            raw[g][0] = ld16(rs_a, off, pp * 128 + 16 * g * p.lda);
+            raw[g][1] = ld16(rs_a, off, pp * 128 + (16 * g + 8) * p.lda);
         }
     };
     auto load_weight_rows = [&](int pp) {
-        const bool there = 2 * pp + 1 < k_tiles || ld_piece < 4;
+        const uint32_t off = b_off[0] | (2 * pp + 1 < k_tiles ? 0u : kill_second);
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             // (tile t is 16 t rows on: a scalar offset, one lane offset for every tile)
-            raw_b[t][0] = there ? ld16_nt(rs_b, b_off[0], pp * 128 + 16 * t * p.ldb) : v4i{0, 0, 0, 0};
-            raw_b[t][1] = there ? ld16_nt(rs_b, b_off[0], pp * 128 + (16 * t + 8) * p.ldb) : v4i{0, 0, 0, 0};
+            raw_b[t][0] = ld16_nt(rs_b, off, pp * 128 + 16 * t * p.ldb);
+            raw_b[t][1] = ld16_nt(rs_b, off, pp * 128 + (16 * t + 8) * p.ldb);
         }
     };
     // rows -> this wave's own LDS.  A wave's LDS operations complete in order, so the fragment reads that follow
@@ -255,24 +258,24 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     };
     auto load = [&](int pp, Frag& f) {
         const int kt0 = 2 * pp, kt1 = 2 * pp + 1;
-        const bool has1 = kt1 < k_tiles;
+        const uint32_t kill1 = kt1 < k_tiles ? 0u : 0x80000000u;      // reads as zero, see load_rows
         if constexpr (MT == 1) {
             f.a[0] = ld16(rs_a, a_off[0], kt0 * 64);
-            f.a[1] = has1 ? ld16(rs_a, a_off[0], kt1 * 64) : v4i{0, 0, 0, 0};
+            f.a[1] = ld16(rs_a, a_off[0] | kill1, kt1 * 64);
         }
         int unit_a = 0, unit_b = 0;
         if constexpr (MODE == MODE_MXT) {
             unit_a = ((pp >> 2) * mx_nblk_a * 2 + ((pp >> 1) & 1)) * 512 + (pp & 1);
             unit_b = ((pp >> 2) * mx_nblk_b * 2 + ((pp >> 1) & 1)) * 512 + (pp & 1);
 #pragma unroll
-            for (int g = 0; g < MT; ++g) f.sa[g] = __builtin_amdgcn_raw_buffer_load_b8(rs_sa, mx_a[g], unit_a, 0);
+            for (int g = 0; g < MT; ++g) f.sa[g] = __builtin_amdgcn_raw_buffer_load_b8(rs_sa, mx_a[MT == 4 ? 0 : g], unit_a + (MT == 4 ? (int)MX_DELTA[g & 3] : 0), 0);
         }
         if constexpr (MODE == MODE_F4T) {
             // FP4: a pair of 64-byte blocks is two 128-element K steps, whose two scale bytes sit side by side
             unit_a = ((pp >> 1) * mx_nblk_a * 2 + (pp & 1)) * 512;
             unit_b = ((pp >> 1) * mx_nblk_b * 2 + (pp & 1)) * 512;
 #pragma unroll
-            for (int g = 0; g < MT; ++g) f.sa[g] = __builtin_amdgcn_raw_buffer_load_b16(rs_sa, mx_a[g], unit_a, 0);
+            for (int g = 0; g < MT; ++g) f.sa[g] = __builtin_amdgcn_raw_buffer_load_b16(rs_sa, mx_a[MT == 4 ? 0 : g], unit_a + (MT == 4 ? (int)MX_DELTA[g & 3] : 0), 0);
         }
         if constexpr (MODE == MODE_BLOCK) {
 #pragma unroll
@@ -284,10 +287,10 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         for (int t = 0; t < NT; ++t) {
             if constexpr (!BROW) {
                 f.b[t][0] = ld16_nt(rs_b, lane16, b_off[t] + kt0 * 1024);
-                f.b[t][1] = has1 ? ld16_nt(rs_b, lane16, b_off[t] + kt1 * 1024) : v4i{0, 0, 0, 0};
+                f.b[t][1] = ld16_nt(rs_b, lane16 | kill1, b_off[t] + kt1 * 1024);
             }
-            if constexpr (MODE == MODE_MXT) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b8(rs_sb, mx_b[t], unit_b, 0);
-            if constexpr (MODE == MODE_F4T) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b16(rs_sb, mx_b[t], unit_b, 0);
+            if constexpr (MODE == MODE_MXT) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b8(rs_sb, mx_b[NT == 4 ? 0 : t], unit_b + (NT == 4 ? (int)MX_DELTA[t & 3] : 0), 0);
+            if constexpr (MODE == MODE_F4T) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b16(rs_sb, mx_b[NT == 4 ? 0 : t], unit_b + (NT == 4 ? (int)MX_DELTA[t & 3] : 0), 0);
         }
     };
     auto mma = [&](const Frag& f) {
