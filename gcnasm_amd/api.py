@@ -78,9 +78,7 @@ def lib():
         L.a8w8_preshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
         L.a8w8_unshuffle_b.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int]
         L.a8w8_preshuffle_b_device.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, vp]
-        L.a8w8_cvt_f32_to_e4m3.restype = ctypes.c_size_t
         L.a8w8_cvt_f32_to_e4m3.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, vp]
-        L.a8w8_cvt_e4m3_to_f32.restype = ctypes.c_size_t
         L.a8w8_cvt_e4m3_to_f32.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int, vp]
         L.a8w8_quantize.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, ctypes.c_int,
                                     ctypes.c_int, vp]
@@ -99,6 +97,7 @@ def lib():
         L.a8w8_kernel_name.restype = ctypes.c_char_p
         L.a8w8_kernel_name.argtypes = [ctypes.POINTER(GemmArgs)]
         L.a8w8_version.restype = ctypes.c_int
+        L.a8w8_init.argtypes = [ctypes.c_int]
         _lib = L
     return _lib
 
@@ -159,19 +158,64 @@ def _out(c, shape, c_dtype, device):
     return c, (BF16 if c.dtype == torch.bfloat16 else FP32)
 
 
-def _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, b_preshuffled, n=None):
+def _check_operand(t, name, dims):
+    """Operands are strided views of device memory whose rows are contiguous; anything else would be misread."""
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU")
+    if t.dim() not in dims:
+        raise ValueError(f"{name} must have {' or '.join(str(d) for d in dims)} dimensions, got {t.dim()}")
+    if t.dim() >= 1 and t.shape[-1] > 1 and t.stride(-1) != 1:
+        raise ValueError(f"{name}: the last dimension must be contiguous (stride {t.stride(-1)})")
+
+
+def _check_scales(t, name, scale_mode):
+    """Scale arrays are read with the strides their shape implies: they have to be contiguous, on the GPU, and of
+    the element type of the scale mode (fp32, or uint8 for the E8M0 modes)."""
+    import torch
+    want = torch.uint8 if scale_mode in (MX, MX_TILED) else torch.float32
+    if not t.is_cuda or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous GPU tensor")
+    if t.dtype != want:
+        raise TypeError(f"{name} must be {want} for this scale mode, got {t.dtype}")
+
+
+def _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, b_preshuffled, n=None, scaled=True):
+    _check_operand(a, "a", (2, 3))
+    _check_operand(b, "b", (1, 2) if b_preshuffled else (2, 3))
+    if scaled:
+        _check_scales(sfa, "sfa", scale_mode)
+        _check_scales(sfb, "sfb", scale_mode)
     batch = a.shape[0] if a.dim() == 3 else 1
     m, k = a.shape[-2], a.shape[-1]
     if n is None:
         n = b.shape[-2]
     shape = (batch, m, n) if a.dim() == 3 else (m, n)
     c, c_dtype = _out(c, shape, c_dtype, a.device)
+    if c.dim() >= 2 and c.shape[-1] > 1 and c.stride(-1) != 1:
+        raise ValueError("c: the last dimension must be contiguous")
     g = raw_gemm_args(a.data_ptr(), b.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, scale_mode,
                       c_dtype, batch, stride_a=a.stride(-2), stride_b=(k if b_preshuffled else b.stride(-2)),
                       stride_c=c.stride(-2), b_preshuffled=b_preshuffled)
     if a.dim() == 3:
         g.stride_a_batch, g.stride_c_batch = a.stride(0), c.stride(0)
-        g.stride_b_batch = b.stride(0) if b.dim() >= 2 and not b_preshuffled else n * k
+        if b_preshuffled:
+            # flat shuffled weights: of every batch entry back to back, or one matrix shared by all of them
+            per_entry = n * k * a.element_size() // b.element_size()
+            if b.numel() == batch * per_entry:
+                g.stride_b_batch = n * k
+            elif b.numel() == per_entry:
+                g.stride_b_batch = 0
+                g.stride_sfb_batch = 0
+            else:
+                raise ValueError(f"shuffled b holds {b.numel()} elements, expected {per_entry} or {batch} x {per_entry}")
+        elif b.dim() == 3:
+            if b.shape[0] != batch:
+                raise ValueError(f"b has {b.shape[0]} batch entries, a has {batch}")
+            g.stride_b_batch = b.stride(0)
+        else:
+            # one weight matrix shared by every batch entry, and with it one set of weight scales
+            g.stride_b_batch = 0
+            g.stride_sfb_batch = 0
     return g, c
 
 
@@ -186,7 +230,7 @@ def gemm(a, b, sfa, sfb, scale_mode, c=None, c_dtype=BF16, n=None):
 def gemm_a16w16(a, b, c=None, c_dtype=BF16, n=None):
     """C = A @ B^T for bf16 a [.., M, K] and b [.., N, K] (torch.bfloat16 on the GPU) through a16w16_gemm; with `n`
     given, b is the flat pre-shuffled weight of n rows (preshuffle_b_bf16_device)."""
-    g, c = _args_from_tensors(a, b, a, b, TENSOR, c, c_dtype, 0 if n is None else 1, n=n)
+    g, c = _args_from_tensors(a, b, a, b, TENSOR, c, c_dtype, 0 if n is None else 1, n=n, scaled=False)
     _check(lib().a16w16_gemm(ctypes.byref(g), _stream()), "a16w16_gemm")
     return c
 
@@ -200,7 +244,7 @@ def preshuffle_b_bf16_device(b):
 
 def flatmm_a16w16(a, b_shuffled, n, c=None, c_dtype=BF16):
     """Skinny-M bf16 GEMM over weights from preshuffle_b_bf16_device."""
-    g, c = _args_from_tensors(a, b_shuffled, a, a, TENSOR, c, c_dtype, 1, n=n)
+    g, c = _args_from_tensors(a, b_shuffled, a, a, TENSOR, c, c_dtype, 1, n=n, scaled=False)
     _check(lib().a16w16_flatmm(ctypes.byref(g), _stream()), "a16w16_flatmm")
     return c
 
@@ -287,9 +331,8 @@ def cvt_f32_to_e4m3(x, dialect=OCP, clamp240=False):
     import torch
     x = x.contiguous()
     out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
-    done = lib().a8w8_cvt_f32_to_e4m3(x.data_ptr(), out.data_ptr(), x.numel(), dialect, int(clamp240), _stream())
-    if done != x.numel():
-        raise A8W8Error(-6, "a8w8_cvt_f32_to_e4m3")
+    _check(lib().a8w8_cvt_f32_to_e4m3(x.data_ptr(), out.data_ptr(), x.numel(), dialect, int(clamp240), _stream()),
+           "a8w8_cvt_f32_to_e4m3")
     return out
 
 
@@ -297,9 +340,8 @@ def cvt_e4m3_to_f32(codes, dialect=OCP):
     import torch
     codes = codes.contiguous()
     out = torch.empty(codes.shape, dtype=torch.float32, device=codes.device)
-    done = lib().a8w8_cvt_e4m3_to_f32(codes.data_ptr(), out.data_ptr(), codes.numel(), dialect, _stream())
-    if done != codes.numel():
-        raise A8W8Error(-6, "a8w8_cvt_e4m3_to_f32")
+    _check(lib().a8w8_cvt_e4m3_to_f32(codes.data_ptr(), out.data_ptr(), codes.numel(), dialect, _stream()),
+           "a8w8_cvt_e4m3_to_f32")
     return out
 
 
@@ -370,6 +412,11 @@ def load_weights(path):
     _check(lib().a8w8_weights_load(os.fsencode(path), b.ctypes.data, b.nbytes, raw.ctypes.data, raw.nbytes), "a8w8_weights_load")
     scales = raw if h.scale_mode in (MX, MX_TILED) else raw.view(np.float32)
     return h, (b if h.b_preshuffled else b.reshape(h.n, h.k)), scales
+
+
+def init(device=-1):
+    """Explicit one-time set-up of a device (the current one by default); see a8w8_init."""
+    _check(lib().a8w8_init(int(device)), "a8w8_init")
 
 
 def kernel_name(g):

@@ -5,39 +5,108 @@
 #include <stdio.h>
 #include <string.h>
 #include <algorithm>
+#include <mutex>
+#include <tuple>
+#include <utility>
 
 #include "cvt.hpp"
 #include "flatmm.hpp"
 #include "gemm_general.hpp"
 #include "gemm_persist.hpp"
 #include "gemm_small.hpp"
-#include "gemm_tile.hpp"
 #include "gemm_wide.hpp"
 
 using namespace a8w8;
 
 namespace {
 
-int g_num_cus[64];
+// ---------------------------------------------------------------- per-device set-up, done once
+// What a device needs before its first launch: its architecture and compute-unit count, and the
+// dynamic-LDS limit of every kernel instantiation that uses more than the 64 KiB default.  It runs
+// exactly once per device (std::call_once: concurrent first calls from several threads wait for
+// it), either from a8w8_init or from the first entry point called with that device current.
+constexpr int MAX_DEVICES = 64;
+struct DeviceState {
+    std::once_flag once;
+    int status = A8W8_ERR_NO_DEVICE;
+    int num_cus = 0;
+};
+DeviceState g_dev[MAX_DEVICES];
 
-bool device_is_gfx950()
+template <class K>
+bool raise_lds_limit(K kern, int bytes)
 {
-    static int cached[64];   // 0 unknown, 1 yes, -1 no
+    return hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess;
+}
+
+constexpr int persist_lds_bytes(int mode)
+{
+    return mode == MODE_MX ? PERSIST_LDS_BYTES_MX : mode == MODE_ROWCOL ? PERSIST_LDS_BYTES_ROWCOL : PERSIST_LDS_BYTES;
+}
+
+template <int MODE>
+bool raise_lds_limits_of_mode()
+{
+    bool ok = true;
+    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_BF16)
+        ok = ok && raise_lds_limit(gemm_a8w8_persist<MODE, C_BF16>, persist_lds_bytes(MODE)) &&
+             raise_lds_limit(gemm_a8w8_persist<MODE, C_FP32>, persist_lds_bytes(MODE));
+    if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT || MODE == MODE_BF16 || MODE == MODE_F4T)
+        ok = ok && raise_lds_limit(gemm_a8w8_wide<MODE, C_BF16>, wide_lds_bytes(MODE)) &&
+             raise_lds_limit(gemm_a8w8_wide<MODE, C_FP32>, wide_lds_bytes(MODE));
+    if constexpr (MODE != MODE_F4)
+        ok = ok && raise_lds_limit(gemm_a8w8_tile128<MODE, C_BF16, 2>, small_lds_bytes(MODE, 2)) &&
+             raise_lds_limit(gemm_a8w8_tile128<MODE, C_FP32, 2>, small_lds_bytes(MODE, 2)) &&
+             raise_lds_limit(gemm_a8w8_tile128<MODE, C_BF16, 4>, small_lds_bytes(MODE, 4)) &&
+             raise_lds_limit(gemm_a8w8_tile128<MODE, C_FP32, 4>, small_lds_bytes(MODE, 4));
+    return ok;
+}
+
+// runs with device `dev` current
+void set_up_device(int dev)
+{
+    DeviceState& d = g_dev[dev];
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) { d.status = A8W8_ERR_NO_DEVICE; return; }
+    d.num_cus = prop.multiProcessorCount;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) { d.status = A8W8_ERR_NO_DEVICE; return; }
+    const bool ok = raise_lds_limits_of_mode<MODE_TENSOR>() && raise_lds_limits_of_mode<MODE_ROWCOL>() &&
+                    raise_lds_limits_of_mode<MODE_BLOCK>() && raise_lds_limits_of_mode<MODE_MX>() &&
+                    raise_lds_limits_of_mode<MODE_MXT>() && raise_lds_limits_of_mode<MODE_BF16>() &&
+                    raise_lds_limits_of_mode<MODE_F4T>();
+    d.status = ok ? A8W8_OK : A8W8_ERR_LAUNCH;
+}
+
+// A8W8_OK when the current device is a gfx950 that has been set up (setting it up on first use).
+int device_status()
+{
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-    if (cached[dev] == 0) {
-        hipDeviceProp_t prop;
-        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return false;
-        g_num_cus[dev] = prop.multiProcessorCount;
-        cached[dev] = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
-    }
-    return cached[dev] == 1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return A8W8_ERR_NO_DEVICE;
+    std::call_once(g_dev[dev].once, set_up_device, dev);
+    return g_dev[dev].status;
 }
 
-int launch_status()
+// One kernel launch; the status is that of this launch alone (hipLaunchKernel's own return value, not the
+// thread's sticky last error, which an earlier unrelated runtime call may have set).
+template <class... P, class... A, size_t... I>
+int launch_impl(void (*kern)(P...), dim3 grid, dim3 block, unsigned lds, hipStream_t s, std::index_sequence<I...>, A&&... a)
 {
-    return hipGetLastError() == hipSuccess ? A8W8_OK : A8W8_ERR_LAUNCH;
+    std::tuple<P...> params{static_cast<P>(std::forward<A>(a))...};
+    void* ptrs[] = {(void*)&std::get<I>(params)...};
+    return hipLaunchKernel((const void*)kern, grid, block, ptrs, lds, s) == hipSuccess ? A8W8_OK : A8W8_ERR_LAUNCH;
 }
+template <class... P, class... A>
+int launch(void (*kern)(P...), dim3 grid, dim3 block, unsigned lds, hipStream_t s, A&&... a)
+{
+    static_assert(sizeof...(P) == sizeof...(A), "one argument per kernel parameter");
+    return launch_impl(kern, grid, block, lds, s, std::index_sequence_for<P...>{}, std::forward<A>(a)...);
+}
+// a launch in the middle of a sequence: leave with its status if it failed
+#define A8W8_LAUNCH_OR_RETURN(...)                       \
+    do {                                                 \
+        const int st_ = launch(__VA_ARGS__);             \
+        if (st_ != A8W8_OK) return st_;                  \
+    } while (0)
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
@@ -69,6 +138,10 @@ int validate_common(const a8w8_gemm_args* g)
     const long long b_span = g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k;
     if (a_span >= (1ll << 31) || b_span >= (1ll << 31)) return A8W8_ERR_TOO_LARGE;
     if (g->batch > 65535) return A8W8_ERR_TOO_LARGE;
+    // ... and the A-side block scales of all K groups, and count 128 x 128 tiles with an int
+    if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128 && (long long)(g->k / 128) * g->stride_sfa * 4 >= (1ll << 31))
+        return A8W8_ERR_TOO_LARGE;
+    if ((long long)((g->m + 127) / 128) * ((g->n + 127) / 128) >= (1ll << 31)) return A8W8_ERR_TOO_LARGE;
     return A8W8_OK;
 }
 
@@ -126,8 +199,6 @@ bool persist_ok(const a8w8_gemm_args* g)
 {
     // tiled MX scales come in pairs of K steps (one dword serves two steps)
     if (g->scale_mode == A8W8_SCALE_MX_E8M0_TILED && (g->k / BK) % 2 != 0) return false;
-    // the load offsets are formed with 24-bit multiplies
-    if (g->m >= (1 << 23) || g->n >= (1 << 23) || g->stride_a >= (1 << 23) || g->stride_b >= (1 << 23)) return false;
     return g->k >= 2 * BK &&
            (long long)g->batch * ((g->m + BM - 1) / BM) * ((g->n + BN - 1) / BN) < (1ll << 30);
 }
@@ -143,23 +214,22 @@ bool wide_ok(const a8w8_gemm_args* g)
 template <int MODE, int CDT>
 int launch_general(const GemmParams& p, int batch, hipStream_t stream);
 
+// compute units of the current device (256 before the device has been set up: kernel-name queries on a CPU box)
 int num_cus()
 {
     int dev = 0;
-    (void)hipGetDevice(&dev);
-    return g_num_cus[dev & 63] > 0 ? g_num_cus[dev & 63] : 256;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return 256;
+    return g_dev[dev].num_cus > 0 ? g_dev[dev].num_cus : 256;
 }
 
 // 128 x 128 tiles when all of them fit on the chip at once, two workgroups per compute unit: a problem of that
 // size leaves 256 x 256 tiles with at most half of the compute units.  Measured on 256 compute units against the
 // 256-tile kernels (block / row-col / tiled MX): 2.2x / 1.7x / 1.6x at 64 workgroups, 1.9x / 1.6x / 1.5x at 256,
 // +45% / +21% / +15% at 400, +37% / +17% / +9% at 512; beyond that the second round of workgroups costs more than
-// the idle compute units did (-9% for row/col at 576).  The scale loads of the block mode use 32-bit byte offsets.
+// the idle compute units did (-9% for row/col at 576).
 bool small_ok(const a8w8_gemm_args* g)
 {
-    const bool block = g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128;
     const bool mxt = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;
-    if (block && (long long)(g->k / BK) * g->stride_sfa * 4 >= (1ll << 31)) return false;
     // tiled MX scales with an odd number of K steps have no 256-tile kernel: any size runs here
     if (mxt && (g->k / BK) % 2 != 0) return true;
     const long long items128 = (long long)g->batch * ((g->m + SM_BM - 1) / SM_BM) * ((g->n + SM_BN - 1) / SM_BN);
@@ -169,19 +239,8 @@ bool small_ok(const a8w8_gemm_args* g)
 template <int MODE, int CDT, int STAGES>
 int launch_small_stages(const GemmParams& q, int batch, hipStream_t stream)
 {
-    static bool attr_set[64];
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    auto kern = gemm_a8w8_tile128<MODE, CDT, STAGES>;
-    constexpr int lds_bytes = small_lds_bytes(MODE, STAGES);
-    if (!attr_set[dev & 63]) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-            return A8W8_ERR_LAUNCH;
-        attr_set[dev & 63] = true;
-    }
     dim3 grid((unsigned)(q.tiles_m * q.tiles_n), 1, (unsigned)batch);
-    hipLaunchKernelGGL(kern, grid, dim3(SM_THREADS), lds_bytes, stream, q);
-    return launch_status();
+    return launch(gemm_a8w8_tile128<MODE, CDT, STAGES>, grid, dim3(SM_THREADS), small_lds_bytes(MODE, STAGES), stream, q);
 }
 
 // Up to one workgroup per compute unit: four LDS stages (deep prefetch, one workgroup per compute unit).  More: two
@@ -203,27 +262,6 @@ int launch_small(const GemmParams& p, int batch, hipStream_t stream)
 }
 
 template <int MODE, int CDT>
-int launch_tiled(const GemmParams& p, int batch, hipStream_t stream)
-{
-    static bool attr_set[64];
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if constexpr (MODE == MODE_MXT) return launch_general<MODE, CDT>(p, batch, stream);   // single K step: rare
-    else {
-    auto kern = gemm_a8w8_tile256<MODE, CDT>;
-    constexpr int lds_bytes = MODE == MODE_MX ? GEMM_LDS_BYTES_MX : GEMM_LDS_BYTES;
-    if (!attr_set[dev & 63]) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-            return A8W8_ERR_LAUNCH;
-        attr_set[dev & 63] = true;
-    }
-    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)batch);
-    hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), lds_bytes, stream, p);
-    return launch_status();
-    }
-}
-
-template <int MODE, int CDT>
 int launch_wide(const GemmParams& p, int batch, hipStream_t stream);
 
 // Persistent pipelined kernel (eight waves): one workgroup per CU walks the (batch, tile) list.
@@ -233,24 +271,13 @@ int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
     // tiled MX scales exist on the four-wave kernel only (whatever passes persist_ok with them also passes wide_ok)
     if constexpr (MODE == MODE_MXT) return launch_wide<MODE, CDT>(p, batch, stream);
     else {
-    static bool attr_set[64];
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    auto kern = gemm_a8w8_persist<MODE, CDT>;
-    constexpr int lds_bytes = MODE == MODE_MX ? PERSIST_LDS_BYTES_MX : MODE == MODE_ROWCOL ? PERSIST_LDS_BYTES_ROWCOL : PERSIST_LDS_BYTES;
-    if (!attr_set[dev & 63]) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-            return A8W8_ERR_LAUNCH;
-        attr_set[dev & 63] = true;
-    }
     PersistParams pp;
     pp.g = p;
     pp.batch = batch;
     pp.items = batch * p.tiles_m * p.tiles_n;
-    const int cus = g_num_cus[dev & 63] > 0 ? g_num_cus[dev & 63] : 256;
+    const int cus = num_cus();
     dim3 grid((unsigned)(pp.items < cus ? pp.items : cus), 1, 1);
-    hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), lds_bytes, stream, pp);
-    return launch_status();
+    return launch(gemm_a8w8_persist<MODE, CDT>, grid, dim3(GEMM_THREADS), persist_lds_bytes(MODE), stream, pp);
     }
 }
 
@@ -259,24 +286,13 @@ template <int MODE, int CDT>
 int launch_wide(const GemmParams& p, int batch, hipStream_t stream)
 {
     if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT || MODE == MODE_BF16 || MODE == MODE_F4T) {
-        static bool attr_set[64];
-        int dev = 0;
-        (void)hipGetDevice(&dev);
-        auto kern = gemm_a8w8_wide<MODE, CDT>;
-        constexpr int lds_bytes = wide_lds_bytes(MODE);
-        if (!attr_set[dev & 63]) {
-            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
-                return A8W8_ERR_LAUNCH;
-            attr_set[dev & 63] = true;
-        }
         PersistParams pp;
         pp.g = p;
         pp.batch = batch;
         pp.items = batch * p.tiles_m * p.tiles_n;
-        const int cus = g_num_cus[dev & 63] > 0 ? g_num_cus[dev & 63] : 256;
+        const int cus = num_cus();
         dim3 grid((unsigned)(pp.items < cus ? pp.items : cus), 1, 1);
-        hipLaunchKernelGGL(kern, grid, dim3(WIDE_THREADS), lds_bytes, stream, pp);
-        return launch_status();
+        return launch(gemm_a8w8_wide<MODE, CDT>, grid, dim3(WIDE_THREADS), wide_lds_bytes(MODE), stream, pp);
     } else {
         return launch_persist<MODE, CDT>(p, batch, stream);
     }
@@ -286,8 +302,7 @@ template <int MODE, int CDT>
 int launch_general(const GemmParams& p, int batch, hipStream_t stream)
 {
     dim3 grid((unsigned)((p.n + 15) / 16), (unsigned)((p.m + 15) / 16), (unsigned)batch);
-    hipLaunchKernelGGL((gemm_a8w8_general<MODE, CDT>), grid, dim3(256), 0, stream, p);
-    return launch_status();
+    return launch(gemm_a8w8_general<MODE, CDT>, grid, dim3(256), 0, stream, p);
 }
 
 
@@ -306,10 +321,6 @@ int launch_general(const GemmParams& p, int batch, hipStream_t stream)
         default: return A8W8_ERR_BAD_MODE;                                                  \
     }
 
-int dispatch_tiled(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
-{
-    A8W8_DISPATCH(launch_tiled, g->scale_mode, g->c_dtype, p, g->batch, s)
-}
 int dispatch_persist(const a8w8_gemm_args* g, const GemmParams& p, hipStream_t s)
 {
     A8W8_DISPATCH(launch_persist, g->scale_mode, g->c_dtype, p, g->batch, s)
@@ -358,8 +369,7 @@ int launch_flat_nt(const GemmParams& p, int batch, hipStream_t stream)
 {
     const int n_tiles = p.n / 16;
     dim3 grid((unsigned)(((n_tiles + NT - 1) / NT) * ((p.m + 16 * MT - 1) / (16 * MT))), 1, (unsigned)batch);
-    hipLaunchKernelGGL((flatmm_a8w8<NT, MT, CDT, MODE, BROW>), grid, dim3(FLAT_THREADS), 0, stream, p);
-    return launch_status();
+    return launch(flatmm_a8w8<NT, MT, CDT, MODE, BROW>, grid, dim3(FLAT_THREADS), 0, stream, p);
 }
 
 // Up to four groups of 16 activation rows share one pass over the weights; as many weight tiles per workgroup as
@@ -489,7 +499,9 @@ int launch_dense_fp8(const a8w8_gemm_args* g, hipStream_t s)
     if (!tiled_ok(g)) return dispatch_general(g, p, s);
     if (small_ok(g)) return dispatch_small(g, p, s);
     if (wide_ok(g)) return dispatch_wide(g, p, s);
-    return persist_ok(g) ? dispatch_persist(g, p, s) : dispatch_tiled(g, p, s);
+    // what is left has a single K step (k = 128) or more work items than the persistent kernels index: the 128-tile
+    // kernel runs any number of steps and tiles
+    return persist_ok(g) ? dispatch_persist(g, p, s) : dispatch_small(g, p, s);
 }
 
 }  // namespace
@@ -505,7 +517,7 @@ int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream)
     const a8w8_gemm_args* g = &local;
     const int shuf = validate_shuffled_b(g);
     if (shuf != A8W8_OK) return shuf;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
     // a skinny problem on shuffled weights: the flat kernel where it is the faster one
     if (g->b_preshuffled && validate_flat(g) == A8W8_OK && prefer_flat_fp8(g)) return launch_flat_fp8(g, s);
@@ -530,7 +542,7 @@ static int a16w16_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) * 2;
     const long long b_span = (g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k) * 2;
     if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
     // the tiled kernel reads bf16 rows as byte rows of 2k columns
     a8w8_gemm_args bytes = *g;
@@ -562,14 +574,14 @@ static int a16w16_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     }
     dim3 grid((unsigned)((g->n + 15) / 16), (unsigned)((g->m + 15) / 16), (unsigned)g->batch);
     if (g->c_dtype == A8W8_C_BF16)
-        hipLaunchKernelGGL((gemm_a16w16_general<C_BF16>), grid, dim3(256), 0, s, (const unsigned short*)g->a,
+        A8W8_LAUNCH_OR_RETURN((gemm_a16w16_general<C_BF16>), grid, dim3(256), 0, s, (const unsigned short*)g->a,
                            (const unsigned short*)g->b, g->c, g->m, g->n, g->k, g->stride_a, g->stride_b, g->stride_c,
                            (long long)g->stride_a_batch, (long long)g->stride_b_batch, (long long)g->stride_c_batch);
     else
-        hipLaunchKernelGGL((gemm_a16w16_general<C_FP32>), grid, dim3(256), 0, s, (const unsigned short*)g->a,
+        A8W8_LAUNCH_OR_RETURN((gemm_a16w16_general<C_FP32>), grid, dim3(256), 0, s, (const unsigned short*)g->a,
                            (const unsigned short*)g->b, g->c, g->m, g->n, g->k, g->stride_a, g->stride_b, g->stride_c,
                            (long long)g->stride_a_batch, (long long)g->stride_b_batch, (long long)g->stride_c_batch);
-    return launch_status();
+    return A8W8_OK;
 }
 
 int a16w16_gemm(const a8w8_gemm_args* g, void* hip_stream) { return a16w16_gemm_impl(g, hip_stream, true); }
@@ -599,7 +611,7 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
     const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) / 2;
     const long long b_span = (g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k) / 2;
     if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
     // the tiled kernel reads packed rows as byte rows of k/2 columns
     a8w8_gemm_args bytes = *g;
@@ -628,7 +640,7 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
     }
     dim3 grid((unsigned)((g->n + 15) / 16), (unsigned)((g->m + 15) / 16), (unsigned)g->batch);
 #define A4W4_GENERAL(CDT, TILED)                                                                                        \
-    hipLaunchKernelGGL((gemm_a4w4_general<CDT, TILED>), grid, dim3(256), 0, s, (const uint8_t*)g->a, (const uint8_t*)g->b, \
+    A8W8_LAUNCH_OR_RETURN((gemm_a4w4_general<CDT, TILED>), grid, dim3(256), 0, s, (const uint8_t*)g->a, (const uint8_t*)g->b, \
                        (const uint8_t*)g->sfa, (const uint8_t*)g->sfb, g->c, g->m, g->n, g->k, g->stride_a / 2,            \
                        g->stride_b / 2, g->stride_c, g->stride_sfa, g->stride_sfb, (long long)g->stride_a_batch / 2,       \
                        (long long)g->stride_b_batch / 2, (long long)g->stride_c_batch, (long long)g->stride_sfa_batch,     \
@@ -636,7 +648,7 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
     if (g->c_dtype == A8W8_C_BF16) { if (tiled) A4W4_GENERAL(C_BF16, true); else A4W4_GENERAL(C_BF16, false); }
     else { if (tiled) A4W4_GENERAL(C_FP32, true); else A4W4_GENERAL(C_FP32, false); }
 #undef A4W4_GENERAL
-    return launch_status();
+    return A8W8_OK;
 }
 
 int a4w4_gemm(const a8w8_gemm_args* g, void* hip_stream) { return a4w4_gemm_impl(g, hip_stream, true); }
@@ -659,7 +671,7 @@ static int a4w4_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
                          g->stride_sfb_batch % 16 != 0))
         return A8W8_ERR_MISALIGNED;
     if ((long long)g->n * g->k / 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     // several groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
     if (allow_dense && !prefer_flat(g->m, g->n, g->k / 2, false) && a4w4_gemm_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
@@ -688,25 +700,25 @@ int a4w4_quantize_mx(const float* src, int rows, int k, int ld, uint8_t* q, uint
     if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
     if (ld < k) return A8W8_ERR_BAD_STRIDE;
     if (tiled && ((uintptr_t)scale & 3)) return A8W8_ERR_MISALIGNED;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
     const long long threads = (long long)rows * k;
     if (tiled) {
         if (rows % 64 != 0 || k % 512 != 0) {
             const size_t dwords = mx_tiled_bytes(rows, k) / 4;
-            hipLaunchKernelGGL(mx_tiled_fill_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0, s, (uint32_t*)scale, dwords);
+            A8W8_LAUNCH_OR_RETURN(mx_tiled_fill_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0, s, (uint32_t*)scale, dwords);
         }
         if (quant_vec_ok(src, rows, k, ld, q, 4))
-            hipLaunchKernelGGL(quant_mxfp4_vec_kernel<true>, dim3((unsigned)((threads / 8 + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+            A8W8_LAUNCH_OR_RETURN(quant_mxfp4_vec_kernel<true>, dim3((unsigned)((threads / 8 + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
         else
-            hipLaunchKernelGGL(quant_mxfp4_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+            A8W8_LAUNCH_OR_RETURN(quant_mxfp4_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
     } else {
         if (quant_vec_ok(src, rows, k, ld, q, 4))
-            hipLaunchKernelGGL(quant_mxfp4_vec_kernel<false>, dim3((unsigned)((threads / 8 + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+            A8W8_LAUNCH_OR_RETURN(quant_mxfp4_vec_kernel<false>, dim3((unsigned)((threads / 8 + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
         else
-            hipLaunchKernelGGL(quant_mxfp4_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
+            A8W8_LAUNCH_OR_RETURN(quant_mxfp4_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k, ld, q, scale);
     }
-    return launch_status();
+    return A8W8_OK;
 }
 
 static int a16w16_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_dense)
@@ -721,7 +733,10 @@ static int a16w16_flat_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     if (!aligned16(g->a) || !aligned16(g->b) || g->stride_a % 8 != 0) return A8W8_ERR_MISALIGNED;
     if (g->batch > 1 && (g->stride_a_batch % 8 != 0 || g->stride_b_batch % 8 != 0)) return A8W8_ERR_MISALIGNED;
     if ((long long)g->n * g->k * 2 >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    // batch strides are doubled into byte counts held in an int
+    if (g->batch > 1 && ((long long)g->stride_a_batch * 2 >= (1ll << 31) || (long long)g->stride_b_batch * 2 >= (1ll << 31)))
+        return A8W8_ERR_TOO_LARGE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     // several groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
     if (allow_dense && !prefer_flat(g->m, g->n, 2ll * g->k, false) && a16w16_gemm_impl(g, hip_stream, false) == A8W8_OK)
         return A8W8_OK;
@@ -750,7 +765,7 @@ int a8w8_flatmm(const a8w8_gemm_args* g, void* hip_stream)
 {
     const int st = validate_flat(g);
     if (st != A8W8_OK) return st;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
     // several groups of 16 rows over weights too large to stay in cache: the MFMA kernels read the same weights
     if (!prefer_flat_fp8(g)) {
@@ -796,40 +811,40 @@ int a8w8_preshuffle_b_device(const void* b_dev, void* out_dev, int n, int k, voi
     if (n <= 0 || k <= 0) return A8W8_ERR_BAD_SHAPE;
     if (n % 16 != 0 || k % 64 != 0) return A8W8_ERR_BAD_GROUP;
     if (!aligned16(out_dev)) return A8W8_ERR_MISALIGNED;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     const long long units = (long long)n * k / 16;
-    hipLaunchKernelGGL(preshuffle_b_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0,
+    A8W8_LAUNCH_OR_RETURN(preshuffle_b_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0,
                        (hipStream_t)hip_stream, (const uint8_t*)b_dev, (uint8_t*)out_dev, n, k);
-    return launch_status();
+    return A8W8_OK;
 }
 
-size_t a8w8_cvt_f32_to_e4m3(const float* src, uint8_t* dst, size_t n, int dialect, int clamp240, void* hip_stream)
+int a8w8_cvt_f32_to_e4m3(const float* src, uint8_t* dst, size_t n, int dialect, int clamp240, void* hip_stream)
 {
-    if (!src || !dst || n == 0) return 0;
-    if (dialect != A8W8_E4M3_OCP && dialect != A8W8_E4M3_FNUZ) return 0;
-    if (!device_is_gfx950()) return 0;
+    if (dialect != A8W8_E4M3_OCP && dialect != A8W8_E4M3_FNUZ) return A8W8_ERR_BAD_MODE;
+    if (n == 0) return A8W8_OK;
+    if (!src || !dst) return A8W8_ERR_NULL_POINTER;
+    if ((n + 3) / 4 > 0x7fffffffull * 256) return A8W8_ERR_TOO_LARGE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
     const dim3 grid((unsigned)(((n + 3) / 4 + 255) / 256)), block(256);
-    if (dialect == A8W8_E4M3_OCP) {
-        if (clamp240) hipLaunchKernelGGL((cvt_f32_to_e4m3_kernel<0, 1>), grid, block, 0, s, src, dst, n);
-        else hipLaunchKernelGGL((cvt_f32_to_e4m3_kernel<0, 0>), grid, block, 0, s, src, dst, n);
-    } else {
-        if (clamp240) hipLaunchKernelGGL((cvt_f32_to_e4m3_kernel<1, 1>), grid, block, 0, s, src, dst, n);
-        else hipLaunchKernelGGL((cvt_f32_to_e4m3_kernel<1, 0>), grid, block, 0, s, src, dst, n);
-    }
-    return launch_status() == A8W8_OK ? n : 0;
+    if (dialect == A8W8_E4M3_OCP)
+        return clamp240 ? launch(cvt_f32_to_e4m3_kernel<0, 1>, grid, block, 0, s, src, dst, n)
+                        : launch(cvt_f32_to_e4m3_kernel<0, 0>, grid, block, 0, s, src, dst, n);
+    return clamp240 ? launch(cvt_f32_to_e4m3_kernel<1, 1>, grid, block, 0, s, src, dst, n)
+                    : launch(cvt_f32_to_e4m3_kernel<1, 0>, grid, block, 0, s, src, dst, n);
 }
 
-size_t a8w8_cvt_e4m3_to_f32(const uint8_t* src, float* dst, size_t n, int dialect, void* hip_stream)
+int a8w8_cvt_e4m3_to_f32(const uint8_t* src, float* dst, size_t n, int dialect, void* hip_stream)
 {
-    if (!src || !dst || n == 0) return 0;
-    if (dialect != A8W8_E4M3_OCP && dialect != A8W8_E4M3_FNUZ) return 0;
-    if (!device_is_gfx950()) return 0;
+    if (dialect != A8W8_E4M3_OCP && dialect != A8W8_E4M3_FNUZ) return A8W8_ERR_BAD_MODE;
+    if (n == 0) return A8W8_OK;
+    if (!src || !dst) return A8W8_ERR_NULL_POINTER;
+    if (n > 0x7fffffffull * 256) return A8W8_ERR_TOO_LARGE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
     const dim3 grid((unsigned)((n + 255) / 256)), block(256);
-    if (dialect == A8W8_E4M3_OCP) hipLaunchKernelGGL((cvt_e4m3_to_f32_kernel<0>), grid, block, 0, s, src, dst, n);
-    else hipLaunchKernelGGL((cvt_e4m3_to_f32_kernel<1>), grid, block, 0, s, src, dst, n);
-    return launch_status() == A8W8_OK ? n : 0;
+    return dialect == A8W8_E4M3_OCP ? launch(cvt_e4m3_to_f32_kernel<0>, grid, block, 0, s, src, dst, n)
+                                    : launch(cvt_e4m3_to_f32_kernel<1>, grid, block, 0, s, src, dst, n);
 }
 
 int a8w8_quantize(const float* src, int rows, int k, int ld, uint8_t* q, void* scale, int scale_mode, int group_rows,
@@ -841,82 +856,82 @@ int a8w8_quantize(const float* src, int rows, int k, int ld, uint8_t* q, void* s
     hipStream_t s = (hipStream_t)hip_stream;
     switch (scale_mode) {
         case A8W8_SCALE_TENSOR: {
-            if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+            if (const int ds = device_status(); ds != A8W8_OK) return ds;
             const long long total = (long long)rows * k;
             const unsigned grid = (unsigned)(total / 256 + 1 < 4096 ? total / 256 + 1 : 4096);
-            hipLaunchKernelGGL(quant_tensor_clear_kernel, dim3(1), dim3(1), 0, s, (float*)scale);
+            A8W8_LAUNCH_OR_RETURN(quant_tensor_clear_kernel, dim3(1), dim3(1), 0, s, (float*)scale);
             if (ld == k && total % 4 == 0 && aligned16(src) && ((uintptr_t)q & 3) == 0) {
                 const size_t units = (size_t)(total / 4);
                 const unsigned vgrid = (unsigned)(units / 1024 + 1 < 2048 ? units / 1024 + 1 : 2048);
-                hipLaunchKernelGGL(quant_tensor_amax_vec_kernel, dim3(vgrid), dim3(256), 0, s, (const float4*)src, units, (float*)scale);
-                hipLaunchKernelGGL(quant_tensor_apply_vec_kernel, dim3(vgrid), dim3(256), 0, s, (const float4*)src, units, (uint32_t*)q,
+                A8W8_LAUNCH_OR_RETURN(quant_tensor_amax_vec_kernel, dim3(vgrid), dim3(256), 0, s, (const float4*)src, units, (float*)scale);
+                A8W8_LAUNCH_OR_RETURN(quant_tensor_apply_vec_kernel, dim3(vgrid), dim3(256), 0, s, (const float4*)src, units, (uint32_t*)q,
                                    (const float*)scale);
             } else {
-                hipLaunchKernelGGL(quant_tensor_amax_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, (float*)scale);
-                hipLaunchKernelGGL(quant_tensor_apply_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, q, (const float*)scale);
+                A8W8_LAUNCH_OR_RETURN(quant_tensor_amax_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, (float*)scale);
+                A8W8_LAUNCH_OR_RETURN(quant_tensor_apply_kernel, dim3(grid), dim3(256), 0, s, src, rows, k, ld, q, (const float*)scale);
             }
-            hipLaunchKernelGGL(quant_tensor_finish_kernel, dim3(1), dim3(1), 0, s, (float*)scale);
-            return launch_status();
+            A8W8_LAUNCH_OR_RETURN(quant_tensor_finish_kernel, dim3(1), dim3(1), 0, s, (float*)scale);
+            return A8W8_OK;
         }
         case A8W8_SCALE_ROWCOL:
-            if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+            if (const int ds = device_status(); ds != A8W8_OK) return ds;
             if (quant_vec_ok(src, rows, k, ld, q, 4) && k <= 8192)
-                hipLaunchKernelGGL(quant_rowwise_vec_kernel<true>, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
+                A8W8_LAUNCH_OR_RETURN(quant_rowwise_vec_kernel<true>, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
             else if (quant_vec_ok(src, rows, k, ld, q, 4))
-                hipLaunchKernelGGL(quant_rowwise_vec_kernel<false>, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
+                A8W8_LAUNCH_OR_RETURN(quant_rowwise_vec_kernel<false>, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
             else
-                hipLaunchKernelGGL(quant_rowwise_kernel, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
-            return launch_status();
+                A8W8_LAUNCH_OR_RETURN(quant_rowwise_kernel, dim3((unsigned)rows), dim3(256), 0, s, src, k, ld, q, (float*)scale);
+            return A8W8_OK;
         case A8W8_SCALE_BLOCK_1x128_128x128:
             if (k % 128 != 0) return A8W8_ERR_BAD_GROUP;
             if (group_rows == 1) {
-                if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+                if (const int ds = device_status(); ds != A8W8_OK) return ds;
                 const long long waves = (long long)rows * (k / 128);
                 if (quant_vec_ok(src, rows, k, ld, q, 4))
-                    hipLaunchKernelGGL(quant_1x128_vec_kernel, dim3((unsigned)((waves + 8 * QUANT_1X128_GROUPS - 1) / (8 * QUANT_1X128_GROUPS))), dim3(256), 0, s, src, rows, k, ld, q,
+                    A8W8_LAUNCH_OR_RETURN(quant_1x128_vec_kernel, dim3((unsigned)((waves + 8 * QUANT_1X128_GROUPS - 1) / (8 * QUANT_1X128_GROUPS))), dim3(256), 0, s, src, rows, k, ld, q,
                                        (float*)scale);
                 else
-                    hipLaunchKernelGGL(quant_1x128_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, src, rows, k,
+                    A8W8_LAUNCH_OR_RETURN(quant_1x128_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, src, rows, k,
                                        ld, q, (float*)scale);
-                return launch_status();
+                return A8W8_OK;
             }
             if (group_rows == 128) {
                 if (rows % 128 != 0) return A8W8_ERR_BAD_GROUP;
-                if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
-                hipLaunchKernelGGL(quant_128x128_kernel, dim3((unsigned)(k / 128), (unsigned)(rows / 128)), dim3(256), 0,
+                if (const int ds = device_status(); ds != A8W8_OK) return ds;
+                A8W8_LAUNCH_OR_RETURN(quant_128x128_kernel, dim3((unsigned)(k / 128), (unsigned)(rows / 128)), dim3(256), 0,
                                    s, src, k, ld, q, (float*)scale);
-                return launch_status();
+                return A8W8_OK;
             }
             return A8W8_ERR_BAD_MODE;
         case A8W8_SCALE_MX_E8M0_1x32: {
             if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
-            if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+            if (const int ds = device_status(); ds != A8W8_OK) return ds;
             const long long threads = (long long)rows * k;
             if (quant_vec_ok(src, rows, k, ld, q, 4))
-                hipLaunchKernelGGL(quant_mx_vec_kernel<false>, dim3((unsigned)((threads / (4 * QUANT_MX_CHUNKS) + 255) / 256)), dim3(256), 0, s, src,
+                A8W8_LAUNCH_OR_RETURN(quant_mx_vec_kernel<false>, dim3((unsigned)((threads / (4 * QUANT_MX_CHUNKS) + 255) / 256)), dim3(256), 0, s, src,
                                    rows, k, ld, q, (uint8_t*)scale);
             else
-                hipLaunchKernelGGL(quant_mx_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k,
+                A8W8_LAUNCH_OR_RETURN(quant_mx_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows, k,
                                    ld, q, (uint8_t*)scale);
-            return launch_status();
+            return A8W8_OK;
         }
         case A8W8_SCALE_MX_E8M0_TILED: {
             if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
-            if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+            if (const int ds = device_status(); ds != A8W8_OK) return ds;
             if (((uintptr_t)scale & 3) != 0) return A8W8_ERR_MISALIGNED;
             const long long threads = (long long)rows * k;
             if (rows % 64 != 0 || k % 512 != 0) {   // positions no (row, block) owns: 127 first
                 const size_t dwords = mx_tiled_bytes(rows, k) / 4;
-                hipLaunchKernelGGL(mx_tiled_fill_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0, s,
+                A8W8_LAUNCH_OR_RETURN(mx_tiled_fill_kernel, dim3((unsigned)((dwords + 255) / 256)), dim3(256), 0, s,
                                    (uint32_t*)scale, dwords);
             }
             if (quant_vec_ok(src, rows, k, ld, q, 4))
-                hipLaunchKernelGGL(quant_mx_vec_kernel<true>, dim3((unsigned)((threads / (4 * QUANT_MX_CHUNKS) + 255) / 256)), dim3(256), 0, s, src,
+                A8W8_LAUNCH_OR_RETURN(quant_mx_vec_kernel<true>, dim3((unsigned)((threads / (4 * QUANT_MX_CHUNKS) + 255) / 256)), dim3(256), 0, s, src,
                                    rows, k, ld, q, (uint8_t*)scale);
             else
-                hipLaunchKernelGGL(quant_mx_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows,
+                A8W8_LAUNCH_OR_RETURN(quant_mx_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, src, rows,
                                    k, ld, q, (uint8_t*)scale);
-            return launch_status();
+            return A8W8_OK;
         }
         default:
             return A8W8_ERR_BAD_MODE;
@@ -930,11 +945,11 @@ int a8w8_mx_tile_scales(const uint8_t* sf, int rows, int k, int stride, uint8_t*
     if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
     if (stride < k / 32) return A8W8_ERR_BAD_STRIDE;
     if (!aligned16(out)) return A8W8_ERR_MISALIGNED;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     const size_t units = mx_tiled_bytes(rows, k) >> 10;
-    hipLaunchKernelGGL(mx_tile_scales_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0,
+    A8W8_LAUNCH_OR_RETURN(mx_tile_scales_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0,
                        (hipStream_t)hip_stream, sf, rows, stride, out, (const uint8_t*)nullptr, 0, 0, (uint8_t*)nullptr, k);
-    return launch_status();
+    return A8W8_OK;
 }
 
 int a8w8_mx_tile_scales_ab(const uint8_t* sfa, int m, int stride_sfa, uint8_t* out_a, const uint8_t* sfb, int n,
@@ -945,11 +960,11 @@ int a8w8_mx_tile_scales_ab(const uint8_t* sfa, int m, int stride_sfa, uint8_t* o
     if (k % 32 != 0) return A8W8_ERR_BAD_GROUP;
     if (stride_sfa < k / 32 || stride_sfb < k / 32) return A8W8_ERR_BAD_STRIDE;
     if (!aligned16(out_a) || !aligned16(out_b)) return A8W8_ERR_MISALIGNED;
-    if (!device_is_gfx950()) return A8W8_ERR_NO_DEVICE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
     const size_t units0 = mx_tiled_bytes(m, k) >> 10, units1 = mx_tiled_bytes(n, k) >> 10;
-    hipLaunchKernelGGL(mx_tile_scales_kernel, dim3((unsigned)((units0 + units1 + 3) / 4)), dim3(256), 0,
+    A8W8_LAUNCH_OR_RETURN(mx_tile_scales_kernel, dim3((unsigned)((units0 + units1 + 3) / 4)), dim3(256), 0,
                        (hipStream_t)hip_stream, sfa, m, stride_sfa, out_a, sfb, n, stride_sfb, out_b, k);
-    return launch_status();
+    return A8W8_OK;
 }
 
 size_t a8w8_mx_tiled_bytes(int rows, int k)
@@ -1079,10 +1094,25 @@ const char* a8w8_kernel_name(const a8w8_gemm_args* g)
     if (!tiled_ok(g)) return "gemm_a8w8_general";
     if (small_ok(g)) return "gemm_a8w8_tile128";
     if (wide_ok(g)) return "gemm_a8w8_wide";
-    if (persist_ok(g)) return "gemm_a8w8_persist";
-    return g->scale_mode == A8W8_SCALE_MX_E8M0_TILED ? "gemm_a8w8_general" : "gemm_a8w8_tile256";
+    return persist_ok(g) ? "gemm_a8w8_persist" : "gemm_a8w8_tile128";
 }
 
-int a8w8_version(void) { return 200; }
+int a8w8_init(int device)
+{
+    int current = 0;
+    if (hipGetDevice(&current) != hipSuccess) return A8W8_ERR_NO_DEVICE;
+    if (device < 0) device = current;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || device >= count || device >= MAX_DEVICES) return A8W8_ERR_NO_DEVICE;
+    if (device != current && hipSetDevice(device) != hipSuccess) {
+        (void)hipGetLastError();      // the failed switch must not linger as the thread's last error
+        return A8W8_ERR_NO_DEVICE;
+    }
+    const int st = device_status();
+    if (device != current) (void)hipSetDevice(current);
+    return st;
+}
+
+int a8w8_version(void) { return 300; }
 
 }  // extern "C"

@@ -69,7 +69,7 @@ A8W8_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes)
 // Pre-shuffled B [n/16][k/64][4][16][16 B]: the piece's 64-wide K block, its quarter of the block, the row's slot.
 A8W8_DEV int b_lane_offset(const GemmParams& p, int row, int piece_bytes)
 {
-    if (p.b_kshift == 7) return __mul24(row, p.ldb) + piece_bytes;
+    if (p.b_kshift == 7) return row * p.ldb + piece_bytes;
     return (row >> 4) * (p.k << 4) + ((piece_bytes >> 6) << 10) + (((piece_bytes >> 4) & 3) << 8) + ((row & 15) << 4);
 }
 // Extent of one batch entry of B for its buffer descriptor (rows past n read as zero in both layouts).

@@ -25,7 +25,7 @@
 #pragma once
 #include <utility>
 
-#include "gemm_tile.hpp"
+#include "gemm_common.hpp"
 
 namespace a8w8 {
 
@@ -124,7 +124,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         const int m0 = tm * BM, n0 = tn * BN;
         rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
         rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, b_extent_bytes(p));
-        ld_voff_a = __mul24(m0 + ld_row, p.lda) + ld_piece16;
+        ld_voff_a = (m0 + ld_row) * p.lda + ld_piece16;
         ld_voff_b = b_lane_offset(p, n0 + ld_row, ld_piece16);
         if constexpr (MODE == MODE_MX) {
             const bool is_b = wave >= 4;           // waves 0-3 stage A-row scales, 4-7 B-row scales

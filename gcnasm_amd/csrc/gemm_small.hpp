@@ -12,7 +12,7 @@
 // direct-to-LDS load per wave, so that the loop's wait counts stay fixed and no global load has to be waited
 // for inside a step.  Operands: FP8 E4M3, bf16 (byte rows of 2k columns), packed E2M1 (byte rows of k/2 columns).
 #pragma once
-#include "gemm_tile.hpp"
+#include "gemm_common.hpp"
 
 namespace a8w8 {
 

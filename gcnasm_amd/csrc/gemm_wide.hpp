@@ -151,7 +151,7 @@ gemm_a8w8_wide(PersistParams pp)
         rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, b_extent_bytes(p));
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            ld_voff_a[h] = __mul24(tm * BM + 128 * h + ld_row, p.lda) + ld_piece16;
+            ld_voff_a[h] = (tm * BM + 128 * h + ld_row) * p.lda + ld_piece16;
             ld_voff_b[h] = b_lane_offset(p, tn * BN + 128 * h + ld_row, ld_piece16);
         }
     };

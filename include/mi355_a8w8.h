@@ -33,7 +33,7 @@ typedef enum {
     A8W8_ERR_BAD_MODE = -6,       /* unknown scale_mode / c_dtype / dialect, or a combination
                                      the entry point does not implement                    */
     A8W8_ERR_TOO_LARGE = -7,      /* an offset would not fit the 32-bit addressing in use   */
-    A8W8_ERR_LAUNCH = -8,         /* hipGetLastError() reported a failed launch             */
+    A8W8_ERR_LAUNCH = -8,         /* the kernel launch itself returned an error             */
     A8W8_ERR_NO_DEVICE = -9,      /* no gfx950 device is current                            */
     A8W8_ERR_IO = -10,            /* a weight file could not be opened, read or written     */
     A8W8_ERR_BAD_FILE = -11       /* not a weight file of this version, truncated, or its
@@ -49,10 +49,16 @@ typedef enum {
  *   MX      uint8 E8M0 exponents, one per 32 K-elements, value 2^(e-127):
  *             sfa[i*stride_sfa + k/32], sfb[j*stride_sfb + k/32]
  *   MX_TILED  the same exponents re-arranged by a8w8_mx_tile_scales (or written that way by
- *             a8w8_quantize) so that the GEMM reads them as whole cache lines:
- *             sf[((kb/16)*rows + r)*16 + (kb%4)*4 + (kb/4)%4],  kb = k/32, rows = m or n;
- *             stride_sfa / stride_sfb are ignored, ceil(k/512)*rows*16 bytes each.  With row-major
- *             scales every 16 bytes the kernel needs sit in a different 128-byte line.       */
+ *             a8w8_quantize) so that the GEMM reads them as whole cache lines; stride_sfa /
+ *             stride_sfb are ignored.  a8w8_mx_tiled_bytes(rows, k) =
+ *             ceil(k/512) * ceil(rows/64) * 1024 bytes per array (rows = m or n), laid out as
+ *                 [k/512][ceil(rows/64)][pair: 2][r16: 16][g: 4][jp: 2][par: 2][s: 2]   (one byte each)
+ *             With kb = k/32 (the 32-wide K block) and rr = r % 64, the exponent of (row r, block kb) is byte
+ *                 ((((kb/16) * ceil(rows/64) + r/64) * 2 + (kb/8)%2) * 64 + (4*((rr/8)%4) + rr%4) * 4 + kb%4) * 8
+ *                   + (rr/32) * 4 + ((rr/4)%2) * 2 + (kb/4)%2
+ *             (pair = (kb/8)%2, r16 = 4*((rr/8)%4) + rr%4, g = kb%4, jp = rr/32, par = (rr/4)%2, s = (kb/4)%2).
+ *             Positions no (row, block) owns (rows past m or n, blocks past k) hold 127, the identity scale.
+ *             With row-major scales every 16 bytes the kernel needs sit in a different 128-byte line. */
 typedef enum {
     A8W8_SCALE_TENSOR = 0,
     A8W8_SCALE_ROWCOL = 1,
@@ -159,21 +165,25 @@ A8W8_API int a8w8_preshuffle_b_device(const void* b_dev, void* out_dev, int n, i
 
 /* fp32 -> E4M3, device buffers, one byte per element.
  *   clamp240 != 0: to_fp8_raw_from_fp32 (cvt_fp8/test.cpp:21-43): finite inputs are
- *       clamped to [-240, 240] by a median-of-three and then converted by the hardware
- *       instruction; NaN/Inf bypass the clamp.
+ *       clamped to [-240, 240] by a median-of-three and then converted; NaN/Inf bypass the
+ *       clamp and are converted as they are.
  *   clamp240 == 0: the unclamped packed convert of pk_cvt_fp8x4_fp32x4_rne
  *       (pk_cvt/test.cpp:220-257): elements 4i..4i+3 become the four bytes of word i,
- *       little-endian, saturating to the largest finite value.
- * dialect OCP uses the gfx950 hardware convert; FNUZ reproduces the gfx942 hardware result
- * (bias 8, max 240, NaN 0x80) in software on the device.  Returns the element count
- * converted, or 0 on error. */
-A8W8_API size_t a8w8_cvt_f32_to_e4m3(const float* src_dev, uint8_t* dst_dev, size_t n, int dialect,
-                                     int clamp240, void* hip_stream);
+ *       little-endian.
+ * dialect OCP is the gfx950 hardware convert (the instruction both reference programs call by
+ * builtin), round to nearest even and NOT saturating: NaN -> 0xFF, +-Inf -> 0x7F / 0xFF, and a
+ * magnitude that rounds beyond 448 (anything above 464) -> the NaN code 0x7F | sign; so only
+ * clamp240 protects against overflow.  Dialect FNUZ (bias 8, max 240, NaN 0x80, no -0: what
+ * gfx942 hardware converts to) is computed in software on the device with the arithmetic of
+ * ROCm's __hip_fp8_e4m3_fnuz: round to nearest even, saturating to +-240, NaN/Inf -> 0x80.
+ * n == 0 is a no-op.  Returns an a8w8_status. */
+A8W8_API int a8w8_cvt_f32_to_e4m3(const float* src_dev, uint8_t* dst_dev, size_t n, int dialect,
+                                  int clamp240, void* hip_stream);
 /* E4M3 -> fp32, device buffers: fp8_e4m3fnuz_to_fp32_raw (cvt_fp8/test.cpp:59-90) and
  * run_cast_from_f8<fp8, float, true> (pk_cvt/test.cpp:340-421) for FNUZ (0x80 -> NaN with
- * bits 0x7F800001); the hardware convert for OCP. */
-A8W8_API size_t a8w8_cvt_e4m3_to_f32(const uint8_t* src_dev, float* dst_dev, size_t n, int dialect,
-                                     void* hip_stream);
+ * bits 0x7F800001); the hardware convert for OCP.  Returns an a8w8_status. */
+A8W8_API int a8w8_cvt_e4m3_to_f32(const uint8_t* src_dev, float* dst_dev, size_t n, int dialect,
+                                  void* hip_stream);
 
 /* Quantisation front end: fp32 rows [rows, k] (leading dimension ld, elements) -> OCP E4M3
  * bytes [rows, k] plus scales, in the layouts a8w8_gemm consumes.
@@ -232,6 +242,14 @@ A8W8_API const char* a8w8_status_string(int status);
 /* Name of the kernel variant a8w8_gemm / a8w8_flatmm would launch for these arguments
  * (for logs and profiles); NULL if the arguments are rejected. */
 A8W8_API const char* a8w8_kernel_name(const a8w8_gemm_args* args);
+
+/* Optional explicit set-up of one device (device < 0: the current one): queries its architecture and
+ * compute-unit count and raises the dynamic-LDS limit of every kernel variant.  The same work happens,
+ * once per device and thread-safely, inside the first entry point called with that device current; call
+ * this beforehand when that first call would otherwise fall inside a stream capture or a timed region.
+ * No counterpart in the reference (its program configures nothing: one kernel, static LDS).
+ * A8W8_OK, or A8W8_ERR_NO_DEVICE if the device is not a gfx950. */
+A8W8_API int a8w8_init(int device);
 
 /* Library version, major*10000 + minor*100 + patch. */
 A8W8_API int a8w8_version(void);

@@ -55,6 +55,9 @@ def lib():
         L.orc_f32_to_bf16.argtypes = [ctypes.c_float]
         L.orc_decode_vec.argtypes = [_u8p, _f32p, ctypes.c_size_t, ctypes.c_int]
         L.orc_encode_vec.argtypes = [_f32p, _u8p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int]
+        L.orc_convert_vec.argtypes = [_f32p, _u8p, ctypes.c_size_t, ctypes.c_int]
+        L.orc_e4m3_ocp_encode_hw.restype = ctypes.c_uint8
+        L.orc_e4m3_ocp_encode_hw.argtypes = [ctypes.c_float]
         L.orc_bf16_vec.argtypes = [_f32p, _u16p, ctypes.c_size_t]
         L.orc_gemm_ref.argtypes = [_u8p, _u8p, _f32p, _f32p, _f32p] + [ctypes.c_int] * 14
         L.orc_gemm_ref_mx.argtypes = [_u8p, _u8p, _u8p, _u8p, _f32p] + [ctypes.c_int] * 11
@@ -113,6 +116,15 @@ def encode(x, dialect=OCP, clamp240=False):
     x = _c(x, np.float32)
     out = np.empty(x.shape, np.uint8)
     lib().orc_encode_vec(_p(x, _f32p), _p(out, _u8p), x.size, dialect, int(clamp240))
+    return out
+
+
+def convert(x, dialect=OCP):
+    """The device's unclamped convert: the gfx950 instruction (OCP, not saturating: overflow and Inf
+    give the NaN code) or, for FNUZ, the saturating conversion of __hip_fp8_e4m3_fnuz."""
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint8)
+    lib().orc_convert_vec(_p(x, _f32p), _p(out, _u8p), x.size, dialect)
     return out
 
 

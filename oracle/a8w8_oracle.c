@@ -16,9 +16,13 @@
  *   orc_e4m3_ocp_decode    closed form of the OCP FP8 spec; hip_fp8.h fixture.
  *   orc_e4m3_*_encode      brute-force nearest-even over the decode table,
  *       hip_fp8.h fixture, known tie -54 -> -56 (cvt_fp8/test.cpp:133).
- *   orc_cvt_fp8_clamp240   finite inputs pinned as above; NaN/Inf inputs are
- *       whatever the hardware convert returns and are PARITY UNPINNED here
- *       (the reference prints, never asserts, those cases).
+ *   orc_e4m3_ocp_encode_hw   the gfx950 hardware convert the reference calls by builtin
+ *       (cvt_fp8/test.cpp:37, pk_cvt/test.cpp:242-243): the OCP FP8 specification's
+ *       non-saturating conversion.  Equal to the saturating encoder wherever the rounded
+ *       magnitude is representable (the hip_fp8.h fixture), overflow / Inf -> sign | 0x7F and
+ *       NaN -> 0xFF as the specification's non-saturating mode prescribes; the GPU tests feed
+ *       NaN, +-Inf, +-1e9, +-449, +-464, +-465 and +-241 to the instruction itself.
+ *   orc_cvt_fp8_clamp240   the clamp is a median of three, the convert as above.
  *   orc_gemm_ref / orc_gemm_ref_mx   brute force in float64 on tiny shapes,
  *       exact-integer inputs, scale-mode reductions.
  *   orc_preshuffle_b       bijection + flatmm(A, shuffle(B)) == gemm(A, B).
@@ -160,11 +164,32 @@ static uint8_t encode_e4m3(float x, int fnuz)
 ORC_API uint8_t orc_e4m3_ocp_encode(float x) { return encode_e4m3(x, 0); }
 ORC_API uint8_t orc_e4m3_fnuz_encode(float x) { return encode_e4m3(x, 1); }
 
+/* What __builtin_amdgcn_cvt_pk_fp8_f32 returns on gfx950 (the instruction behind
+ * cvt_fp8/test.cpp:37 and pk_cvt/test.cpp:242-243 on this target): OCP E4M3, round to nearest
+ * even, NOT saturating -- the non-saturating conversion of the OCP FP8 specification:
+ *   NaN (either sign)                  -> 0xFF
+ *   +-Inf                              -> sign | 0x7F   (the NaN code: E4M3 has no infinity)
+ *   magnitude that rounds beyond 448   -> sign | 0x7F   (everything above the tie 464;
+ *                                         (448, 464] still rounds to 448 = 0x7E)
+ *   everything else                    as the saturating encoder above. */
+ORC_API uint8_t orc_e4m3_ocp_encode_hw(float x)
+{
+    const uint32_t u = f2u(x);
+    const uint8_t sign = (uint8_t)((u >> 31) << 7);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0xff;
+    if (fabsf(x) > 464.0f) return (uint8_t)(sign | 0x7f);      /* includes +-Inf */
+    return encode_e4m3(x, 0);
+}
+/* The convert of dialect `fnuz`: the gfx950 instruction for OCP; for FNUZ the conversion of ROCm's
+ * __hip_fp8_e4m3_fnuz (round to nearest even, saturating to +-240, NaN/Inf -> 0x80), which is what
+ * the library computes in software for that dialect. */
+static uint8_t convert_e4m3(float x, int fnuz) { return fnuz ? encode_e4m3(x, 1) : orc_e4m3_ocp_encode_hw(x); }
+
 /* to_fp8_raw_from_fp32, cvt_fp8/test.cpp:21-43: unless the input is NaN/Inf it is clamped
  * to [-240, 240] with a median-of-three, then converted by the hardware instruction in
  * the dialect of the target (fnuz != 0: gfx942, fnuz == 0: gfx950 / OCP).  NaN/Inf inputs
- * bypass the clamp and produce whatever the hardware convert produces; this restatement
- * returns the dialect's NaN code for them (PARITY UNPINNED for those inputs). */
+ * bypass the clamp and go through the convert as they are: on gfx950 NaN -> 0xFF,
+ * +Inf -> 0x7F, -Inf -> 0xFF; FNUZ 0x80 for all three. */
 ORC_API uint8_t orc_cvt_fp8_clamp240(float v, int fnuz)
 {
     uint32_t u = f2u(v);
@@ -172,17 +197,18 @@ ORC_API uint8_t orc_cvt_fp8_clamp240(float v, int fnuz)
         if (v > 240.0f) v = 240.0f;
         if (v < -240.0f) v = -240.0f;
     }
-    return encode_e4m3(v, fnuz);
+    return convert_e4m3(v, fnuz);
 }
 
 /* pk_cvt_fp8x4_fp32x4_rne, pk_cvt/test.cpp:220-257: two packed converts (s0,s1)->x and
  * (s2,s3)->y, both into the low word, then a byte permute with selector 0x05040100 that
  * yields bytes [x.b0, x.b1, y.b0, y.b1], i.e. little-endian [f8(s0), f8(s1), f8(s2), f8(s3)].
- * No clamp is applied before the convert. */
+ * No clamp is applied before the convert, so on gfx950 magnitudes that round beyond 448 come out
+ * as the NaN code (orc_e4m3_ocp_encode_hw). */
 ORC_API uint32_t orc_pk_cvt_fp8x4(const float s[4], int fnuz)
 {
-    uint32_t x = (uint32_t)encode_e4m3(s[0], fnuz) | ((uint32_t)encode_e4m3(s[1], fnuz) << 8);
-    uint32_t y = (uint32_t)encode_e4m3(s[2], fnuz) | ((uint32_t)encode_e4m3(s[3], fnuz) << 8);
+    uint32_t x = (uint32_t)convert_e4m3(s[0], fnuz) | ((uint32_t)convert_e4m3(s[1], fnuz) << 8);
+    uint32_t y = (uint32_t)convert_e4m3(s[2], fnuz) | ((uint32_t)convert_e4m3(s[3], fnuz) << 8);
     /* v_perm_b32(y, x, 0x05040100): selector bytes 0,1 pick x.b0,x.b1; 4,5 pick y.b0,y.b1 */
     return (x & 0xffffu) | ((y & 0xffffu) << 16);
 }
@@ -209,6 +235,11 @@ ORC_API void orc_encode_vec(const float* in, uint8_t* out, size_t n, int dialect
 #pragma omp parallel for schedule(static)
     for (size_t i = 0; i < n; ++i)
         out[i] = clamp240 ? orc_cvt_fp8_clamp240(in[i], dialect) : encode_e4m3(in[i], dialect);
+}
+/* the unclamped convert of the device (pk_cvt_fp8x4_fp32x4_rne element by element) */
+ORC_API void orc_convert_vec(const float* in, uint8_t* out, size_t n, int dialect)
+{
+    for (size_t i = 0; i < n; ++i) out[i] = convert_e4m3(in[i], dialect);
 }
 ORC_API void orc_bf16_vec(const float* in, uint16_t* out, size_t n)
 {

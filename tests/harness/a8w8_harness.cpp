@@ -38,22 +38,22 @@ int orc_num_threads(void);
 #define HARNESS_KIND 0   // 0 block scale, 1 dense 8-wave, 2 flatmm
 #endif
 
-#define CHECK_HIP(call)                                                                              \
-    do {                                                                                             \
-        hipError_t status_ = call;                                                                   \
-        if (status_ != hipSuccess) {                                                                 \
-            fprintf(stderr, "HIP error (%s:%d): %s\n", __FILE__, __LINE__, hipGetErrorString(status_)); \
-            exit(1);                                                                                 \
-        }                                                                                            \
-    } while (0)
-#define CHECK_A8W8(call)                                                                      \
-    do {                                                                                      \
-        int status_ = call;                                                                   \
-        if (status_ != 0) {                                                                   \
-            fprintf(stderr, "a8w8 error (%s:%d): %s\n", __FILE__, __LINE__, a8w8_status_string(status_)); \
-            exit(1);                                                                          \
-        }                                                                                     \
-    } while (0)
+// Every runtime and library call is checked; a failure names the call site and ends the program with status 1,
+// which is what the reference program does on a HIP error (host.cc:17-26).
+static void require_hip(hipError_t err, const char* what, int line)
+{
+    if (err == hipSuccess) return;
+    fprintf(stderr, "%s failed at line %d: %s\n", what, line, hipGetErrorString(err));
+    exit(1);
+}
+static void require_a8w8(int status, const char* what, int line)
+{
+    if (status == A8W8_OK) return;
+    fprintf(stderr, "%s failed at line %d: %s\n", what, line, a8w8_status_string(status));
+    exit(1);
+}
+#define CHECK_HIP(call) require_hip((call), #call, __LINE__)
+#define CHECK_A8W8(call) require_a8w8((call), #call, __LINE__)
 
 // Seeded replacement for the reference's rand_vector (host.cc:32-44, unseeded there): splitmix64
 // stream -> uniform [lo, hi); Box-Muller for normals.
@@ -138,24 +138,41 @@ static bool valid_vector(const float* ref, const float* out, size_t n, float rel
     return errors <= allowed;
 }
 
-// benchmark_kernel (host.cc:92-126): 200 warm-up launches, 100 timed between two events
+// A pair of HIP events on the default stream (the stream every launch of this program uses).
+struct StreamTimer {
+    hipEvent_t first{}, last{};
+    StreamTimer()
+    {
+        CHECK_HIP(hipEventCreate(&first));
+        CHECK_HIP(hipEventCreate(&last));
+    }
+    ~StreamTimer()
+    {
+        (void)hipEventDestroy(first);
+        (void)hipEventDestroy(last);
+    }
+    void begin() { CHECK_HIP(hipEventRecord(first)); }
+    float end_ms()
+    {
+        float ms = 0.f;
+        CHECK_HIP(hipEventRecord(last));
+        CHECK_HIP(hipEventSynchronize(last));
+        CHECK_HIP(hipEventElapsedTime(&ms, first, last));
+        return ms;
+    }
+};
+
+// The reference's timing protocol (benchmark_kernel, host.cc:92-126): untimed warm-up launches (200 there), then
+// `iterations` launches (100 there) between two events; returns the mean time of one launch in ms.
 template <class F>
-static float benchmark(F launch, int warmup = 200, int iterations = 100)
+static float benchmark(F launch, int warmup, int iterations)
 {
     for (int i = 0; i < warmup; ++i) launch(i);
-    hipEvent_t start, stop;
-    CHECK_HIP(hipEventCreate(&start));
-    CHECK_HIP(hipEventCreate(&stop));
     CHECK_HIP(hipDeviceSynchronize());
-    CHECK_HIP(hipEventRecord(start));
+    StreamTimer timer;
+    timer.begin();
     for (int i = 0; i < iterations; ++i) launch(i);
-    CHECK_HIP(hipEventRecord(stop));
-    CHECK_HIP(hipEventSynchronize(stop));
-    float total = 0.f;
-    CHECK_HIP(hipEventElapsedTime(&total, start, stop));
-    CHECK_HIP(hipEventDestroy(start));
-    CHECK_HIP(hipEventDestroy(stop));
-    return total / iterations;
+    return timer.end_ms() / (float)iterations;
 }
 
 template <class T>
@@ -172,39 +189,44 @@ int main(int argc, char** argv)
     // defaults of the reference program (host.cc:134-138) for the block-scale build
     int M = HARNESS_KIND == 2 ? 16 : 256, N = HARNESS_KIND == 2 ? 16384 : 512, K = HARNESS_KIND == 2 ? 7168 : 256;
     int batch = HARNESS_KIND == 0 ? 8 : 1, verify = 0, seed = 0xA8A8, rotate = 4;
+    int iters = 100, warmup = 200;      // the reference's protocol (host.cc:92-94); --iters / --warmup change it
     std::string scale_mode = HARNESS_KIND == 0 ? "block" : "rowcol";
 
-    // "-m 4096" and "-m=4096" are both accepted (host.cc:140-173)
-    auto parse_val = [](const char* arg, const char* flag) -> const char* {
-        const size_t len = strlen(flag);
-        if (strncmp(arg, flag, len) == 0) {
-            if (arg[len] == '=') return arg + len + 1;
-            if (arg[len] == '\0') return reinterpret_cast<const char*>(1);
-        }
-        return nullptr;
+    // Flags take their value as the next argument ("-m 4096") or after an equals sign ("-m=4096"), as in the
+    // reference program (host.cc:140-173); unknown arguments are ignored there and here.
+    struct Option {
+        const char* short_name;
+        const char* long_name;
+        int* number;
+        std::string* text;
+    };
+    const Option options[] = {
+        {"-m", "--m", &M, nullptr},          {"-n", "--n", &N, nullptr},
+        {"-k", "--k", &K, nullptr},          {"-b", "--b", &batch, nullptr},
+        {"-v", "--verify", &verify, nullptr}, {nullptr, "--scale-mode", nullptr, &scale_mode},
+        {nullptr, "--seed", &seed, nullptr}, {nullptr, "--rotate-buffers", &rotate, nullptr},
+        {nullptr, "--iters", &iters, nullptr}, {nullptr, "--warmup", &warmup, nullptr},
     };
     for (int i = 1; i < argc; ++i) {
-        const char* arg = argv[i];
-        const char* val = nullptr;
-        auto take = [&](const char* short_flag, const char* long_flag) -> const char* {
-            if ((val = parse_val(arg, short_flag)) || (long_flag && (val = parse_val(arg, long_flag)))) {
-                if (val == reinterpret_cast<const char*>(1)) return i + 1 < argc ? argv[++i] : "";
-                return val;
-            }
-            return nullptr;
-        };
-        const char* v;
-        if ((v = take("-m", "--m"))) { M = atoi(v); continue; }
-        if ((v = take("-n", "--n"))) { N = atoi(v); continue; }
-        if ((v = take("-k", "--k"))) { K = atoi(v); continue; }
-        if ((v = take("-b", "--b"))) { batch = atoi(v); continue; }
-        if ((v = take("-v", "--verify"))) { verify = atoi(v); continue; }
-        if ((v = take("--scale-mode", nullptr))) { scale_mode = v; continue; }
-        if ((v = take("--seed", nullptr))) { seed = atoi(v); continue; }
-        if ((v = take("--rotate-buffers", nullptr))) { rotate = atoi(v); continue; }
+        const std::string arg = argv[i];
+        const size_t eq = arg.find('=');
+        const std::string name = arg.substr(0, eq);
+        for (const Option& o : options) {
+            if (!((o.short_name && name == o.short_name) || (o.long_name && name == o.long_name))) continue;
+            std::string value;
+            if (eq != std::string::npos) value = arg.substr(eq + 1);
+            else if (i + 1 < argc) value = argv[++i];
+            if (o.number) *o.number = atoi(value.c_str());
+            else *o.text = value;
+            break;
+        }
     }
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) {
         fprintf(stderr, "Invalid problem size: M, N, K and batch must be positive.\n");
+        return 1;
+    }
+    if (iters <= 0 || warmup < 0) {
+        fprintf(stderr, "--iters must be positive and --warmup non-negative.\n");
         return 1;
     }
     int mode = A8W8_SCALE_ROWCOL;
@@ -218,6 +240,7 @@ int main(int argc, char** argv)
     }
     if (HARNESS_KIND == 2 && batch != 1) { fprintf(stderr, "flatmm harness runs batch 1\n"); return 1; }
 
+    CHECK_A8W8(a8w8_init(-1));      // device set-up outside the timed loop
     Rng rng((uint64_t)seed);
     const size_t a_elems = (size_t)batch * M * K, b_elems = (size_t)batch * N * K, c_elems = (size_t)batch * M * N;
     std::vector<uint8_t> host_a(a_elems), host_b(b_elems);
@@ -352,7 +375,7 @@ int main(int argc, char** argv)
     }
 
     printf("\n");
-    const float avg_time = benchmark(launch);
+    const float avg_time = benchmark(launch, warmup, iters);
     const double flop = 2.0 * M * N * K * batch;
     printf("Kernel Performance: avg_time=%.4f ms, %.2f TFlops\n", avg_time, flop / 1.0e9 / avg_time);
     const double bytes = (double)a_elems + b_elems + c_bytes;

@@ -18,7 +18,7 @@ def test_every_declared_symbol_is_exported():
     text = open(os.path.join(ROOT, "include", "mi355_a8w8.h")).read()
     names = set(re.findall(r"A8W8_API\s+[\w\s\*]+?\b(a8w8_\w+)\s*\(", text))
     assert {"a8w8_gemm", "a8w8_gemm_blockscale", "a8w8_flatmm", "a8w8_preshuffle_b", "a8w8_cvt_f32_to_e4m3",
-            "a8w8_cvt_e4m3_to_f32", "a8w8_status_string"} <= names
+            "a8w8_cvt_e4m3_to_f32", "a8w8_status_string", "a8w8_init"} <= names
     L = ctypes.CDLL(g.library_path())
     for n in names:
         assert hasattr(L, n), n
@@ -115,7 +115,11 @@ def test_kernel_selection():
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, **big)) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(mode=g.TENSOR, k=1024, **big)) == "gemm_a8w8_wide"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=384, **big)) == "gemm_a8w8_persist"
-    assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=128, **big)) == "gemm_a8w8_tile256"
+    # a single K step: the 128-tile kernel at any size (the pipelined kernels stage two steps ahead)
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL, k=128, **big)) == "gemm_a8w8_tile128"
+    # row strides of 2^23 bytes and more keep their kernel (row offsets are full 32-bit products)
+    assert g.kernel_name(_ok_args(mode=g.ROWCOL, m=512, n=16, k=256, stride_b=1 << 23)) == "gemm_a8w8_tile128"
+    assert g.lib().a8w8_gemm(ctypes.byref(_ok_args(mode=g.ROWCOL, m=4096, n=512, k=256, stride_b=1 << 23)), None) == -7   # 2 GiB span
     # every scale mode: 128 x 128 tiles while all of them fit on the chip at once (two workgroups per compute unit)
     assert g.kernel_name(_ok_args()) == "gemm_a8w8_tile128"
     assert g.kernel_name(_ok_args(mode=g.ROWCOL, m=1024, n=2048, k=128)) == "gemm_a8w8_tile128"
@@ -227,10 +231,15 @@ def test_sibling_entry_points_reject_bad_arguments():
     assert L.a4w4_quantize_mx(0x1000, 4, 48, 48, 0x2000, 0x3000, 0, None) == -3
     assert L.a4w4_quantize_mx(0x1000, 4, 64, 32, 0x2000, 0x3000, 0, None) == -4
     assert L.a4w4_quantize_mx(0x1000, 4, 64, 64, 0x2000, 0x3002, 1, None) == -5
-    # conversions return the number of elements converted: nothing on bad arguments
-    assert L.a8w8_cvt_f32_to_e4m3(None, 0x2000, 16, g.OCP, 0, None) == 0
-    assert L.a8w8_cvt_f32_to_e4m3(0x1000, 0x2000, 16, 5, 0, None) == 0
-    assert L.a8w8_cvt_e4m3_to_f32(0x1000, None, 16, g.OCP, None) == 0
+    # conversions return a status like every other entry point; zero elements is a no-op, not an error
+    assert L.a8w8_cvt_f32_to_e4m3(None, 0x2000, 16, g.OCP, 0, None) == -1
+    assert L.a8w8_cvt_f32_to_e4m3(0x1000, 0x2000, 16, 5, 0, None) == -6
+    assert L.a8w8_cvt_e4m3_to_f32(0x1000, None, 16, g.OCP, None) == -1
+    assert L.a8w8_cvt_e4m3_to_f32(0x1000, 0x2000, 16, 2, None) == -6
+    assert L.a8w8_cvt_f32_to_e4m3(None, None, 0, g.OCP, 0, None) == 0
+    assert L.a8w8_cvt_e4m3_to_f32(None, None, 0, g.FNUZ, None) == 0
+    # block scales: the A-side scale offsets of all K groups have to fit 32 bits
+    assert L.a8w8_gemm(ctypes.byref(_ok_args(mode=g.BLOCK, m=256, n=256, k=1024, stride_sfa=1 << 27)), None) == -7
     assert L.a8w8_preshuffle_b_device(0x1000, 0x2000, 40, 192, None) == -3
     assert L.a8w8_preshuffle_b_device(0x1000, 0x2004, 48, 192, None) == -5
 
@@ -241,6 +250,32 @@ def test_good_arguments_pass_validation_and_stop_at_the_device():
         pytest.skip("GPU present: the call would launch")
     assert g.lib().a8w8_gemm(ctypes.byref(_ok_args()), None) == -9
     assert "gfx950" in g.status_string(-9)
+
+
+def test_header_states_the_tiled_scale_layout(orc):
+    """The byte position include/mi355_a8w8.h gives for the exponent of (row r, 32-block kb) in the MX_TILED layout,
+    evaluated as written, is where the oracle's layout walk puts it (ragged row and K counts included)."""
+    text = open(os.path.join(ROOT, "include", "mi355_a8w8.h")).read()
+    m = re.search(r"the exponent of \(row r, block kb\) is byte\s*\*\s*(.+?)\n\s*\*\s*(.+?)\n\s*\*\s*\(pair =", text, re.S)
+    assert m, "the header no longer states the formula in the expected place"
+    formula = (m.group(1) + " " + m.group(2)).replace("ceil(rows/64)", "((rows + 63) // 64)")
+    formula = re.sub(r"(?<![/])/(?![/])", "//", formula)
+    size = re.search(r"ceil\(k/512\) \* ceil\(rows/64\) \* 1024 bytes", text)
+    assert size, "the header no longer states the size"
+    for rows, k in ((64, 512), (200, 1600), (130, 96), (1, 32)):
+        kb_n = k // 32
+        rng = np.random.Generator(np.random.Philox(rows))
+        sf = rng.integers(0, 255, (rows, kb_n)).astype(np.uint8)
+        tiled = orc.mx_tile_scales(sf)
+        assert tiled.size == ((k + 511) // 512) * ((rows + 63) // 64) * 1024 == g.lib().a8w8_mx_tiled_bytes(rows, k)
+        seen = np.zeros(tiled.size, bool)
+        for r in range(rows):
+            rr = r % 64
+            for kb in range(kb_n):
+                pos = eval(formula, {"rows": rows, "r": r, "rr": rr, "kb": kb})
+                assert tiled[pos] == sf[r, kb], (rows, k, r, kb, pos)
+                seen[pos] = True
+        assert (tiled[~seen] == 127).all()
 
 
 def test_host_preshuffle_matches_oracle(orc):

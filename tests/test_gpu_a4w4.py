@@ -91,7 +91,7 @@ def test_full_size_8192(orc):
     c = g.gemm_a4w4(qa, qb, ta, tb)
     ref = orc.gemm_ref_mxfp4(qa[:8].cpu().numpy(), qb.cpu().numpy(), ea.cpu().numpy(), eb.cpu().numpy())
     got = c[:8].float().cpu().numpy()
-    assert (np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-2).mean() >= 0.999
+    assert (np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-2).all()
     np.testing.assert_allclose(got, ref, rtol=2e-2, atol=2e-2 * np.abs(ref).max())
     # permuting the rows of A (with their scales) permutes the rows of C bit for bit
     perm = torch.randperm(m, generator=torch.Generator().manual_seed(3)).cuda()

@@ -7,7 +7,7 @@ import torch
 
 import datagen
 import gcnasm_amd as g
-from gpu_util import MFMA_ACC_ERR, dev
+from gpu_util import MFMA_ACC_ERR, assert_close, dev, exact64
 
 pytestmark = pytest.mark.gpu
 
@@ -111,5 +111,10 @@ def test_batched_persistent(orc, mode):
     c = g.gemm(dev(a), dev(b), dev(sa), dev(sb), mode, c_dtype=g.FP32).cpu().numpy()
     for i in range(batch):
         ref = orc.gemm_ref(a[i], b[i], sa[i], sb[i], mode)
-        assert (np.abs(c[i] - ref) <= 1e-2 * np.abs(ref) + 1e-2).mean() >= 0.999
+        if mode == g.MX:
+            # wide-range inputs: outputs that cancel to almost zero are judged against float64 (gpu_util.assert_close)
+            exact, mag = exact64(orc, a[i], b[i], sa[i], sb[i], mode)
+            assert_close(c[i], ref, f"batch entry {i}", exact=exact, mag=mag)
+        else:
+            assert datagen.tolerance_ok(c[i], ref).all(), i
         np.testing.assert_allclose(c[i], ref, rtol=2e-3, atol=2e-3 * np.abs(ref).max())

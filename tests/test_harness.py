@@ -54,3 +54,21 @@ def test_flatmm_program():
     r = _run("flatmm_a8w8.exe", "-m", "16", "-n", "2048", "-k", "1024", "-v", "1")
     assert r.returncode == 0, r.stdout + r.stderr
     assert "[Overall] ALL BATCHES VALID" in r.stdout and "Kernel Performance:" in r.stdout
+
+
+@pytest.mark.gpu
+def test_iteration_flags():
+    r = _run("gemm_a8w8_8wave.exe", "-m", "256", "-n", "256", "-k", "256", "--iters", "3", "--warmup=2")
+    assert r.returncode == 0 and "Kernel Performance:" in r.stdout, r.stdout + r.stderr
+    r = _run("gemm_a8w8_8wave.exe", "--iters", "0")
+    assert r.returncode == 1 and "--iters must be positive" in r.stderr
+
+
+@pytest.mark.gpu
+def test_buffer_range_check_covers_the_scalar_offset():
+    """The kernels move between row groups with the scalar offset of their buffer loads and rely on rows past the
+    end of a matrix reading as zero: the hardware's range check has to include that offset (measured on the device,
+    every address inside one live allocation)."""
+    r = _run("buffer_bounds_probe.exe")
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count(" ok\n") == 5 and "UNEXPECTED" not in r.stdout

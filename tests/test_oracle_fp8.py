@@ -141,6 +141,37 @@ def test_cvt_fp8_clamp240(orc):
     assert (orc.encode(x, orc.OCP, clamp240=True) == orc.encode(x, orc.OCP)).all()
 
 
+def test_hardware_convert_matches_the_gfx950_record(orc):
+    """orc_e4m3_ocp_encode_hw / orc_cvt_fp8_clamp240 against what the instruction returned on a gfx950
+    device for NaN, Inf and out-of-range inputs (tests/golden/gfx950_cvt_pk_fp8_specials.txt)."""
+    rows = _load("gfx950_cvt_pk_fp8_specials.txt")
+    x = np.array([r[0] for r in rows], np.uint32).view(np.float32)
+    got = orc.convert(x, orc.OCP)
+    bad = [(hex(r[0]), hex(g_), hex(r[1])) for r, g_ in zip(rows, got) if g_ != r[1]]
+    assert not bad, bad
+    got = orc.encode(x, orc.OCP, clamp240=True)
+    bad = [(hex(r[0]), hex(g_), hex(r[2])) for r, g_ in zip(rows, got) if g_ != r[2]]
+    assert not bad, bad
+
+
+def test_hardware_convert_is_the_saturating_one_where_nothing_overflows(orc):
+    """Non-saturating and saturating conversions differ only for NaN and for magnitudes that round
+    beyond 448: everywhere else the hip_fp8.h fixture pins both."""
+    rows = _load("hip_fp8_encode.txt")
+    x = np.array([r[0] for r in rows], np.uint32).view(np.float32)
+    want = np.array([r[1] for r in rows], np.uint8)
+    got = orc.convert(x, orc.OCP)
+    with np.errstate(invalid="ignore"):
+        over = np.isnan(x) | (np.abs(x) > 464.0)
+    assert (got[~over] == want[~over]).all()
+    assert over.sum() > 10
+    sign = (x.view(np.uint32) >> 31).astype(np.uint8) << 7
+    assert (got[over & ~np.isnan(x)] == (sign | 0x7F)[over & ~np.isnan(x)]).all()     # overflow, Inf: the NaN code, signed
+    assert (got[np.isnan(x)] == 0xFF).all()
+    # FNUZ: the saturating conversion of __hip_fp8_e4m3_fnuz throughout
+    assert (orc.convert(x, orc.FNUZ) == np.array([r[2] for r in rows], np.uint8)).all()
+
+
 def test_pk_cvt_byte_order(orc):
     """bytes come out as [f8(s0), f8(s1), f8(s2), f8(s3)] (perm selector 0x05040100)."""
     for base in range(-128, 124, 4):   # the harness sweep i - pixels/2, pk_cvt/test.cpp:441-443
