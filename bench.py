@@ -12,8 +12,12 @@ quantiser can emit them) and the one-launch path on row-major scales are timed b
 The other configurations and the M=16 flatmm are timed afterwards and reported in the same
 JSON line under "other_workloads".
 Timing uses HIP events recorded on the stream the kernels are launched on, W untimed
-warm-up launches, then exactly K timed launches.  The CPU baseline is the oracle (a port
-of the reference's host GEMM) timed on a bounded slab of the same problem.
+warm-up launches, then exactly K timed launches.  The chip's clocks take a few hundred
+milliseconds of load to settle, so every timed workload is preceded by a time-based run of
+the same launches that is counted neither in W nor in K; for the headline workload the same
+W + K protocol is also run once before that, on the cold chip, and reported beside the
+steady number ("first_region").  The CPU baseline is the oracle (a port of the reference's
+host GEMM) timed on a bounded slab of each configuration.
 """
 import argparse
 import json
@@ -29,9 +33,24 @@ PEAK_FP8_TFLOPS = 5000.0      # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E, published
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA, published
 PEAK_FP4_TFLOPS = 10100.0     # MI355X dense FP4 MFMA, published
-# Bytes that crossed the L2 <-> fabric boundary per launch, from two rocprofv3 --pmc runs of this file
-# (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a 117 MB device copy calibrates; profiles/).
-MEASURED_TRAFFIC = {"mxfp8_8192": 1.08e9, "flatmm_16x16384x7168": 1.190e8}
+
+
+def measured_traffic():
+    """Bytes that crossed the L2 <-> fabric boundary per launch of each workload's dominant kernel, as the tracked
+    summary of the two rocprofv3 --pmc runs of this file states them (FETCH_SIZE and WRITE_SIZE, each scaled by what
+    the counter reads for a device copy of known size); None for a workload the summary does not list."""
+    import re
+    path = os.path.join(ROOT, "profiles", "traffic_fetch_write.md")
+    out = {}
+    try:
+        for line in open(path):
+            m = re.match(r"\s*traffic_bytes_per_launch\s+(\S+)\s*=\s*([0-9.eE+]+)", line)
+            if m:
+                out[m.group(1)] = float(m.group(2))
+    except OSError:
+        pass
+    return out
+
 
 WORKLOADS = {
     # name: (mode, m, n, k, algorithmic bytes per launch)
@@ -107,14 +126,31 @@ def time_launches(torch, fn, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall_ms / steps
 
 
+CONDITION_S = 0.5      # load applied before a timed region, counted in neither W nor K
+
+
+def condition_clocks(torch, fn, seconds=CONDITION_S):
+    """Runs the workload's own launches for `seconds` of wall time so that the timed region that follows sees
+    the clocks the chip sustains under this load rather than the ramp from idle."""
+    t0 = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
+
+
+def time_steady(torch, fn, steps, warmup):
+    """The headline protocol: conditioning, then W warm-up launches and exactly K timed ones."""
+    condition_clocks(torch, fn)
+    return time_launches(torch, fn, steps, warmup)
+
+
 def time_best_of(torch, fn, steps, warmup, rounds=3):
     """For the secondary workloads: bring the clocks up with at least 100 ms of warm-up launches,
     then report the best of `rounds` timed regions of `steps` launches each."""
-    t0 = time.perf_counter()
-    while time.perf_counter() - t0 < 0.1:
-        for _ in range(20):
-            fn(0)
-        torch.cuda.synchronize()
+    condition_clocks(torch, fn, 0.1)
     best = None
     for _ in range(rounds):
         r = time_launches(torch, fn, steps, warmup)
@@ -153,12 +189,46 @@ def run_workload(name, torch, g, steps, warmup, seed, headline=True):
             if L.a8w8_flatmm(flat_args[0], stream) != 0:
                 raise RuntimeError("a8w8_flatmm failed")
 
-        timer = time_launches if headline else time_best_of
+        timer = time_steady if headline else time_best_of
         ms, wall = timer(torch, fn_rot, steps, warmup)
         ms_same, _ = timer(torch, fn_same, steps, warmup)
         res.update(ms_per_launch=ms, wall_ms_per_launch=wall, gbs=abytes / ms / 1e6, gbs_same_buffer=abytes / ms_same / 1e6,
                    tflops=flops / ms / 1e9, frac_hbm_peak=abytes / ms / 1e6 / PEAK_HBM_GBS,
                    note="four rotating copies of B (470 MB) defeat the 256 MB Infinity Cache; gbs_same_buffer re-reads one copy")
+        # the same launches replayed from one HIP graph: what is left of the gap between back-to-back launches
+        graph_steps = 64
+        side = torch.cuda.Stream()
+        side_stream = ctypes.c_void_p(side.cuda_stream)
+        with torch.cuda.stream(side):
+            for i in range(4):
+                L.a8w8_flatmm(flat_args[i], side_stream)
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                cap = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for i in range(graph_steps):
+                    if L.a8w8_flatmm(flat_args[i & 3], cap) != 0:
+                        raise RuntimeError("a8w8_flatmm failed under capture")
+        ms_graph, _ = time_best_of(torch, lambda i: graph.replay(), max(2, steps // 16), 2)
+        ms_graph /= graph_steps
+        res.update(ms_per_launch_in_graph=ms_graph, gbs_in_graph=abytes / ms_graph / 1e6,
+                   frac_hbm_peak_in_graph=abytes / ms_graph / 1e6 / PEAK_HBM_GBS,
+                   graph_note=f"{graph_steps} launches (rotating B) captured in one HIP graph and replayed")
+        # yardstick: what a kernel that only reads the same rotating buffers gets on this box
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        probe_args = [(ctypes.c_void_p(x.data_ptr()), x.numel()) for x in copies]
+
+        def fn_probe(i):
+            ptr, nbytes = probe_args[i & 3]
+            if L.a8w8_hbm_read_probe(ptr, nbytes, ctypes.c_void_p(sink.data_ptr()), stream) != 0:
+                raise RuntimeError("a8w8_hbm_read_probe failed")
+
+        ms_probe, _ = time_best_of(torch, fn_probe, steps, warmup)
+        wbytes = copies[0].numel()
+        res.update(achievable_read_gbs=wbytes / ms_probe / 1e6, achievable_read_ms=ms_probe,
+                   frac_of_achievable_read=(abytes / ms) / (wbytes / ms_probe),
+                   achievable_note="a8w8_hbm_read_probe: 16-byte non-temporal loads over the same four weight buffers, nothing else "
+                                   "(after the reference's bandwidth_memread)")
         fn = fn_rot
     else:
         gemm_args = args_for(inp["b"], 0)
@@ -171,7 +241,7 @@ def run_workload(name, torch, g, steps, warmup, seed, headline=True):
                 raise RuntimeError("gemm call failed")
 
         fn = fn_direct
-        timer = time_launches if headline else time_best_of
+        timer = time_steady if headline else time_best_of
         if mode == "mx":
             # row-major scales in, tiled scales for the kernel: two re-ordering launches + the GEMM
             ta = torch.empty(g.mx_tiled_bytes(m, k), dtype=torch.uint8, device="cuda")
@@ -191,6 +261,10 @@ def run_workload(name, torch, g, steps, warmup, seed, headline=True):
                     raise RuntimeError("a8w8_mx_tile_scales_ab / a8w8_gemm failed")
 
             res["kernel"] = g.kernel_name(tiled_args)
+            if headline:
+                # the same protocol on the chip as it is found (idle clocks), reported beside the steady number
+                first_ms, _ = time_launches(torch, fn, steps, warmup)
+                res.update(first_region_ms_per_step=first_ms, first_region_tflops=flops / first_ms / 1e9)
             ms, wall = timer(torch, fn, steps, warmup)
             ms_gemm, _ = timer(torch, fn_gemm_only, steps, warmup)
             ms_direct, _ = timer(torch, fn_direct, steps, warmup)
@@ -244,10 +318,10 @@ def run_quantizers(torch, g, steps, warmup, seed):
 
 
 # What the reference publishes for its own block-scale program (fp32 C, A~U[0,1), B~U[-.5,.5), scales~U[.8,1.2);
-# opus_gemm/block_scale_gemm/README.md:111-114) and as the expected output of its flat program
+# opus_gemm/block_scale_gemm/README.md:111-115) and as the expected output of its flat program
 # (opus_fmm/README.md:43-49, 2*16*4096*4096 flops), on MI355X.
 REFERENCE_PUBLISHED = {"block_fp32_1024": 118.96, "block_fp32_2048": 616.77, "block_fp32_4096": 2237.77, "block_fp32_8192": 2710.24,
-                       "flatmm_16x4096x4096": 20.64}
+                       "block_fp32_16384": 2686.87, "flatmm_16x4096x4096": 20.64}
 
 
 def run_reference_program_sizes(torch, g, steps, warmup, seed):
@@ -260,13 +334,16 @@ def run_reference_program_sizes(torch, g, steps, warmup, seed):
         return torch.rand(shape, generator=gen, device="cuda", dtype=torch.float32) * (hi - lo) + lo
 
     out = []
-    for size in (1024, 2048, 4096, 8192):
+    for size in (1024, 2048, 4096, 8192, 16384):
         m = n = k = size
         a = g.cvt_f32_to_e4m3(uniform((m, k), 0.0, 1.0))
+        torch.cuda.empty_cache()
         b = g.cvt_f32_to_e4m3(uniform((n, k), -0.5, 0.5))
+        torch.cuda.empty_cache()
         sfa, sfb = uniform((k // 128, m), 0.8, 1.2), uniform((n // 128, k // 128), 0.8, 1.2)
         c = torch.empty((m, n), dtype=torch.float32, device="cuda")
-        ms, wall = time_best_of(torch, lambda i: g.gemm_blockscale(a, b, sfa, sfb, c=c), steps, warmup)
+        big_steps = steps if size < 16384 else max(5, steps // 5)      # 3.5 ms a launch: fewer of them
+        ms, wall = time_best_of(torch, lambda i: g.gemm_blockscale(a, b, sfa, sfb, c=c), big_steps, min(warmup, big_steps))
         name = f"block_fp32_{size}"
         tf = 2.0 * m * n * k / ms / 1e9
         out.append({"workload": name, "m": m, "n": n, "k": k, "kernel": g.kernel_name(g.raw_gemm_args(
@@ -350,10 +427,11 @@ def run_flat_variants(torch, g, steps, warmup, seed):
     return out
 
 
-def cpu_baseline(name, inp, c_gpu, torch, budget_s=15.0):
+def cpu_baseline(name, inp, c_gpu, torch, budget_s=15.0, max_rows=256):
     """Times the oracle (port of the reference's host GEMM: per-MAC software fp8 decode,
     OpenMP over (i, j), gemm_a8w8_blockscale_host.cc:66-90) on the first rows of the same
-    problem, sized to about budget_s seconds, and checks the GPU result on that slab."""
+    problem -- as many as about budget_s seconds allow, at most max_rows -- and checks the GPU
+    result on that slab.  A slab smaller than the problem is extrapolated linearly and says so."""
     import numpy as np
     import oracle
     mode, m, n, k, _ = WORKLOADS[name]
@@ -366,17 +444,18 @@ def cpu_baseline(name, inp, c_gpu, torch, budget_s=15.0):
     t0 = time.perf_counter()
     oracle.gemm_ref(a, b, sfa, sfb, omode, rows=(0, 1), decode_per_mac=True)
     t_row = time.perf_counter() - t0
-    rows = int(max(1, min(m, 256, budget_s / max(t_row, 1e-4))))
+    rows = int(max(1, min(m, max_rows, budget_s / max(t_row, 1e-4))))
     t0 = time.perf_counter()
     ref = oracle.gemm_ref(a, b, sfa, sfb, omode, rows=(0, rows), decode_per_mac=True)
     dt = time.perf_counter() - t0
     got = c_gpu[:rows].float().cpu().numpy()
     ok = np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-2
+    whole = rows == m
+    sample = (f"the whole problem ({m} rows of C), {dt:.2f} s" if whole else
+              f"first {rows} of {m} rows of C (all N, all K), {dt:.2f} s; full problem extrapolates linearly to {dt * m / rows:.0f} s")
     return {
         "value": 2.0 * rows * n * k / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
-        "sample": f"first {rows} of {m} rows of C (all N, all K), {dt:.2f} s; full problem extrapolates to "
-                  f"{dt * m / rows:.0f} s",
-        "gpu_slab_within_tolerance": float(ok.mean()),
+        "sample": sample, "extrapolated": not whole, "gpu_slab_within_tolerance": float(ok.mean()),
     }
 
 
@@ -405,13 +484,13 @@ def main():
     if mode == "flat":
         value, unit = res["gbs"], "GB/s"
         roof = {"bound": "hbm", "achieved": res["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": res["gbs"] / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC.get(args.workload), "kernel": "flatmm_a8w8"}
+                "frac": res["gbs"] / PEAK_HBM_GBS, "traffic": measured_traffic().get(args.workload), "kernel": "flatmm_a8w8"}
     else:
         value, unit = res["tflops"], "TFLOP/s"
         # the dominant kernel alone (for MX: the GEMM launch without the two scale re-ordering launches)
         kern_tflops = res.get("tflops_gemm_kernel", res["tflops"])
         roof = {"bound": "mfma", "achieved": kern_tflops, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                "frac": kern_tflops / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC.get(args.workload),
+                "frac": kern_tflops / PEAK_FP8_TFLOPS, "traffic": measured_traffic().get(args.workload),
                 "kernel": res.get("kernel")}
     line = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -422,9 +501,12 @@ def main():
         "roofline": roof,
     }
     for key in ("step", "ms_gemm_kernel", "tflops_gemm_kernel", "ms_row_major_scales_one_launch",
-                "tflops_row_major_scales_one_launch"):
+                "tflops_row_major_scales_one_launch", "first_region_ms_per_step", "first_region_tflops"):
         if key in res:
             line["config"][key] = res[key]
+    line["config"]["timing"] = (f"{CONDITION_S} s of the same launches (counted in neither W nor K) bring the clocks to what the chip "
+                                "sustains, then W warm-up and K timed launches between two HIP events on the launch stream; "
+                                "first_region_* is the same W + K protocol run before that on the chip as found")
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.workload, inp, c, torch)
     del inp, c
@@ -436,6 +518,9 @@ def main():
                 continue
             r, i2, c2 = run_workload(name, torch, g, args.steps, args.warmup, args.seed + 1, headline=False)
             r["timing"] = "best of 3 regions of K launches after 100 ms of warm-up"
+            if not args.no_cpu and WORKLOADS[name][0] not in ("bf16", "f4"):
+                # the two small configurations whole, the large ones on a 64-row slab
+                r["cpu_baseline"] = cpu_baseline(name, i2, c2, torch, budget_s=4.0, max_rows=WORKLOADS[name][1] if WORKLOADS[name][1] <= 256 else 64)
             others.append(r)
             del i2, c2
             torch.cuda.empty_cache()

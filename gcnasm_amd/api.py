@@ -98,6 +98,7 @@ def lib():
         L.a8w8_kernel_name.argtypes = [ctypes.POINTER(GemmArgs)]
         L.a8w8_version.restype = ctypes.c_int
         L.a8w8_init.argtypes = [ctypes.c_int]
+        L.a8w8_hbm_read_probe.argtypes = [vp, ctypes.c_size_t, vp, vp]
         _lib = L
     return _lib
 

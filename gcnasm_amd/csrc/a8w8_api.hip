@@ -15,6 +15,7 @@
 #include "gemm_persist.hpp"
 #include "gemm_small.hpp"
 #include "gemm_wide.hpp"
+#include "hbm_probe.hpp"
 
 using namespace a8w8;
 
@@ -1095,6 +1096,21 @@ const char* a8w8_kernel_name(const a8w8_gemm_args* g)
     if (small_ok(g)) return "gemm_a8w8_tile128";
     if (wide_ok(g)) return "gemm_a8w8_wide";
     return persist_ok(g) ? "gemm_a8w8_persist" : "gemm_a8w8_tile128";
+}
+
+int a8w8_hbm_read_probe(const void* src, size_t bytes, void* sink, void* hip_stream)
+{
+    if (!src || !sink) return A8W8_ERR_NULL_POINTER;
+    if (bytes == 0) return A8W8_ERR_BAD_SHAPE;
+    if (bytes % 16 != 0 || !aligned16(src) || ((uintptr_t)sink & 3)) return A8W8_ERR_MISALIGNED;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
+    const size_t n16 = bytes / 16;
+    // eight workgroups per compute unit, fewer for buffers that do not give each thread a full round of loads
+    const size_t want = (n16 + (size_t)HBM_PROBE_THREADS * HBM_PROBE_UNROLL - 1) / ((size_t)HBM_PROBE_THREADS * HBM_PROBE_UNROLL);
+    const size_t most = (size_t)num_cus() * 8;
+    const unsigned grid = (unsigned)(want < most ? (want ? want : 1) : most);
+    return launch(hbm_read_probe_kernel, dim3(grid), dim3(HBM_PROBE_THREADS), 0, (hipStream_t)hip_stream, (const v4i*)src, n16,
+                  (int*)sink);
 }
 
 int a8w8_init(int device)

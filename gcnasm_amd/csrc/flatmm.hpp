@@ -32,7 +32,10 @@ constexpr int FLAT_THREADS = FLAT_WAVES * 64;
 // ids to the 8 XCDs in turn, so they run on one XCD at the same time and all but the first find the weights in its L2.
 A8W8_DEV void flat_work_of_block(int bid, int n_groups, int m_tiles, int& n_group, int& m_tile)
 {
-    if ((n_groups & 7) == 0) {
+    if (m_tiles == 1) {      // the common case without its divisions: every cycle before the first load is a cycle of idle memory
+        m_tile = 0;
+        n_group = bid;
+    } else if ((n_groups & 7) == 0) {
         const int rest = bid >> 3;
         m_tile = rest % m_tiles;
         n_group = (rest / m_tiles) * 8 + (bid & 7);
@@ -83,6 +86,12 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
     const int batch = blockIdx.z;
     const int r16 = lane & 15, kq = lane >> 4;
 
+    // What the epilogue needs of the arguments is read now and kept in registers: left to itself the compiler fetches
+    // it from the argument block after the K loop, a scalar load that misses its cache at the one point where the
+    // whole workgroup waits for it.
+    int ldc = p.ldc;
+    long long c_batch_off = (long long)batch * p.c_batch;
+    asm volatile("" : "+s"(ldc), "+s"(c_batch_off));
     const int n_tiles = p.n >> 4;
     const int k_tiles = p.k >> 6;
     int n_group, m_tile_;
@@ -118,7 +127,8 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
             }
         }
     };
-    if constexpr (ROUNDS == 1) fetch_scales(0);      // with more rounds the registers are worth more than the head start
+    // (fetched once the first weight loads are under way; with more rounds than one the registers are worth more than
+    // the head start and the fetch waits until the K loop is over)
 
     // MT = 1: lane (r16, kq) reads bytes [16 kq, 16 kq + 16) of row r16 in each K block.
     // MT > 1: lane (row = lane / 4, c = lane % 4) reads bytes [32 c, 32 c + 32) of the pair's 128-byte line.
@@ -194,9 +204,9 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         blk_b = (const float*)p.sfb + (long long)batch * p.sfb_batch + (long long)(nt0 >> 3) * p.stride_sfb;
     }
 
-    // K blocks are consumed in pairs; wave w takes pairs w, w + 8, ...: at any moment the eight waves read 16 KiB in
-    // a row of each weight tile.  (Contiguous shares put the waves K/8 bytes apart, which for a power-of-two K
-    // lands all of them, in every workgroup, on the same few memory channels.)
+    // K blocks are consumed in pairs, eight consecutive pairs a round, one per wave: at any moment the eight waves
+    // read 16 KiB in a row of each weight tile.  (Contiguous shares put the waves K/8 bytes apart, which for a
+    // power-of-two K lands all of them, in every workgroup, on the same few memory channels.)
     const int pairs = (k_tiles + 1) >> 1;
     constexpr int PSTEP = FLAT_WAVES;
 
@@ -346,38 +356,49 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         }
     };
 
-    if (wave < pairs) {
+    {
         Frag f0, f1;
         constexpr bool STAGING = MT > 1 || BROW;
         auto load_staged = [&](int q) {
             if constexpr (MT > 1) load_rows(q);
             if constexpr (BROW) load_weight_rows(q);
         };
-        // This wave's pairs are wave, wave + 8, ...; it starts at one that depends on the workgroup and wraps around,
-        // so that workgroups running side by side are at different K offsets: with rows (or weight tiles) a power of
-        // two apart they would otherwise all sit on the same memory channels at any moment.
-        const int count = (pairs - wave + PSTEP - 1) / PSTEP;
-        // (the same for the workgroups of one group of weight tiles: those read the weights together, through L2)
-        int at = (n_group * 5) % count;
+        // Round j of the K walk covers pairs 8 j .. 8 j + 7, one per wave; the wave takes slot (wave + 3 j) % 8 of its
+        // round.  A fixed slot would advance every wave by exactly 16 KiB per round, and memory channels repeat with
+        // a period that divides 16 KiB: each wave would then sit on the same few channels for its whole life, all
+        // waves of all workgroups aliasing onto one another (16 x 16384 x 7168: 20.0 us with fixed slots, 18.9 us
+        // rotating).  The wave starts at a round that depends on the workgroup and wraps around, so that workgroups
+        // running side by side are at different K offsets as well: with rows (or weight tiles) a power of two apart
+        // they would otherwise all sit on the same memory channels at any moment.
+        const int rounds = (pairs + PSTEP - 1) / PSTEP;
+        auto pair_of = [&](int j) { return ((wave + 3 * j) & (PSTEP - 1)) + PSTEP * j; };
+        // the last round may be partial: this wave has a pair in it only if its slot there exists
+        const int count = pair_of(rounds - 1) < pairs ? rounds : rounds - 1;
+        // (the same start for the workgroups of one group of weight tiles: those read the weights together, through L2)
+        // (a multiplicative hash of the group index scaled into [0, count): no division in front of the first load)
+        int at = (int)((((uint32_t)n_group * 40503u) & 0xffffu) * (uint32_t)count >> 16);
         auto next_of = [&](int j) { return j + 1 == count ? 0 : j + 1; };
         int left = count;
-        load_staged(wave + PSTEP * at);
-        load(wave + PSTEP * at, f0);
+        if (count > 0) {
+            load_staged(pair_of(at));
+            load(pair_of(at), f0);
+        }
+        if constexpr (ROUNDS == 1) fetch_scales(0);
         // two register stages, loads of the next pair in flight while the current one is used
-        while (true) {
+        while (left > 0) {
             if constexpr (STAGING) stage_rows();
             at = next_of(at);
             if (left > 1) {
-                load_staged(wave + PSTEP * at);
-                load(wave + PSTEP * at, f1);
+                load_staged(pair_of(at));
+                load(pair_of(at), f1);
             }
             mma(f0);
             if (--left == 0) break;
             if constexpr (STAGING) stage_rows();
             at = next_of(at);
             if (left > 1) {
-                load_staged(wave + PSTEP * at);
-                load(wave + PSTEP * at, f0);
+                load_staged(pair_of(at));
+                load(pair_of(at), f0);
             }
             mma(f1);
             if (--left == 0) break;
@@ -403,10 +424,10 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
 #pragma unroll
             for (int w = 1; w < FLAT_WAVES; ++w) s += red[(w * PER_ROUND + wave) * 64 + lane];
             s *= sb[r] * sa[r];
-            const long long ci = (long long)batch * p.c_batch + (long long)cm[r] * p.ldc + cn[r];
+            const long long ci = c_batch_off + (long long)cm[r] * ldc + cn[r];
             if constexpr (CDT == C_BF16) {
                 unsigned short* dst = (unsigned short*)p.c + ci;
-                if ((p.ldc & 3) == 0 && (((uintptr_t)p.c + 2 * (long long)batch * p.c_batch) & 7) == 0) {
+                if ((ldc & 3) == 0 && (((uintptr_t)p.c + 2 * c_batch_off) & 7) == 0) {
                     *(v4u16*)dst = v4u16{bf16_bits(s.x), bf16_bits(s.y), bf16_bits(s.z), bf16_bits(s.w)};
                 } else {
 #pragma unroll

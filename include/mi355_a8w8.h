@@ -243,6 +243,13 @@ A8W8_API const char* a8w8_status_string(int status);
  * (for logs and profiles); NULL if the arguments are rejected. */
 A8W8_API const char* a8w8_kernel_name(const a8w8_gemm_args* args);
 
+/* Measurement aid, not part of the GEMM path: reads `bytes` of device memory once with 16-byte non-temporal loads
+ * from a grid sized to the machine and discards the values (`sink_dev`, 4 bytes, is never written for ordinary
+ * data).  bytes / its launch time is the read bandwidth this device actually gives a streaming kernel -- the
+ * yardstick beside the published HBM peak for a8w8_flatmm, after the reference's own
+ * bandwidth_memread/bandwidth_kernel.cu:68-92.  bytes % 16 == 0, src_dev 16-byte aligned. */
+A8W8_API int a8w8_hbm_read_probe(const void* src_dev, size_t bytes, void* sink_dev, void* hip_stream);
+
 /* Optional explicit set-up of one device (device < 0: the current one): queries its architecture and
  * compute-unit count and raises the dynamic-LDS limit of every kernel variant.  The same work happens,
  * once per device and thread-safely, inside the first entry point called with that device current; call
