@@ -1105,10 +1105,11 @@ int a8w8_hbm_read_probe(const void* src, size_t bytes, void* sink, void* hip_str
     if (bytes % 16 != 0 || !aligned16(src) || ((uintptr_t)sink & 3)) return A8W8_ERR_MISALIGNED;
     if (const int ds = device_status(); ds != A8W8_OK) return ds;
     const size_t n16 = bytes / 16;
-    // eight workgroups per compute unit, fewer for buffers that do not give each thread a full round of loads
-    const size_t want = (n16 + (size_t)HBM_PROBE_THREADS * HBM_PROBE_UNROLL - 1) / ((size_t)HBM_PROBE_THREADS * HBM_PROBE_UNROLL);
+    // eight workgroups per compute unit (the best of the grids tried on a 117 MB buffer), fewer for buffers that do not
+    // give every thread a load
+    const size_t want = (n16 + HBM_PROBE_THREADS - 1) / HBM_PROBE_THREADS;
     const size_t most = (size_t)num_cus() * 8;
-    const unsigned grid = (unsigned)(want < most ? (want ? want : 1) : most);
+    const unsigned grid = (unsigned)(want < most ? want : most);
     return launch(hbm_read_probe_kernel, dim3(grid), dim3(HBM_PROBE_THREADS), 0, (hipStream_t)hip_stream, (const v4i*)src, n16,
                   (int*)sink);
 }

@@ -10,7 +10,7 @@
 namespace a8w8 {
 
 constexpr int HBM_PROBE_THREADS = 256;
-constexpr int HBM_PROBE_UNROLL = 8;
+constexpr int HBM_PROBE_UNROLL = 16;     // with eight workgroups per compute unit the best of the configurations tried (unroll 4 / 8 / 16, 1 .. 64 workgroups per compute unit)
 
 __global__ void __launch_bounds__(HBM_PROBE_THREADS) hbm_read_probe_kernel(const v4i* src, size_t n16, int* sink)
 {
