@@ -143,6 +143,8 @@ int validate_common(const a8w8_gemm_args* g)
     if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128 && (long long)(g->k / 128) * g->stride_sfa * 4 >= (1ll << 31))
         return A8W8_ERR_TOO_LARGE;
     if ((long long)((g->m + 127) / 128) * ((g->n + 127) / 128) >= (1ll << 31)) return A8W8_ERR_TOO_LARGE;
+    // ... and the 256 rows of a C tile (stride_c below 4 Mi elements)
+    if ((long long)(BM - 1) * g->stride_c * 4 + BN * 4 >= (1ll << 32)) return A8W8_ERR_TOO_LARGE;
     return A8W8_OK;
 }
 

@@ -325,6 +325,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         // a tile that lies inside the matrix and takes 16-byte stores is written without per-lane checks (the
         // checked path spends more instructions on masks and branches than on stores)
         const bool whole = vec_ok && m0 + BM <= p.m && n0 + BN <= p.n;
+        // such a tile goes out through a buffer descriptor over its own rows (store_c_16), with 32-bit offsets
+        constexpr int C_ES = CDT == C_BF16 ? 2 : 4;
+        const __amdgpu_buffer_rsrc_t tile_rs =
+            make_rsrc(c_base + ((long long)m0 * p.ldc + n0) * C_ES, (uint32_t)((BM - 1) * p.ldc + BN) * C_ES);
+        const int tile_lane_off = ((wave_m * WAVE_M + r16) * p.ldc + wave_n * WAVE_N + 8 * g) * C_ES;
+        const int tile_row16 = 16 * p.ldc * C_ES;
 #pragma unroll
         for (int jp = 0; jp < TN / 2; ++jp) {
             const int cn = cn_base + 32 * jp;
@@ -339,16 +345,17 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                     if constexpr (MODE == MODE_ROWCOL) v[e] *= sb[jp][e] * sa[i];
                 }
                 if (whole) {
+                    // lane offset + 32 jp columns (an immediate) | 16 i rows (a scalar)
+                    const int voff = tile_lane_off + 32 * jp * C_ES, soff = i * tile_row16;
                     if constexpr (CDT == C_BF16) {
                         v4i w;
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                             w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
-                        A8W8_STORE_C((v4i*)((unsigned short*)c_base + (long long)cm * p.ldc + cn), w);
+                        store_c_16(tile_rs, w, voff, soff);
                     } else {
-                        float* dst = (float*)c_base + (long long)cm * p.ldc + cn;
-                        A8W8_STORE_C((v4f*)dst, (v4f{v[0], v[1], v[2], v[3]}));
-                        A8W8_STORE_C((v4f*)(dst + 4), (v4f{v[4], v[5], v[6], v[7]}));
+                        store_c_16(tile_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), voff, soff);
+                        store_c_16(tile_rs, __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), voff + 16, soff);
                     }
                     continue;
                 }

@@ -293,6 +293,9 @@ gemm_a8w8_wide(PersistParams pp)
     int tile_seq = 0;                               // tiles this workgroup has started: picks the row/col scale buffer
     float ep_ts = 1.f;
     bool ep_vec_ok = false;                         // C rows of this batch entry take 16-byte stores
+    // whole tiles go out through a buffer descriptor over the tile's own rows (store_c_16)
+    __amdgpu_buffer_rsrc_t ep_rs;
+    int ep_lane_off = 0, ep_row_bytes = 0;
     // One piece = the lane's eight consecutive n of MFMA tile row i and tile pair jp: scale, convert,
     // one 16-byte store (bf16) or two (fp32).
     auto store_piece = [&](auto I, auto JP, bool checked) __attribute__((always_inline)) {
@@ -320,8 +323,24 @@ gemm_a8w8_wide(PersistParams pp)
                 v[4 + e] *= hi[e] * sa;
             }
         }
-        if (checked && cm >= p.m) return;
-        const bool vec = !checked || (ep_vec_ok && cn + 7 < p.n);
+        if (!checked) {
+            // a whole tile: through the tile's buffer descriptor
+            constexpr int ES = CDT == C_BF16 ? 2 : 4;
+            constexpr int row = PERM_A ? 32 * (i >> 1) + 4 * (i & 1) : 16 * i;
+            const int voff = ep_lane_off + 32 * jp * ES, soff = row * ep_row_bytes;
+            if constexpr (CDT == C_BF16) {
+                v4i w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+                store_c_16(ep_rs, w, voff, soff);
+            } else {
+                store_c_16(ep_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), voff, soff);
+                store_c_16(ep_rs, __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), voff + 16, soff);
+            }
+            return;
+        }
+        if (cm >= p.m) return;
+        const bool vec = ep_vec_ok && cn + 7 < p.n;
         if constexpr (CDT == C_BF16) {
             unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
             if (vec) {
@@ -605,6 +624,12 @@ gemm_a8w8_wide(PersistParams pp)
                 ep_vec_ok = (p.ldc & (CDT == C_BF16 ? 7 : 3)) == 0 && (c_addr & 15) == 0;
                 // pieces are written without checks: only for whole tiles with aligned rows
                 const bool fast = ep_vec_ok && m0 + BM <= p.m && n0 + BN <= p.n;
+                {
+                    constexpr int ES = CDT == C_BF16 ? 2 : 4;
+                    ep_rs = make_rsrc((const char*)c_addr + ((long long)m0 * p.ldc + n0) * ES, (uint32_t)((BM - 1) * p.ldc + BN) * ES);
+                    ep_row_bytes = p.ldc * ES;
+                    ep_lane_off = ((wave_m * 128 + (PERM_A ? 8 * (r16 >> 2) + (r16 & 3) : r16)) * p.ldc + wave_n * 128 + 8 * g) * ES;
+                }
                 if (fast) {
                     step(T{}, F{}, T{});
                     have_prev = true;
