@@ -395,10 +395,7 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
             return launch_flat_nt<2, 8, CDT, MODE, BROW>(p, batch, stream);
     }
     if (mt == 4) {
-        // four weight tiles x four row groups fill the register file; the scale bytes of MXFP8 on top would spill
-        if constexpr (MODE != MODE_MXT) {
-            if (tiles >= 4ll * cus) return launch_flat_nt<4, 4, CDT, MODE, BROW>(p, batch, stream);
-        }
+        if (tiles >= 4ll * cus) return launch_flat_nt<4, 4, CDT, MODE, BROW>(p, batch, stream);
         return launch_flat_nt<2, 4, CDT, MODE, BROW>(p, batch, stream);
     }
     if (mt == 3) {
@@ -417,15 +414,14 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 // On shuffled weights both the flat GEMM and the MFMA kernels can run a skinny problem; the entry points take the
 // one a small cost model calls faster.  Times in microseconds, W = weight bytes, row_bytes = bytes of one weight row:
 //   flat:  one pass over the weights at ~6.3 TB/s; every further group of 16 activation rows adds ~2 us of
-//          activation traffic and MFMA work.  With the scale bytes of MXFP8, four groups only fit the registers with two
-//          weight tiles per workgroup, which costs another ~30%.
+//          activation traffic and MFMA work (the scale bytes of MXFP8 add about a tenth).
 //   dense: the 128-tile kernel has only n/128 workgroups to pull the weights with, ~28 GB/s each (128 rows a
 //          workgroup), and ~5 TB/s at best over the chip.
 // Weights of at most 32 MiB always go flat.  Measured on MI355X, M = 16 / 32 / 48 / 64, flat against dense:
-//   16384 x 7168   FP8 21 / 21 / 23 / 24 against 37-40, MXFP8 20 / 22 / 24 / 35 against 38-41,
+//   16384 x 7168   FP8 21 / 21 / 23 / 24 against 37-40, MXFP8 20 / 22 / 24 / 27 against 38-41,
 //                  MXFP4 12 / 13 / 14 / 20 against 21-22, bf16 37 / 38 / 41 / 45 against 66-72
 //   8192 x 8192    FP8 13 / 14 / 16 / 18 against 40-41 (64 workgroups on the dense side)
-//   28672 x 4096   FP8 21 / 23 / 26 / 28 against 26-27, MXFP8 22 / 25 / 28 / 40 against 26-28,
+//   28672 x 4096   FP8 21 / 23 / 26 / 28 against 26-27, MXFP8 22 / 25 / 28 / 29 against 26-28,
 //                  MXFP4 13 / 16 / 17 / 25 against 15-16, bf16 43 / 43 / 48 / 52 against 47-48
 // The model takes the faster side in these except where the two are within ~8% of each other.
 // Row-major weights (a8w8_gemm without b_preshuffled; the flat kernel stages the weight rows through LDS, whole lines
@@ -445,7 +441,6 @@ bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, double 
         flat = 3.5 + w / 6.3e6 + 2.0 * (groups - 1);      // one pass with six or eight row groups (see launch_flat)
     } else {
         flat = 3.5 + w / 6.3e6 + 2.0 * (mt - 1);
-        if (mt == 4 && scaled_in_loop) flat *= 1.3;
         if (passes == 2) flat *= 1.55;      // the second pass reads the weights from L2
     }
     flat *= layout_factor;      // row-major weights: rows staged through LDS, rows a power of two apart share channels
@@ -456,7 +451,7 @@ bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, double 
 
 bool prefer_flat_fp8(const a8w8_gemm_args* g)
 {
-    const bool scaled_in_loop = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;      // four row groups: two weight tiles per workgroup
+    const bool scaled_in_loop = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;      // no kernel with eight row groups
     const double layout_factor = g->b_preshuffled ? 1.0 : g->stride_b % 4096 == 0 ? 1.3 : 1.05;
     return prefer_flat(g->m, g->n, g->k, scaled_in_loop, layout_factor);
 }

@@ -61,6 +61,26 @@ A8W8_DEV v4i ld16_nt(__amdgpu_buffer_rsrc_t rs, uint32_t voffset, int soffset)
 // touch every LDS bank once.
 constexpr int FLAT_STAGE_SLOTS = 8 * 18;
 
+// Scaled FP8 MFMA whose two E8M0 scales are bytes `byte_b` / `byte_a` (0 .. 3, constants once the caller's loops are
+// unrolled) of the registers sb / sa.
+template <int OB, int OA>
+A8W8_DEV v4f mfma_mx_sel(v8i b, v8i a, v4f c, int sb, int sa)
+{
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b, a, c, 0, 0, OB, sb, OA, sa);
+}
+A8W8_DEV v4f mfma_mx_bytes(v8i b, v8i a, v4f c, int byte_b, int sb, int byte_a, int sa)
+{
+    switch (byte_b * 4 + byte_a) {
+#define A8W8_MX_CASE(B, A) case B * 4 + A: return mfma_mx_sel<B, A>(b, a, c, sb, sa);
+        A8W8_MX_CASE(0, 0) A8W8_MX_CASE(0, 1) A8W8_MX_CASE(0, 2) A8W8_MX_CASE(0, 3)
+        A8W8_MX_CASE(1, 0) A8W8_MX_CASE(1, 1) A8W8_MX_CASE(1, 2) A8W8_MX_CASE(1, 3)
+        A8W8_MX_CASE(2, 0) A8W8_MX_CASE(2, 1) A8W8_MX_CASE(2, 2) A8W8_MX_CASE(2, 3)
+        A8W8_MX_CASE(3, 0) A8W8_MX_CASE(3, 1) A8W8_MX_CASE(3, 2) A8W8_MX_CASE(3, 3)
+#undef A8W8_MX_CASE
+    }
+    return c;
+}
+
 // MT groups of 16 activation rows per workgroup share one pass over the weights.  With MT = 1 a lane gathers its
 // MFMA fragment straight from memory (16 bytes of one row per lane: 16 cache lines per quarter wave, affordable
 // once per pair of K blocks).  With MT > 1 that gather would cost more than the weight stream, so the wave reads
@@ -293,17 +313,38 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
                 f.fsa[g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_blk_a, blk_a_off + 64u * g, pp * p.stride_sfa * 4, 0));
             f.fsb = blk_b[pp];
         }
+        // (the scale bytes before the weights: loads complete in issue order, and pack_scales waits for these only)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if constexpr (MODE == MODE_MXT) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b8(rs_sb, mx_b[NT == 4 ? 0 : t], unit_b + (NT == 4 ? (int)MX_DELTA[t & 3] : 0), 0);
+            if constexpr (MODE == MODE_F4T) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b16(rs_sb, mx_b[NT == 4 ? 0 : t], unit_b + (NT == 4 ? (int)MX_DELTA[t & 3] : 0), 0);
+        }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             if constexpr (!BROW) {
                 f.b[t][0] = ld16_nt(rs_b, lane16, b_off[t] + kt0 * 1024);
                 f.b[t][1] = ld16_nt(rs_b, lane16 | kill1, b_off[t] + kt1 * 1024);
             }
-            if constexpr (MODE == MODE_MXT) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b8(rs_sb, mx_b[NT == 4 ? 0 : t], unit_b + (NT == 4 ? (int)MX_DELTA[t & 3] : 0), 0);
-            if constexpr (MODE == MODE_F4T) f.sb[t] = __builtin_amdgcn_raw_buffer_load_b16(rs_sb, mx_b[NT == 4 ? 0 : t], unit_b + (NT == 4 ? (int)MX_DELTA[t & 3] : 0), 0);
         }
     };
-    auto mma = [&](const Frag& f) {
+    // MXFP8: the pair's scale bytes, four to a register (byte g % 4 / byte t, picked by the MFMA's op_sel): the
+    // registers they arrived in are free for the next pair's before its loads are issued
+    struct Packed { int a[(MT + 3) / 4], b; };
+    auto pack_scales = [&](const Frag& f) {
+        Packed q{};
+        if constexpr (MODE == MODE_MXT) {
+#pragma unroll
+            for (int g = 0; g < MT; ++g) q.a[g >> 2] = (g & 3) ? q.a[g >> 2] | (f.sa[g] << (8 * (g & 3))) : f.sa[g];
+            q.b = f.sb[0];
+#pragma unroll
+            for (int t = 1; t < NT; ++t) q.b |= f.sb[t] << (8 * t);
+#pragma unroll
+            for (int w = 0; w < (MT + 3) / 4; ++w) asm volatile("" : "+v"(q.a[w]));
+            asm volatile("" : "+v"(q.b));
+        }
+        return q;
+    };
+    auto mma = [&](const Frag& f, const Packed q) {
         v4i blo[NT], bhi[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
@@ -348,7 +389,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
                         (v8i{bhi[t].x, bhi[t].y, bhi[t].z, bhi[t].w, 0, 0, 0, 0}), (v8i{ahi.x, ahi.y, ahi.z, ahi.w, 0, 0, 0, 0}),
                         acc[g][t], 4, 4, 1, f.sb[t], 1, f.sa[g]);
                 } else if constexpr (MODE == MODE_MXT) {
-                    acc[g][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[g][t], 0, 0, 0, f.sb[t], 0, f.sa[g]);
+                    acc[g][t] = mfma_mx_bytes(fb, fa, acc[g][t], t, q.b, g & 3, q.a[g >> 2]);
                 } else {
                     acc[g][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[g][t], 0, 0, 0, 0, 0, 0);
                 }
@@ -388,19 +429,21 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
         while (left > 0) {
             if constexpr (STAGING) stage_rows();
             at = next_of(at);
+            const Packed q0 = pack_scales(f0);
             if (left > 1) {
                 load_staged(pair_of(at));
                 load(pair_of(at), f1);
             }
-            mma(f0);
+            mma(f0, q0);
             if (--left == 0) break;
             if constexpr (STAGING) stage_rows();
             at = next_of(at);
+            const Packed q1 = pack_scales(f1);
             if (left > 1) {
                 load_staged(pair_of(at));
                 load(pair_of(at), f0);
             }
-            mma(f1);
+            mma(f1, q1);
             if (--left == 0) break;
         }
     }
