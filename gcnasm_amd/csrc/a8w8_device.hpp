@@ -96,17 +96,21 @@ A8W8_DEV void load_to_lds_16(__amdgpu_buffer_rsrc_t rsrc, A8W8_LDS void* lds_bas
 #define A8W8_STORE_C(ptr, val) (*(ptr) = (val))
 #endif
 
-// 16 bytes of a whole C tile through a buffer descriptor over the tile.  The store carries the sc1 bit: the line is
-// written through to memory as it is stored instead of waiting in this XCD's L2 for the write-back at the end of the
-// kernel, which otherwise delays the next launch (2 us less per launch measured for a 32 MiB C).
+// 16 bytes of a whole C tile through a buffer descriptor over the tile.
+// WRITE_THROUGH: the store carries the sc1 bit: the line is written through to memory as it is stored instead of
+// waiting in this XCD's L2 for the write-back at the end of the kernel, which otherwise delays the next launch (2 us
+// less per launch measured for a 32 MiB bf16 C).  Only for stores whose lanes together cover whole 64-byte pieces
+// of a line, as the bf16 ones do; the fp32 stores are interleaved 16-byte pieces that L2 has to merge first (written
+// through, a 8192 x 8192 fp32 C took 557 us instead of 452).
 // A 16-byte buffer store reads its data registers for a few cycles after it issues.  The compiler keeps the next
 // write to them at a distance only when the scalar-offset field holds no register; with a register there, fp32
 // outputs stored straight from the accumulators came out overwritten, in some lanes, by the scale products the next
 // instruction put into the same registers.  Hence the two idle cycles, in a statement that keeps `data` alive across
 // them (the build checks that they directly follow every such store).
+template <bool WRITE_THROUGH>
 A8W8_DEV void store_c_16(__amdgpu_buffer_rsrc_t rsrc, v4i data, int lane_offset, int scalar_offset)
 {
-    __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, lane_offset, scalar_offset, 16);
+    __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, lane_offset, scalar_offset, WRITE_THROUGH ? 16 : 0);
     asm volatile("s_nop 1" ::"v"(data));
 }
 

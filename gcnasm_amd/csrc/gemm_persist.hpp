@@ -352,10 +352,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                             w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
-                        store_c_16(tile_rs, w, voff, soff);
+                        store_c_16<true>(tile_rs, w, voff, soff);
                     } else {
-                        store_c_16(tile_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), voff, soff);
-                        store_c_16(tile_rs, __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), voff + 16, soff);
+                        store_c_16<false>(tile_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), voff, soff);
+                        store_c_16<false>(tile_rs, __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), voff + 16, soff);
                     }
                     continue;
                 }

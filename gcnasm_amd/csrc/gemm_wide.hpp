@@ -332,10 +332,10 @@ gemm_a8w8_wide(PersistParams pp)
                 v4i w;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
-                store_c_16(ep_rs, w, voff, soff);
+                store_c_16<true>(ep_rs, w, voff, soff);
             } else {
-                store_c_16(ep_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), voff, soff);
-                store_c_16(ep_rs, __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), voff + 16, soff);
+                store_c_16<false>(ep_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), voff, soff);
+                store_c_16<false>(ep_rs, __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), voff + 16, soff);
             }
             return;
         }
