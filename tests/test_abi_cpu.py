@@ -38,6 +38,7 @@ def _ok_args(mode=g.BLOCK, m=256, n=256, k=256, **kw):
     (lambda a: setattr(a, "k", 192), -3),          # K % 128 for block scales
     (lambda a: setattr(a, "stride_a", 128), -4),
     (lambda a: setattr(a, "stride_c", 100), -4),
+    (lambda a: setattr(a, "stride_c", (1 << 22) + (1 << 16)), -7),    # 255 rows of a C tile no longer fit a 32-bit offset
     (lambda a: setattr(a, "stride_sfa", 8), -4),
     (lambda a: setattr(a, "scale_mode", 7), -6),
     (lambda a: setattr(a, "c_dtype", 3), -6),
@@ -182,6 +183,10 @@ def test_pipelined_kernels_use_no_scratch():
     # the four-wave kernels name their accumulator registers themselves: the build checks that the
     # compiler put nothing of its own there (gcnasm_amd/csrc/check_isa.py) and records the verdict
     assert "accumulator registers untouched by the compiler" in text
+    # ... and that every 16-byte buffer store of a C tile is followed by the idle cycles its data registers need
+    assert re.search(r"16-byte buffer stores: \d+ checked, each followed by its idle cycles", text)
+    # MXFP8 flat GEMM: four weight tiles x four row groups exists (and is among the kernels checked above)
+    assert "flatmm_a8w8ILi4ELi4ELi0ELi4ELb0EE" in text
 
 
 def test_sibling_entry_points_reject_bad_arguments():

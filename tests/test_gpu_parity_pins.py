@@ -6,6 +6,8 @@
 * Conversion of NaN, Inf and out-of-range inputs on the hardware, against the oracle's statement of it.
 * Routing corners: row strides of 2^23 bytes and more, a single K step over many tiles, one weight matrix shared
   by a batch, explicit device set-up.
+* The whole-tile C stores (buffer stores through a per-tile descriptor) of both pipelined kernels, bit for bit, in
+  both output types, into a C whose rows are padded.
 """
 import ctypes
 
@@ -172,3 +174,25 @@ def test_explicit_device_setup():
     assert L.a8w8_init(63) == -9                                # no such device
     assert torch.cuda.current_device() == 0
     g.init()
+
+
+@pytest.mark.parametrize("k", [512, 384])       # an even number of K steps: the four-wave kernel; odd: the eight-wave one
+@pytest.mark.parametrize("c_dtype", [g.BF16, g.FP32])
+def test_whole_tile_stores_bit_for_bit(orc, k, c_dtype):
+    """Exact integers with row/col scales that are powers of two: every output is exact in fp32 (bf16: its one
+    rounding, to nearest even on both sides), so any byte a store drops, moves or overwrites shows.  C has padded rows (stride_c > n), must keep its padding, and is
+    written by workgroups that run two tiles back to back (more tiles than compute units)."""
+    m, n, ldc = 4352, 4608, 4608 + 64
+    a, b = datagen.small_ints(m, n, k, seed=7300 + k, lo=-1, hi=1)
+    rng = np.random.Generator(np.random.Philox(7301))
+    sa = np.exp2(rng.integers(-2, 3, m)).astype(np.float32)
+    sb = np.exp2(rng.integers(-2, 3, n)).astype(np.float32)
+    want = (torch.from_numpy(orc.decode(a)).cuda() @ torch.from_numpy(orc.decode(b)).cuda().T) * dev(sa)[:, None] * dev(sb)[None, :]
+    torch_dtype = torch.bfloat16 if c_dtype == g.BF16 else torch.float32
+    store = torch.full((m, ldc), -7.0, dtype=torch_dtype, device="cuda")
+    c = store[:, :n]
+    g.gemm(dev(a), dev(b), dev(sa), dev(sb), g.ROWCOL, c=c, c_dtype=c_dtype)
+    args = g.raw_gemm_args(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, m, n, k, g.ROWCOL, c_dtype=c_dtype, stride_c=ldc)
+    assert g.kernel_name(args) == ("gemm_a8w8_wide" if k == 512 else "gemm_a8w8_persist")
+    assert torch.equal(c.float(), want.to(torch_dtype).float())
+    assert bool((store[:, n:] == -7.0).all())
