@@ -314,6 +314,14 @@ A8W8_DEV int mx_block_exponent(float amax, float top)
     return e;
 }
 
+// 16 bytes of an input that is read once: a non-temporal load (the line is not kept in L2 in place of something that
+// will be read again; 8192 x 8192 fp32 to FP8 with row scales 58.9 -> 54.2 us, to MXFP8 56.6 -> 54.1 us)
+A8W8_DEV float4 load_once4(const float* p)
+{
+    const v4f t = __builtin_nontemporal_load((const v4f*)p);
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+
 // MX E4M3 with one E8M0 exponent per 32 elements.  A wave takes 1024 consecutive elements of the
 // flattened [rows, k] array as four chunks of 256: lane l owns elements 4l..4l+3 of each chunk, eight
 // lanes share a block.  Every load and store instruction of a wave covers one contiguous run of memory;
@@ -338,7 +346,7 @@ __global__ void __launch_bounds__(256) quant_mx_vec_kernel(const float* __restri
         row[c] = live[c] ? e0 / (unsigned)k : 0u;
         col[c] = live[c] ? e0 % (unsigned)k : 0u;
         v[c] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (live[c]) v[c] = *(const float4*)(src + (size_t)row[c] * ld + col[c]);
+        if (live[c]) v[c] = load_once4(src + (size_t)row[c] * ld + col[c]);
     }
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -404,7 +412,7 @@ __global__ void __launch_bounds__(256) quant_rowwise_vec_kernel(const float* __r
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int i = threadIdx.x * 4 + u * 1024;
-            held[u] = i < k ? *(const float4*)(x + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+            held[u] = i < k ? load_once4(x + i) : make_float4(0.f, 0.f, 0.f, 0.f);
             amax = fmaxf(amax, fmaxf(fmaxf(fabsf(held[u].x), fabsf(held[u].y)), fmaxf(fabsf(held[u].z), fabsf(held[u].w))));
         }
     } else {
@@ -456,7 +464,7 @@ __global__ void __launch_bounds__(256) quant_1x128_vec_kernel(const float* __res
         row[u] = live[u] ? (int)((w0 + u) / groups) : 0;
         g[u] = live[u] ? (int)((w0 + u) % groups) : 0;
         v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (live[u]) v[u] = *(const float4*)(src + (size_t)row[u] * ld + g[u] * 128 + 4 * l);
+        if (live[u]) v[u] = load_once4(src + (size_t)row[u] * ld + g[u] * 128 + 4 * l);
     }
 #pragma unroll
     for (int u = 0; u < G; ++u) {
