@@ -74,7 +74,9 @@ typedef enum { A8W8_E4M3_OCP = 0, A8W8_E4M3_FNUZ = 1 } a8w8_fp8_dialect;
  * (opus_gemm/block_scale_gemm/gemm_a8w8_blockscale_common.h:4-25) with the same field
  * meanings: A is [batch, m, k] row-major, B is [batch, n, k] row-major (the column-major
  * K x N weight), C is [batch, m, n]; every stride counts ELEMENTS (common.h:12-17).
- * A and B hold OCP E4M3 bytes.  C[i,j] = sum_k A[i,k] * B[j,k] * scale. */
+ * A and B hold OCP E4M3 bytes.  C[i,j] = sum_k A[i,k] * B[j,k] * scale.
+ * Sizes (else A8W8_ERR_TOO_LARGE): one batch entry of A and of B spans less than 2 GiB, stride_c is below 4 Mi
+ * elements (the 256 rows of a C tile are addressed with 32-bit offsets), batch <= 65535. */
 typedef struct {
     const void* a;
     const void* b;
