@@ -331,6 +331,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             make_rsrc(c_base + ((long long)m0 * p.ldc + n0) * C_ES, (uint32_t)((BM - 1) * p.ldc + BN) * C_ES);
         const int tile_lane_off = ((wave_m * WAVE_M + r16) * p.ldc + wave_n * WAVE_N + 8 * g) * C_ES;
         const int tile_row16 = 16 * p.ldc * C_ES;
+        // fp32: the lane's places in the two stores of a piece (rows 0 .. 7 / 8 .. 15 of the 16, see store_c_f32_piece)
+        const bool upper = r16 >= 8;
+        const int f32_row = (wave_m * WAVE_M + (r16 & 7)) * p.ldc + wave_n * WAVE_N + 8 * g;
+        const int f32_off_low = f32_row * 4 + (upper ? 16 : 0), f32_off_high = (f32_row + 8 * p.ldc) * 4 + (upper ? 0 : 16);
 #pragma unroll
         for (int jp = 0; jp < TN / 2; ++jp) {
             const int cn = cn_base + 32 * jp;
@@ -354,8 +358,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                             w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
                         store_c_16<true>(tile_rs, w, voff, soff);
                     } else {
-                        store_c_16<false>(tile_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), voff, soff);
-                        store_c_16<false>(tile_rs, __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), voff + 16, soff);
+                        (void)voff;
+                        store_c_f32_piece(tile_rs, v4f{v[0], v[1], v[2], v[3]}, v4f{v[4], v[5], v[6], v[7]}, upper,
+                                          f32_off_low + 32 * jp * 4, f32_off_high + 32 * jp * 4, soff);
                     }
                     continue;
                 }

@@ -296,6 +296,7 @@ gemm_a8w8_wide(PersistParams pp)
     // whole tiles go out through a buffer descriptor over the tile's own rows (store_c_16)
     __amdgpu_buffer_rsrc_t ep_rs;
     int ep_lane_off = 0, ep_row_bytes = 0;
+    int ep_f32_low = 0, ep_f32_high = 0;            // fp32: the lane's places in the two stores of a piece (store_c_f32_piece)
     // One piece = the lane's eight consecutive n of MFMA tile row i and tile pair jp: scale, convert,
     // one 16-byte store (bf16) or two (fp32).
     auto store_piece = [&](auto I, auto JP, bool checked) __attribute__((always_inline)) {
@@ -334,8 +335,9 @@ gemm_a8w8_wide(PersistParams pp)
                 for (int e = 0; e < 4; ++e) w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
                 store_c_16<true>(ep_rs, w, voff, soff);
             } else {
-                store_c_16<false>(ep_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), voff, soff);
-                store_c_16<false>(ep_rs, __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), voff + 16, soff);
+                (void)voff;
+                store_c_f32_piece(ep_rs, v4f{v[0], v[1], v[2], v[3]}, v4f{v[4], v[5], v[6], v[7]}, r16 >= 8,
+                                  ep_f32_low + 32 * jp * 4, ep_f32_high + 32 * jp * 4, soff);
             }
             return;
         }
@@ -628,7 +630,14 @@ gemm_a8w8_wide(PersistParams pp)
                     constexpr int ES = CDT == C_BF16 ? 2 : 4;
                     ep_rs = make_rsrc((const char*)c_addr + ((long long)m0 * p.ldc + n0) * ES, (uint32_t)((BM - 1) * p.ldc + BN) * ES);
                     ep_row_bytes = p.ldc * ES;
-                    ep_lane_off = ((wave_m * 128 + (PERM_A ? 8 * (r16 >> 2) + (r16 & 3) : r16)) * p.ldc + wave_n * 128 + 8 * g) * ES;
+                    auto row_of = [&](int r) __attribute__((always_inline)) { return PERM_A ? 8 * (r >> 2) + (r & 3) : r; };
+                    ep_lane_off = ((wave_m * 128 + row_of(r16)) * p.ldc + wave_n * 128 + 8 * g) * ES;
+                    if constexpr (CDT == C_FP32) {
+                        // lanes r and r + 8 of a row of 16 write the line of lane r's row in the first store, of lane r + 8's in the second
+                        const int col = (wave_n * 128 + 8 * g) * 4 + (r16 >= 8 ? 16 : 0);
+                        ep_f32_low = (wave_m * 128 + row_of(r16 & 7)) * p.ldc * 4 + col;
+                        ep_f32_high = (wave_m * 128 + row_of((r16 & 7) + 8)) * p.ldc * 4 + (col ^ 16);
+                    }
                 }
                 if (fast) {
                     step(T{}, F{}, T{});

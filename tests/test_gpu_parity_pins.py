@@ -196,3 +196,24 @@ def test_whole_tile_stores_bit_for_bit(orc, k, c_dtype):
     assert g.kernel_name(args) == ("gemm_a8w8_wide" if k == 512 else "gemm_a8w8_persist")
     assert torch.equal(c.float(), want.to(torch_dtype).float())
     assert bool((store[:, n:] == -7.0).all())
+
+
+@pytest.mark.parametrize("c_dtype", [g.BF16, g.FP32])
+def test_whole_tile_stores_with_tiled_mx_scales(orc, c_dtype):
+    """The four-wave kernel deals the rows of a tile to its lanes differently when the scales are tiled MX; the
+    stores have to follow.  Exact integers, per-row exponents that differ from row to row (a row that lands in
+    another row's place shows), padded C."""
+    m, n, k, ldc = 4352, 4608, 512, 4608 + 32
+    a, b = datagen.small_ints(m, n, k, seed=7400, lo=-1, hi=1)
+    rng = np.random.Generator(np.random.Philox(7401))
+    ea = np.repeat(rng.integers(125, 130, (m, 1)), k // 32, axis=1).astype(np.uint8)
+    eb = np.repeat(rng.integers(125, 130, (n, 1)), k // 32, axis=1).astype(np.uint8)
+    sa = np.exp2(ea[:, 0].astype(np.float32) - 127)
+    sb = np.exp2(eb[:, 0].astype(np.float32) - 127)
+    want = (torch.from_numpy(orc.decode(a)).cuda() @ torch.from_numpy(orc.decode(b)).cuda().T) * dev(sa)[:, None] * dev(sb)[None, :]
+    torch_dtype = torch.bfloat16 if c_dtype == g.BF16 else torch.float32
+    store = torch.full((m, ldc), -7.0, dtype=torch_dtype, device="cuda")
+    c = store[:, :n]
+    g.gemm(dev(a), dev(b), g.mx_tile_scales(dev(ea)), g.mx_tile_scales(dev(eb)), g.MX_TILED, c=c, c_dtype=c_dtype)
+    assert torch.equal(c.float(), want.to(torch_dtype).float())
+    assert bool((store[:, n:] == -7.0).all())
