@@ -100,7 +100,7 @@ A8W8_DEV void load_to_lds_16(__amdgpu_buffer_rsrc_t rsrc, A8W8_LDS void* lds_bas
 // WRITE_THROUGH: the store carries the sc1 bit: the line is written through to memory as it is stored instead of
 // waiting in this XCD's L2 for the write-back at the end of the kernel, which otherwise delays the next launch (2 us
 // less per launch measured for a 32 MiB bf16 C).  Only for stores whose lanes together cover whole 64-byte pieces
-// of a line, as the bf16 ones do and the fp32 ones after store_c_f32_piece has rearranged them; interleaved 16-byte
+// of a line, as store_c_lines arranges them; interleaved 16-byte
 // pieces have to be merged by L2 first (written through, a 8192 x 8192 fp32 C took 557 us instead of 452).
 // A 16-byte buffer store reads its data registers for a few cycles after it issues.  The compiler keeps the next
 // write to them at a distance only when the scalar-offset field holds no register; with a register there, fp32
@@ -120,20 +120,30 @@ A8W8_DEV int from_lane_8_apart(int v)
     return __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false);
 }
 
-// An fp32 piece of a whole C tile: the lane holds eight consecutive columns (32 bytes) of one row, `lo` and `hi`.
-// Stored as they are, the two 16-byte stores of a wave would each cover every other 16 bytes of 16 rows.  Instead the
-// lanes of rows r and r + 8 exchange halves, so that one store writes rows 0 .. 7 of the 16 and the other rows 8 .. 15,
-// each row as one contiguous 128-byte line (lane r < 8: its own `lo`, lane r + 8: the `hi` of lane r, 16 bytes on):
-// whole lines can take the write-through path.  lane_offset_low / _high: the lane's place in the first / second store
-// (set up per tile by the caller); upper: the lane's row index within the 16 is 8 or more.
-A8W8_DEV void store_c_f32_piece(__amdgpu_buffer_rsrc_t rsrc, v4f lo, v4f hi, bool upper, int lane_offset_low, int lane_offset_high,
-                                int scalar_offset)
+// The two 16-byte halves `lo`, `hi` of the eight consecutive fp32 columns a lane holds of one row of a whole C tile
+// (`hi` DISTANCE = 16 bytes after `lo`).  Stored as they are, each store of a wave would cover every other 16 bytes of
+// 16 rows.  Instead the lanes of rows r and r + 8 (of the 16 a wave's store covers) exchange halves, so that one store
+// writes rows 0 .. 7 and the other rows 8 .. 15, each row as one contiguous 128-byte line (lane r < 8: its own `lo`;
+// lane r + 8: the `hi` of lane r, DISTANCE bytes on): whole lines, which can take the write-through path.  (The same
+// for two bf16 pieces side by side, DISTANCE 64, measured no faster than their 64-byte pieces.)
+// lane_offset_low / _high: the lane's place in the first / second store (c_line_offsets, per tile); upper: the
+// lane's row index within the 16 is 8 or more.
+A8W8_DEV void store_c_lines(__amdgpu_buffer_rsrc_t rsrc, v4i lo, v4i hi, bool upper, int lane_offset_low, int lane_offset_high,
+                            int scalar_offset)
 {
-    const v4i x = __builtin_bit_cast(v4i, lo), y = __builtin_bit_cast(v4i, hi);
-    const v4i r = {from_lane_8_apart(y.x), from_lane_8_apart(y.y), from_lane_8_apart(y.z), from_lane_8_apart(y.w)};
-    const v4i first = upper ? r : x, second = upper ? x : r;
+    const v4i r = {from_lane_8_apart(hi.x), from_lane_8_apart(hi.y), from_lane_8_apart(hi.z), from_lane_8_apart(hi.w)};
+    const v4i first = upper ? r : lo, second = upper ? lo : r;
     store_c_16<true>(rsrc, first, lane_offset_low, scalar_offset);
     store_c_16<true>(rsrc, second, lane_offset_high, scalar_offset);
+}
+// The two lane offsets of store_c_lines: row_low / row_high = byte offsets of the rows that lanes (r16 & 7) and
+// (r16 & 7) + 8 own, col = the lane's byte offset inside a row (a multiple of 2 * DISTANCE).
+template <int DISTANCE>
+A8W8_DEV void c_line_offsets(int r16, int row_low, int row_high, int col, int& lane_offset_low, int& lane_offset_high)
+{
+    const bool upper = r16 >= 8;
+    lane_offset_low = row_low + col + (upper ? DISTANCE : 0);
+    lane_offset_high = row_high + col + (upper ? 0 : DISTANCE);
 }
 
 // Barrier without the wait for every outstanding load that __syncthreads() implies: the pipelined kernels

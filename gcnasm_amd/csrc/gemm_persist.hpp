@@ -325,16 +325,50 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         // a tile that lies inside the matrix and takes 16-byte stores is written without per-lane checks (the
         // checked path spends more instructions on masks and branches than on stores)
         const bool whole = vec_ok && m0 + BM <= p.m && n0 + BN <= p.n;
-        // such a tile goes out through a buffer descriptor over its own rows (store_c_16), with 32-bit offsets
+        // such a tile goes out through a buffer descriptor over its own rows (store_c_16, store_c_lines), with 32-bit offsets
         constexpr int C_ES = CDT == C_BF16 ? 2 : 4;
         const __amdgpu_buffer_rsrc_t tile_rs =
             make_rsrc(c_base + ((long long)m0 * p.ldc + n0) * C_ES, (uint32_t)((BM - 1) * p.ldc + BN) * C_ES);
-        const int tile_lane_off = ((wave_m * WAVE_M + r16) * p.ldc + wave_n * WAVE_N + 8 * g) * C_ES;
         const int tile_row16 = 16 * p.ldc * C_ES;
-        // fp32: the lane's places in the two stores of a piece (rows 0 .. 7 / 8 .. 15 of the 16, see store_c_f32_piece)
+        // bf16: one 16-byte store per piece, 64 contiguous bytes per row and instruction.  fp32: the lane's places in
+        // the two stores of store_c_lines (rows 0 .. 7 / 8 .. 15 of the 16 rows of a piece)
+        const int tile_lane_off = ((wave_m * WAVE_M + r16) * p.ldc + wave_n * WAVE_N + 8 * g) * C_ES;
         const bool upper = r16 >= 8;
-        const int f32_row = (wave_m * WAVE_M + (r16 & 7)) * p.ldc + wave_n * WAVE_N + 8 * g;
-        const int f32_off_low = f32_row * 4 + (upper ? 16 : 0), f32_off_high = (f32_row + 8 * p.ldc) * 4 + (upper ? 0 : 16);
+        int line_off_low, line_off_high;
+        c_line_offsets<16>(r16, (wave_m * WAVE_M + (r16 & 7)) * p.ldc * C_ES, (wave_m * WAVE_M + (r16 & 7) + 8) * p.ldc * C_ES,
+                           (wave_n * WAVE_N + 8 * g) * C_ES, line_off_low, line_off_high);
+        auto scaled_piece = [&](int i, int jp, float (&v)[8]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v[e] = acc[i][2 * jp + (e >> 2)][e & 3];
+                if constexpr (MODE == MODE_TENSOR) v[e] *= ts;
+                if constexpr (MODE == MODE_ROWCOL) v[e] *= sb[jp][e] * sa[i];
+            }
+        };
+        auto packed_bf16 = [&](const float (&v)[8]) __attribute__((always_inline)) {
+            v4i w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+            return w;
+        };
+        if (whole) {
+#pragma unroll
+            for (int jp = 0; jp < TN / 2; ++jp)
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    float v[8];
+                    scaled_piece(i, jp, v);
+                    // 32 jp columns on (an immediate), 16 i rows down (a scalar)
+                    if constexpr (CDT == C_BF16) {
+                        store_c_16<true>(tile_rs, packed_bf16(v), tile_lane_off + 32 * jp * C_ES, i * tile_row16);
+                    } else {
+                        store_c_lines(tile_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}),
+                                      __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), upper, line_off_low + 32 * jp * C_ES,
+                                      line_off_high + 32 * jp * C_ES, i * tile_row16);
+                    }
+                }
+            return;
+        }
 #pragma unroll
         for (int jp = 0; jp < TN / 2; ++jp) {
             const int cn = cn_base + 32 * jp;
@@ -342,28 +376,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
             for (int i = 0; i < TM; ++i) {
                 const int cm = cm_of(i);
                 float v[8];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    v[e] = acc[i][2 * jp + (e >> 2)][e & 3];
-                    if constexpr (MODE == MODE_TENSOR) v[e] *= ts;
-                    if constexpr (MODE == MODE_ROWCOL) v[e] *= sb[jp][e] * sa[i];
-                }
-                if (whole) {
-                    // lane offset + 32 jp columns (an immediate) | 16 i rows (a scalar)
-                    const int voff = tile_lane_off + 32 * jp * C_ES, soff = i * tile_row16;
-                    if constexpr (CDT == C_BF16) {
-                        v4i w;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
-                        store_c_16<true>(tile_rs, w, voff, soff);
-                    } else {
-                        (void)voff;
-                        store_c_f32_piece(tile_rs, v4f{v[0], v[1], v[2], v[3]}, v4f{v[4], v[5], v[6], v[7]}, upper,
-                                          f32_off_low + 32 * jp * 4, f32_off_high + 32 * jp * 4, soff);
-                    }
-                    continue;
-                }
+                scaled_piece(i, jp, v);
                 if (cm >= p.m) continue;
                 if constexpr (CDT == C_BF16) {
                     unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;

@@ -296,7 +296,7 @@ gemm_a8w8_wide(PersistParams pp)
     // whole tiles go out through a buffer descriptor over the tile's own rows (store_c_16)
     __amdgpu_buffer_rsrc_t ep_rs;
     int ep_lane_off = 0, ep_row_bytes = 0;
-    int ep_f32_low = 0, ep_f32_high = 0;            // fp32: the lane's places in the two stores of a piece (store_c_f32_piece)
+    int ep_f32_low = 0, ep_f32_high = 0;            // fp32: the lane's places in the two stores of a piece (store_c_lines)
     // One piece = the lane's eight consecutive n of MFMA tile row i and tile pair jp: scale, convert,
     // one 16-byte store (bf16) or two (fp32).
     auto store_piece = [&](auto I, auto JP, bool checked) __attribute__((always_inline)) {
@@ -336,8 +336,8 @@ gemm_a8w8_wide(PersistParams pp)
                 store_c_16<true>(ep_rs, w, voff, soff);
             } else {
                 (void)voff;
-                store_c_f32_piece(ep_rs, v4f{v[0], v[1], v[2], v[3]}, v4f{v[4], v[5], v[6], v[7]}, r16 >= 8,
-                                  ep_f32_low + 32 * jp * 4, ep_f32_high + 32 * jp * 4, soff);
+                store_c_lines(ep_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}),
+                              r16 >= 8, ep_f32_low + 32 * jp * 4, ep_f32_high + 32 * jp * 4, soff);
             }
             return;
         }
@@ -632,12 +632,9 @@ gemm_a8w8_wide(PersistParams pp)
                     ep_row_bytes = p.ldc * ES;
                     auto row_of = [&](int r) __attribute__((always_inline)) { return PERM_A ? 8 * (r >> 2) + (r & 3) : r; };
                     ep_lane_off = ((wave_m * 128 + row_of(r16)) * p.ldc + wave_n * 128 + 8 * g) * ES;
-                    if constexpr (CDT == C_FP32) {
-                        // lanes r and r + 8 of a row of 16 write the line of lane r's row in the first store, of lane r + 8's in the second
-                        const int col = (wave_n * 128 + 8 * g) * 4 + (r16 >= 8 ? 16 : 0);
-                        ep_f32_low = (wave_m * 128 + row_of(r16 & 7)) * p.ldc * 4 + col;
-                        ep_f32_high = (wave_m * 128 + row_of((r16 & 7) + 8)) * p.ldc * 4 + (col ^ 16);
-                    }
+                    if constexpr (CDT == C_FP32)
+                        c_line_offsets<16>(r16, (wave_m * 128 + row_of(r16 & 7)) * p.ldc * 4, (wave_m * 128 + row_of((r16 & 7) + 8)) * p.ldc * 4,
+                                           (wave_n * 128 + 8 * g) * 4, ep_f32_low, ep_f32_high);
                 }
                 if (fast) {
                     step(T{}, F{}, T{});
