@@ -111,6 +111,12 @@ int launch(void (*kern)(P...), dim3 grid, dim3 block, unsigned lds, hipStream_t 
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
+// The pipelined kernels address the 256 rows of a C tile with unsigned 32-bit byte offsets from the tile's origin.
+bool c_tile_fits(long long stride_c)
+{
+    return (long long)(BM - 1) * stride_c * 4 + BN * 4 < (1ll << 32);
+}
+
 // Checks shared by every GEMM entry point (mirrors the reference harness's rejects,
 // gemm_a8w8_blockscale_host.cc:175-187, and adds the pointer/stride checks a library needs).
 int validate_common(const a8w8_gemm_args* g)
@@ -144,7 +150,7 @@ int validate_common(const a8w8_gemm_args* g)
         return A8W8_ERR_TOO_LARGE;
     if ((long long)((g->m + 127) / 128) * ((g->n + 127) / 128) >= (1ll << 31)) return A8W8_ERR_TOO_LARGE;
     // ... and the 256 rows of a C tile (stride_c below 4 Mi elements)
-    if ((long long)(BM - 1) * g->stride_c * 4 + BN * 4 >= (1ll << 32)) return A8W8_ERR_TOO_LARGE;
+    if (!c_tile_fits(g->stride_c)) return A8W8_ERR_TOO_LARGE;
     return A8W8_OK;
 }
 
@@ -539,7 +545,7 @@ static int a16w16_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     if (g->batch > 1 && (g->stride_a_batch < 0 || g->stride_b_batch < 0 || g->stride_c_batch < 0)) return A8W8_ERR_BAD_STRIDE;
     const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) * 2;
     const long long b_span = (g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k) * 2;
-    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
+    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535 || !c_tile_fits(g->stride_c)) return A8W8_ERR_TOO_LARGE;
     if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
     // the tiled kernel reads bf16 rows as byte rows of 2k columns
@@ -608,7 +614,7 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
         return A8W8_ERR_BAD_STRIDE;
     const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) / 2;
     const long long b_span = (g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k) / 2;
-    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
+    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535 || !c_tile_fits(g->stride_c)) return A8W8_ERR_TOO_LARGE;
     if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
     // the tiled kernel reads packed rows as byte rows of k/2 columns

@@ -197,7 +197,8 @@ def test_sibling_entry_points_reject_bad_arguments():
     a = _ok_args(mode=g.TENSOR)
     for mutate, want in [(lambda x: setattr(x, "c", None), -1), (lambda x: setattr(x, "k", 0), -2),
                          (lambda x: setattr(x, "c_dtype", 7), -6),
-                         (lambda x: setattr(x, "stride_b", 100), -4)]:
+                         (lambda x: setattr(x, "stride_b", 100), -4),
+                         (lambda x: setattr(x, "stride_c", (1 << 22) + (1 << 16)), -7)]:     # rows of a C tile past 32-bit offsets
         b = _ok_args(mode=g.TENSOR)
         mutate(b)
         assert L.a16w16_gemm(ref(b), None) == want
@@ -213,6 +214,7 @@ def test_sibling_entry_points_reject_bad_arguments():
     for mutate, want in [(lambda x: setattr(x, "sfa", None), -1), (lambda x: setattr(x, "scale_mode", g.ROWCOL), -6),
                          (lambda x: setattr(x, "k", 48), -3), (lambda x: setattr(x, "stride_a", 200), -4),
                          (lambda x: setattr(x, "stride_a", 259), -5),       # rows must start on a byte
+                         (lambda x: setattr(x, "stride_c", (1 << 22) + (1 << 16)), -7),
                          (lambda x: setattr(x, "stride_sfa", 4), -4)]:
         b = _ok_args(mode=g.MX, m=64, n=64, k=256)
         mutate(b)
