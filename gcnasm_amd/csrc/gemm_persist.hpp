@@ -436,7 +436,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         fetch_step_scales(cur_batch, m0, n0, 0, 0);
     }
     issue_rowcol_scales(cur_batch, m0, n0);
-    __builtin_amdgcn_s_waitcnt(0);
+    // vmcnt(8) lgkmcnt(0): step 0 (and MX scale group 0, issued before step 1's loads) has landed; the eight loads of
+    // step 1 may still be on their way: the first step's end barrier waits for them like any other step's
+    __builtin_amdgcn_s_waitcnt(0x0078);
     A8W8_RAW_BARRIER();
     if constexpr (IS_MX) fetch_step_scales(cur_batch, m0, n0, 0, 0);
     if constexpr (PREFETCH_FRAGS) {
