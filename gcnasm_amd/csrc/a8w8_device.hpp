@@ -142,8 +142,8 @@ template <int DISTANCE>
 A8W8_DEV void c_line_offsets(int r16, int row_low, int row_high, int col, int& lane_offset_low, int& lane_offset_high)
 {
     const bool upper = r16 >= 8;
-    lane_offset_low = row_low + col + (upper ? DISTANCE : 0);
-    lane_offset_high = row_high + col + (upper ? 0 : DISTANCE);
+    lane_offset_low = (int)((uint32_t)row_low + (uint32_t)(col + (upper ? DISTANCE : 0)));
+    lane_offset_high = (int)((uint32_t)row_high + (uint32_t)(col + (upper ? 0 : DISTANCE)));
 }
 
 // Barrier without the wait for every outstanding load that __syncthreads() implies: the pipelined kernels

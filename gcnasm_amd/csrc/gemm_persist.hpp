@@ -329,13 +329,15 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         constexpr int C_ES = CDT == C_BF16 ? 2 : 4;
         const __amdgpu_buffer_rsrc_t tile_rs =
             make_rsrc(c_base + ((long long)m0 * p.ldc + n0) * C_ES, (uint32_t)((BM - 1) * p.ldc + BN) * C_ES);
-        const int tile_row16 = 16 * p.ldc * C_ES;
+        // (unsigned arithmetic: with stride_c in the millions these byte offsets pass 2^31; the hardware takes them as unsigned)
+        const uint32_t ldc_bytes = (uint32_t)p.ldc * C_ES;
+        const int tile_row16 = (int)(16u * ldc_bytes);
         // bf16: one 16-byte store per piece, 64 contiguous bytes per row and instruction.  fp32: the lane's places in
         // the two stores of store_c_lines (rows 0 .. 7 / 8 .. 15 of the 16 rows of a piece)
-        const int tile_lane_off = ((wave_m * WAVE_M + r16) * p.ldc + wave_n * WAVE_N + 8 * g) * C_ES;
+        const int tile_lane_off = (int)((uint32_t)(wave_m * WAVE_M + r16) * ldc_bytes + (uint32_t)((wave_n * WAVE_N + 8 * g) * C_ES));
         const bool upper = r16 >= 8;
         int line_off_low, line_off_high;
-        c_line_offsets<16>(r16, (wave_m * WAVE_M + (r16 & 7)) * p.ldc * C_ES, (wave_m * WAVE_M + (r16 & 7) + 8) * p.ldc * C_ES,
+        c_line_offsets<16>(r16, (int)((uint32_t)(wave_m * WAVE_M + (r16 & 7)) * ldc_bytes), (int)((uint32_t)(wave_m * WAVE_M + (r16 & 7) + 8) * ldc_bytes),
                            (wave_n * WAVE_N + 8 * g) * C_ES, line_off_low, line_off_high);
         auto scaled_piece = [&](int i, int jp, float (&v)[8]) __attribute__((always_inline)) {
 #pragma unroll

@@ -328,7 +328,7 @@ gemm_a8w8_wide(PersistParams pp)
             // a whole tile: through the tile's buffer descriptor
             constexpr int ES = CDT == C_BF16 ? 2 : 4;
             constexpr int row = PERM_A ? 32 * (i >> 1) + 4 * (i & 1) : 16 * i;
-            const int voff = ep_lane_off + 32 * jp * ES, soff = row * ep_row_bytes;
+            const int voff = ep_lane_off + 32 * jp * ES, soff = (int)((uint32_t)row * (uint32_t)ep_row_bytes);
             if constexpr (CDT == C_BF16) {
                 v4i w;
 #pragma unroll
@@ -633,9 +633,10 @@ gemm_a8w8_wide(PersistParams pp)
                     ep_rs = make_rsrc((const char*)c_addr + ((long long)m0 * p.ldc + n0) * ES, (uint32_t)((BM - 1) * p.ldc + BN) * ES);
                     ep_row_bytes = p.ldc * ES;
                     auto row_of = [&](int r) __attribute__((always_inline)) { return PERM_A ? 8 * (r >> 2) + (r & 3) : r; };
-                    ep_lane_off = ((wave_m * 128 + row_of(r16)) * p.ldc + wave_n * 128 + 8 * g) * ES;
+                    // (unsigned arithmetic: with stride_c in the millions these byte offsets pass 2^31; the hardware takes them as unsigned)
+                    ep_lane_off = (int)((uint32_t)(wave_m * 128 + row_of(r16)) * (uint32_t)ep_row_bytes + (uint32_t)((wave_n * 128 + 8 * g) * ES));
                     if constexpr (CDT == C_FP32)
-                        c_line_offsets<16>(r16, (wave_m * 128 + row_of(r16 & 7)) * p.ldc * 4, (wave_m * 128 + row_of((r16 & 7) + 8)) * p.ldc * 4,
+                        c_line_offsets<16>(r16, (int)((uint32_t)(wave_m * 128 + row_of(r16 & 7)) * (uint32_t)ep_row_bytes), (int)((uint32_t)(wave_m * 128 + row_of((r16 & 7) + 8)) * (uint32_t)ep_row_bytes),
                                            (wave_n * 128 + 8 * g) * 4, ep_f32_low, ep_f32_high);
                 }
                 if (fast) {

@@ -217,3 +217,23 @@ def test_whole_tile_stores_with_tiled_mx_scales(orc, c_dtype):
     g.gemm(dev(a), dev(b), g.mx_tile_scales(dev(ea)), g.mx_tile_scales(dev(eb)), g.MX_TILED, c=c, c_dtype=c_dtype)
     assert torch.equal(c.float(), want.to(torch_dtype).float())
     assert bool((store[:, n:] == -7.0).all())
+
+
+@pytest.mark.parametrize("k", [256, 384])
+@pytest.mark.parametrize("c_dtype", [g.BF16, g.FP32])
+def test_c_rows_millions_of_elements_apart(orc, k, c_dtype):
+    """stride_c = 4,000,000: the byte offsets of a C tile's rows pass 2^31 (unsigned 32-bit offsets in the kernels);
+    enough 128-tiles that the pipelined kernels take the problem."""
+    m, n, ldc = 256, 128 * 257, 4_000_000
+    a, b = datagen.small_ints(m, n, k, seed=7500 + k, lo=-1, hi=1)
+    want = torch.from_numpy(orc.decode(a)).cuda() @ torch.from_numpy(orc.decode(b)).cuda().T
+    torch_dtype = torch.bfloat16 if c_dtype == g.BF16 else torch.float32
+    store = torch.empty(m * ldc, dtype=torch_dtype, device="cuda")
+    c = torch.as_strided(store, (m, n), (ldc, 1))
+    ones_m, ones_n = dev(np.ones(m, np.float32)), dev(np.ones(n, np.float32))
+    g.gemm(dev(a), dev(b), ones_m, ones_n, g.ROWCOL, c=c, c_dtype=c_dtype)
+    args = g.raw_gemm_args(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, m, n, k, g.ROWCOL, c_dtype=c_dtype, stride_c=ldc)
+    assert g.kernel_name(args) == ("gemm_a8w8_wide" if k == 256 else "gemm_a8w8_persist")
+    assert torch.equal(c.float(), want.to(torch_dtype).float())
+    del store
+    torch.cuda.empty_cache()
