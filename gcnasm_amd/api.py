@@ -180,6 +180,34 @@ def _check_scales(t, name, scale_mode):
         raise TypeError(f"{name} must be {want} for this scale mode, got {t.dtype}")
 
 
+def scale_elements(scale_mode, rows, k, weight_side):
+    """Elements one batch entry's scale array holds for a matrix of `rows` rows (A: weight_side False, B: True), as the
+    kernels index it with the default strides of raw_gemm_args."""
+    if scale_mode == TENSOR:
+        return 1
+    if scale_mode == ROWCOL:
+        return rows
+    if scale_mode == BLOCK:
+        return ((rows + 127) // 128 if weight_side else rows) * (k // 128)
+    if scale_mode == MX:
+        return rows * (k // 32)
+    return mx_tiled_bytes(rows, k)
+
+
+def _check_scale_sizes(sfa, sfb, scale_mode, m, n, k, batch, b_shared):
+    """An undersized scale array would be read past its end on the device; weights shared by all batch entries come with
+    one set of weight scales (a per-entry set would silently be used for entry 0 only)."""
+    need_a = batch * scale_elements(scale_mode, m, k, False)
+    per_b = scale_elements(scale_mode, n, k, True)
+    need_b = per_b if b_shared else batch * per_b
+    if sfa.numel() < need_a:
+        raise ValueError(f"sfa holds {sfa.numel()} elements, this problem reads {need_a}")
+    if sfb.numel() < need_b:
+        raise ValueError(f"sfb holds {sfb.numel()} elements, this problem reads {need_b}")
+    if b_shared and sfb.numel() >= batch * per_b and sfb.numel() > per_b:
+        raise ValueError(f"b is shared by all {batch} batch entries but sfb holds a set of scales per entry; pass one set")
+
+
 def _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, b_preshuffled, n=None, scaled=True):
     _check_operand(a, "a", (2, 3))
     _check_operand(b, "b", (1, 2) if b_preshuffled else (2, 3))
@@ -217,6 +245,8 @@ def _args_from_tensors(a, b, sfa, sfb, scale_mode, c, c_dtype, b_preshuffled, n=
             # one weight matrix shared by every batch entry, and with it one set of weight scales
             g.stride_b_batch = 0
             g.stride_sfb_batch = 0
+    if scaled:
+        _check_scale_sizes(sfa, sfb, scale_mode, m, n, k, batch, b_shared=(batch > 1 and g.stride_b_batch == 0))
     return g, c
 
 

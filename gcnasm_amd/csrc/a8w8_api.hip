@@ -111,10 +111,12 @@ int launch(void (*kern)(P...), dim3 grid, dim3 block, unsigned lds, hipStream_t 
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
-// The pipelined kernels address the 256 rows of a C tile with unsigned 32-bit byte offsets from the tile's origin.
-bool c_tile_fits(long long stride_c)
+// The two pipelined kernels (and only they) address the 256 rows of a C tile with unsigned 32-bit byte offsets from
+// the tile's origin: (255 stride_c + 256) elements of `elem_bytes` must stay below 2^32.  That is stride_c up to
+// 4,210,751 for fp32 and 8,421,503 for bf16; the other kernels address C with 64-bit pointers and take any stride.
+bool c_tile_fits(long long stride_c, int elem_bytes)
 {
-    return (long long)(BM - 1) * stride_c * 4 + BN * 4 < (1ll << 32);
+    return ((long long)(BM - 1) * stride_c + BN) * elem_bytes < (1ll << 32);
 }
 
 // Checks shared by every GEMM entry point (mirrors the reference harness's rejects,
@@ -149,8 +151,6 @@ int validate_common(const a8w8_gemm_args* g)
     if (g->scale_mode == A8W8_SCALE_BLOCK_1x128_128x128 && (long long)(g->k / 128) * g->stride_sfa * 4 >= (1ll << 31))
         return A8W8_ERR_TOO_LARGE;
     if ((long long)((g->m + 127) / 128) * ((g->n + 127) / 128) >= (1ll << 31)) return A8W8_ERR_TOO_LARGE;
-    // ... and the 256 rows of a C tile (stride_c below 4 Mi elements)
-    if (!c_tile_fits(g->stride_c)) return A8W8_ERR_TOO_LARGE;
     return A8W8_OK;
 }
 
@@ -280,6 +280,7 @@ int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
     // tiled MX scales exist on the four-wave kernel only (whatever passes persist_ok with them also passes wide_ok)
     if constexpr (MODE == MODE_MXT) return launch_wide<MODE, CDT>(p, batch, stream);
     else {
+    if (!c_tile_fits(p.ldc, CDT == C_BF16 ? 2 : 4)) return A8W8_ERR_TOO_LARGE;
     PersistParams pp;
     pp.g = p;
     pp.batch = batch;
@@ -295,6 +296,7 @@ template <int MODE, int CDT>
 int launch_wide(const GemmParams& p, int batch, hipStream_t stream)
 {
     if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT || MODE == MODE_BF16 || MODE == MODE_F4T) {
+        if (!c_tile_fits(p.ldc, CDT == C_BF16 ? 2 : 4)) return A8W8_ERR_TOO_LARGE;
         PersistParams pp;
         pp.g = p;
         pp.batch = batch;
@@ -497,6 +499,17 @@ bool flat_rowmajor_ok(const a8w8_gemm_args* g)
     return (long long)(g->n - 1) * g->stride_b + g->k < (1ll << 31);
 }
 
+// Whether launch_dense_fp8 (and the bf16 / MXFP4 entry points on their byte views) would take one of the two 256-tile
+// kernels: their C tiles must fit 32-bit offsets (c_tile_fits), which the entry points check before any device call.
+bool takes_tile256(const a8w8_gemm_args* g)
+{
+    return tiled_ok(g) && !small_ok(g) && (wide_ok(g) || persist_ok(g));
+}
+bool c_stride_too_large(const a8w8_gemm_args* g, const a8w8_gemm_args* byte_view)
+{
+    return takes_tile256(byte_view) && !c_tile_fits(g->stride_c, g->c_dtype == A8W8_C_BF16 ? 2 : 4);
+}
+
 int launch_dense_fp8(const a8w8_gemm_args* g, hipStream_t s)
 {
     const GemmParams p = make_params(g);
@@ -521,11 +534,12 @@ int a8w8_gemm(const a8w8_gemm_args* args, void* hip_stream)
     const a8w8_gemm_args* g = &local;
     const int shuf = validate_shuffled_b(g);
     if (shuf != A8W8_OK) return shuf;
+    // a skinny problem on shuffled weights: the flat kernel where it is the faster one
+    const bool flat = (g->b_preshuffled && validate_flat(g) == A8W8_OK && prefer_flat_fp8(g)) || (flat_rowmajor_ok(g) && prefer_flat_fp8(g));
+    if (!flat && c_stride_too_large(g, g)) return A8W8_ERR_TOO_LARGE;
     if (const int ds = device_status(); ds != A8W8_OK) return ds;
     hipStream_t s = (hipStream_t)hip_stream;
-    // a skinny problem on shuffled weights: the flat kernel where it is the faster one
-    if (g->b_preshuffled && validate_flat(g) == A8W8_OK && prefer_flat_fp8(g)) return launch_flat_fp8(g, s);
-    if (flat_rowmajor_ok(g) && prefer_flat_fp8(g)) return launch_flat_fp8(g, s);
+    if (flat) return launch_flat_fp8(g, s);
     return launch_dense_fp8(g, s);
 }
 
@@ -545,9 +559,7 @@ static int a16w16_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     if (g->batch > 1 && (g->stride_a_batch < 0 || g->stride_b_batch < 0 || g->stride_c_batch < 0)) return A8W8_ERR_BAD_STRIDE;
     const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) * 2;
     const long long b_span = (g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k) * 2;
-    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535 || !c_tile_fits(g->stride_c)) return A8W8_ERR_TOO_LARGE;
-    if (const int ds = device_status(); ds != A8W8_OK) return ds;
-    hipStream_t s = (hipStream_t)hip_stream;
+    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     // the tiled kernel reads bf16 rows as byte rows of 2k columns
     a8w8_gemm_args bytes = *g;
     bytes.k = g->k * 2;
@@ -555,8 +567,12 @@ static int a16w16_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allo
     bytes.stride_a_batch = g->stride_a_batch * 2; bytes.stride_b_batch = g->stride_b_batch * 2;
     bytes.scale_mode = A8W8_SCALE_TENSOR;
     const bool fits = (long long)g->stride_a_batch * 2 < (1ll << 31) && (long long)g->stride_b_batch * 2 < (1ll << 31);
+    const bool flat_rows = fits && flat_rowmajor_ok(&bytes) && prefer_flat(g->m, g->n, bytes.k, false, bytes.stride_b % 4096 == 0 ? 1.3 : 1.05);
+    if (!flat_rows && fits && c_stride_too_large(g, &bytes)) return A8W8_ERR_TOO_LARGE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
+    hipStream_t s = (hipStream_t)hip_stream;
     // a skinny problem on row-major weights: the flat kernel (weight rows staged through LDS) where it is the faster one
-    if (fits && flat_rowmajor_ok(&bytes) && prefer_flat(g->m, g->n, bytes.k, false, bytes.stride_b % 4096 == 0 ? 1.3 : 1.05)) {
+    if (flat_rows) {
         GemmParams p = make_params(&bytes);
         p.sfa = p.sfb = nullptr;
         return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_BF16, true>(p, g->batch, s)
@@ -614,17 +630,19 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
         return A8W8_ERR_BAD_STRIDE;
     const long long a_span = ((long long)(g->m - 1) * g->stride_a + g->k) / 2;
     const long long b_span = (g->b_preshuffled ? (long long)g->n * g->k : (long long)(g->n - 1) * g->stride_b + g->k) / 2;
-    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535 || !c_tile_fits(g->stride_c)) return A8W8_ERR_TOO_LARGE;
-    if (const int ds = device_status(); ds != A8W8_OK) return ds;
-    hipStream_t s = (hipStream_t)hip_stream;
+    if (a_span >= (1ll << 31) || b_span >= (1ll << 31) || g->batch > 65535) return A8W8_ERR_TOO_LARGE;
     // the tiled kernel reads packed rows as byte rows of k/2 columns
     a8w8_gemm_args bytes = *g;
     bytes.k = g->k / 2;
     bytes.stride_a = g->stride_a / 2; bytes.stride_b = g->b_preshuffled ? bytes.k : g->stride_b / 2;
     bytes.stride_a_batch = g->stride_a_batch / 2; bytes.stride_b_batch = g->stride_b_batch / 2;
     bytes.scale_mode = A8W8_SCALE_MX_E8M0_TILED;
+    const bool flat_rows = tiled && flat_rowmajor_ok(&bytes) && prefer_flat(g->m, g->n, bytes.k, false, bytes.stride_b % 4096 == 0 ? 1.3 : 1.05);
+    if (!flat_rows && tiled && g->k % 256 == 0 && c_stride_too_large(g, &bytes)) return A8W8_ERR_TOO_LARGE;
+    if (const int ds = device_status(); ds != A8W8_OK) return ds;
+    hipStream_t s = (hipStream_t)hip_stream;
     // a skinny problem on row-major weights: the flat kernel where it is the faster one
-    if (tiled && flat_rowmajor_ok(&bytes) && prefer_flat(g->m, g->n, bytes.k, false, bytes.stride_b % 4096 == 0 ? 1.3 : 1.05)) {
+    if (flat_rows) {
         const GemmParams p = make_params(&bytes);
         return g->c_dtype == A8W8_C_BF16 ? launch_flat<C_BF16, MODE_F4T, true>(p, g->batch, s)
                                          : launch_flat<C_FP32, MODE_F4T, true>(p, g->batch, s);

@@ -392,13 +392,19 @@ gemm_a8w8_wide(PersistParams pp)
     point_scales_at(sf_cur, cur_item);
     point_scales_at(sf_next, cur_item + (int)gridDim.x);
     issue_mx_batch(sf_cur, 0, 0);
-    // steps 0 and 1 in full
+    // Steps 0 and 1 in full.  Step 1's quarters go out in the order an odd step of the steady state issues
+    // them (aL, bH, bL, aH): the hand-overs of the step that follows count on it.  Step 0's mid hand-over
+    // waits for "all but the newest 16 loads"; by then aL and bL of step 2 have been issued behind step 1,
+    // so what has landed is the first two quarters of step 1, and these must be the two that the second
+    // half of step 0 reads: aL(1) and bH(1).  The end hand-over covers the other two.
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
 #pragma unroll
-        for (int qt = 0; qt < 4; ++qt)
+        for (int q = 0; q < 4; ++q) {
+            const int qt = st == 0 ? q : (q == 0 ? 0 : 4 - q);
 #pragma unroll
             for (int l = 0; l < 4; ++l) issue_one(st, qt, l);
+        }
         advance_ld();
     }
     // vmcnt(16) lgkmcnt(0): step 0 and the first scale batch have landed; the 16 loads of step 1 may still be on their

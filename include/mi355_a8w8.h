@@ -75,8 +75,10 @@ typedef enum { A8W8_E4M3_OCP = 0, A8W8_E4M3_FNUZ = 1 } a8w8_fp8_dialect;
  * meanings: A is [batch, m, k] row-major, B is [batch, n, k] row-major (the column-major
  * K x N weight), C is [batch, m, n]; every stride counts ELEMENTS (common.h:12-17).
  * A and B hold OCP E4M3 bytes.  C[i,j] = sum_k A[i,k] * B[j,k] * scale.
- * Sizes (else A8W8_ERR_TOO_LARGE): one batch entry of A and of B spans less than 2 GiB, stride_c is below 4 Mi
- * elements (the 256 rows of a C tile are addressed with 32-bit offsets), batch <= 65535. */
+ * Sizes (else A8W8_ERR_TOO_LARGE): one batch entry of A and of B spans less than 2 GiB, batch <= 65535, and, for
+ * problems that run on the two 256 x 256-tile kernels (a8w8_kernel_name: gemm_a8w8_wide, gemm_a8w8_persist), whose
+ * tiles are addressed with unsigned 32-bit byte offsets, (255 stride_c + 256) * sizeof(C element) < 2^32, i.e.
+ * stride_c <= 4,210,751 for fp32 and <= 8,421,503 for bf16; the other kernels take any stride_c. */
 typedef struct {
     const void* a;
     const void* b;

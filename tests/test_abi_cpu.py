@@ -38,7 +38,6 @@ def _ok_args(mode=g.BLOCK, m=256, n=256, k=256, **kw):
     (lambda a: setattr(a, "k", 192), -3),          # K % 128 for block scales
     (lambda a: setattr(a, "stride_a", 128), -4),
     (lambda a: setattr(a, "stride_c", 100), -4),
-    (lambda a: setattr(a, "stride_c", (1 << 22) + (1 << 16)), -7),    # 255 rows of a C tile no longer fit a 32-bit offset
     (lambda a: setattr(a, "stride_sfa", 8), -4),
     (lambda a: setattr(a, "scale_mode", 7), -6),
     (lambda a: setattr(a, "c_dtype", 3), -6),
@@ -49,6 +48,35 @@ def test_gemm_rejects_bad_arguments(mutate, want):
     assert g.lib().a8w8_gemm(ctypes.byref(a), None) == want
     assert g.kernel_name(a) is None
     assert g.status_string(want) != "unknown status"
+
+
+def test_c_stride_limit_applies_to_the_256_tile_kernels_only():
+    """The two 256-tile kernels address a C tile's 256 rows with unsigned 32-bit byte offsets:
+    (255 stride_c + 256) * sizeof(element) < 2^32.  Rejected before any device call; every other kernel takes any stride."""
+    L, ref = g.lib(), ctypes.byref
+    fp32_max, bf16_max = 4_210_751, 8_421_503
+    for mode, k in [(g.ROWCOL, 512), (g.BLOCK, 512), (g.ROWCOL, 384)]:          # wide, persist, persist (odd step count)
+        for c_dtype, most in [(g.FP32, fp32_max), (g.BF16, bf16_max)]:
+            big = _ok_args(mode=mode, m=4096, n=4096, k=k, c_dtype=c_dtype, stride_c=most + 1)
+            assert g.kernel_name(_ok_args(mode=mode, m=4096, n=4096, k=k, c_dtype=c_dtype)) in ("gemm_a8w8_wide", "gemm_a8w8_persist")
+            assert L.a8w8_gemm(ref(big), None) == -7
+            fits = _ok_args(mode=mode, m=4096, n=4096, k=k, c_dtype=c_dtype, stride_c=most)
+            assert L.a8w8_gemm(ref(fits), None) != -7
+    # the 128-tile kernel, the one-thread-per-element kernel and the flat kernel use 64-bit pointers
+    for kw in [dict(mode=g.ROWCOL, m=256, n=256, k=256), dict(mode=g.ROWCOL, m=4096, n=4096, k=200, stride_a=200, stride_b=200),
+               dict(mode=g.ROWCOL, m=16, n=4096, k=4096)]:
+        a = _ok_args(stride_c=1 << 24, **kw)
+        assert g.kernel_name(a) in ("gemm_a8w8_tile128", "gemm_a8w8_general", "flatmm_a8w8")
+        assert L.a8w8_gemm(ref(a), None) != -7
+    # siblings: m, n, k in their own elements
+    big = _ok_args(mode=g.TENSOR, m=4096, n=4096, k=512, c_dtype=g.FP32, stride_c=fp32_max + 1)
+    assert L.a16w16_gemm(ref(big), None) == -7
+    small = _ok_args(mode=g.TENSOR, m=256, n=256, k=256, c_dtype=g.FP32, stride_c=fp32_max + 1)
+    assert L.a16w16_gemm(ref(small), None) != -7
+    big = _ok_args(mode=g.MX_TILED, m=4096, n=4096, k=1024, c_dtype=g.FP32, stride_c=fp32_max + 1)
+    assert L.a4w4_gemm(ref(big), None) == -7
+    small = _ok_args(mode=g.MX_TILED, m=64, n=64, k=256, c_dtype=g.FP32, stride_c=fp32_max + 1)
+    assert L.a4w4_gemm(ref(small), None) != -7
 
 
 def test_null_struct_and_mx_group():
@@ -197,8 +225,7 @@ def test_sibling_entry_points_reject_bad_arguments():
     a = _ok_args(mode=g.TENSOR)
     for mutate, want in [(lambda x: setattr(x, "c", None), -1), (lambda x: setattr(x, "k", 0), -2),
                          (lambda x: setattr(x, "c_dtype", 7), -6),
-                         (lambda x: setattr(x, "stride_b", 100), -4),
-                         (lambda x: setattr(x, "stride_c", (1 << 22) + (1 << 16)), -7)]:     # rows of a C tile past 32-bit offsets
+                         (lambda x: setattr(x, "stride_b", 100), -4)]:
         b = _ok_args(mode=g.TENSOR)
         mutate(b)
         assert L.a16w16_gemm(ref(b), None) == want
@@ -214,7 +241,6 @@ def test_sibling_entry_points_reject_bad_arguments():
     for mutate, want in [(lambda x: setattr(x, "sfa", None), -1), (lambda x: setattr(x, "scale_mode", g.ROWCOL), -6),
                          (lambda x: setattr(x, "k", 48), -3), (lambda x: setattr(x, "stride_a", 200), -4),
                          (lambda x: setattr(x, "stride_a", 259), -5),       # rows must start on a byte
-                         (lambda x: setattr(x, "stride_c", (1 << 22) + (1 << 16)), -7),
                          (lambda x: setattr(x, "stride_sfa", 4), -4)]:
         b = _ok_args(mode=g.MX, m=64, n=64, k=256)
         mutate(b)

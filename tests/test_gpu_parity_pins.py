@@ -166,6 +166,12 @@ def test_batch_sharing_one_weight_matrix(orc):
         g.gemm(dev(a)[:, :, ::2], dev(b)[:, ::2], dev(sa), dev(sb), g.ROWCOL)      # rows that are not contiguous
     with pytest.raises(TypeError):
         g.gemm(dev(a), dev(b), dev(sa.astype(np.float64)), dev(sb), g.ROWCOL)
+    with pytest.raises(ValueError, match="per entry"):
+        g.gemm(dev(a), dev(b), dev(sa), dev(np.stack([sb] * batch)), g.ROWCOL)       # a set of weight scales per entry for shared weights
+    with pytest.raises(ValueError, match="sfa holds"):
+        g.gemm(dev(a), dev(b), dev(sa[:2]), dev(sb), g.ROWCOL)                       # scales of two entries for three
+    with pytest.raises(ValueError, match="sfb holds"):
+        g.gemm(dev(a), dev(b), dev(sa), dev(sb[: n - 1]), g.ROWCOL)
 
 
 def test_explicit_device_setup():
