@@ -63,7 +63,12 @@ WORKLOADS = {
     "a16w16_4096": ("bf16", 4096, 4096, 4096, 100663296),
     # MXFP4 (a4w4_gemm, tiled scales), priced against the dense FP4 peak
     "mxfp4_8192": ("f4", 8192, 8192, 8192, 205520896),
+    # short and wide (a prefill chunk of 256 tokens over a 64 MiB weight): between the flat GEMM's M <= 128 and the
+    # 256-row tiles; A 2 MiB + B 64 MiB + C 4 MiB + scales
+    "gemm_rowcol_256x8192x8192": ("rowcol", 256, 8192, 8192, 73434112),
 }
+# workloads whose weights would stay in the 256 MB Infinity Cache between launches: timed over rotating copies of B
+ROTATE_B = {"gemm_rowcol_256x8192x8192": 5}
 
 
 def make_inputs(name, torch, g, seed):
@@ -236,9 +241,20 @@ def run_workload(name, torch, g, steps, warmup, seed, headline=True):
 
         entry = L.a16w16_gemm if mode == "bf16" else L.a4w4_gemm if mode == "f4" else L.a8w8_gemm
 
-        def fn_direct(i):
-            if entry(gemm_ref_, stream) != 0:
-                raise RuntimeError("gemm call failed")
+        if name in ROTATE_B:
+            b_copies = [inp["b"]] + [inp["b"].clone() for _ in range(ROTATE_B[name] - 1)]
+            rot_structs = [args_for(x, 0) for x in b_copies]
+            rot_refs = [ctypes.byref(x) for x in rot_structs]
+            res["note"] = f"{len(b_copies)} rotating copies of B ({len(b_copies) * n * k >> 20} MiB): every launch reads its weights from HBM"
+            res["frac_hbm_peak"] = None      # filled in below
+
+            def fn_direct(i):
+                if entry(rot_refs[i % len(rot_refs)], stream) != 0:
+                    raise RuntimeError("gemm call failed")
+        else:
+            def fn_direct(i):
+                if entry(gemm_ref_, stream) != 0:
+                    raise RuntimeError("gemm call failed")
 
         fn = fn_direct
         timer = time_steady if headline else time_best_of
@@ -282,6 +298,8 @@ def run_workload(name, torch, g, steps, warmup, seed, headline=True):
             res["frac_fp4_peak"] = flops / ms / 1e9 / PEAK_FP4_TFLOPS
         else:
             res["frac_fp8_peak"] = flops / ms / 1e9 / PEAK_FP8_TFLOPS
+        if name in ROTATE_B:
+            res["frac_hbm_peak"] = abytes / ms / 1e6 / PEAK_HBM_GBS
     fn(0)
     torch.cuda.synchronize()
     return res, inp, c
@@ -528,6 +546,22 @@ def main():
         others.extend(run_reference_program_sizes(torch, g, args.steps, args.warmup, args.seed + 3))
         others.extend(run_flat_variants(torch, g, args.steps, args.warmup, args.seed + 4))
         line["other_workloads"] = others
+        # the secondary results in short form inside `config`, which a truncated record still holds
+        by_name = {w["workload"]: w for w in others}
+        def pick(workload, key):
+            v = by_name.get(workload, {}).get(key)
+            return None if v is None else round(v, 4)
+        line["config"].update(
+            c2_frac=pick("rowcol_4096", "frac_fp8_peak"), c3_frac=pick("block_4096x7168x2048", "frac_fp8_peak"),
+            c3_us=pick("block_4096x7168x2048", "ms_per_launch") and round(by_name["block_4096x7168x2048"]["ms_per_launch"] * 1e3, 2),
+            c5_frac_hbm=pick("flatmm_16x16384x7168", "frac_hbm_peak"), c5_frac_hbm_in_graph=pick("flatmm_16x16384x7168", "frac_hbm_peak_in_graph"),
+            c5_frac_of_achievable_read=pick("flatmm_16x16384x7168", "frac_of_achievable_read"),
+            block_fp32_4096_vs_ref=pick("block_fp32_4096", "vs_reference_published"),
+            block_fp32_8192_vs_ref=pick("block_fp32_8192", "vs_reference_published"),
+            block_fp32_16384_vs_ref=pick("block_fp32_16384", "vs_reference_published"),
+            gemm_rowcol_256x8192x8192_us=pick("gemm_rowcol_256x8192x8192", "ms_per_launch") and round(by_name["gemm_rowcol_256x8192x8192"]["ms_per_launch"] * 1e3, 2),
+            flatmm_rowcol_64_frac_hbm=pick("flatmm_rowcol_64x16384x7168", "frac_hbm_peak"),
+            a16w16_4096_frac=pick("a16w16_4096", "frac_bf16_peak"), mxfp4_8192_frac=pick("mxfp4_8192", "frac_fp4_peak"))
     print(json.dumps(line))
 
 

@@ -45,6 +45,9 @@ constexpr int persist_lds_bytes(int mode)
     return mode == MODE_MX ? PERSIST_LDS_BYTES_MX : mode == MODE_ROWCOL ? PERSIST_LDS_BYTES_ROWCOL : PERSIST_LDS_BYTES;
 }
 
+// LDS stages of the 128 x 64 variant of the 128-tile kernel: as many as fit 160 KiB
+constexpr int narrow_stages(int mode) { return mode == MODE_MXT || mode == MODE_F4T ? 5 : 6; }
+
 template <int MODE>
 bool raise_lds_limits_of_mode()
 {
@@ -59,7 +62,9 @@ bool raise_lds_limits_of_mode()
         ok = ok && raise_lds_limit(gemm_a8w8_tile128<MODE, C_BF16, 2>, small_lds_bytes(MODE, 2)) &&
              raise_lds_limit(gemm_a8w8_tile128<MODE, C_FP32, 2>, small_lds_bytes(MODE, 2)) &&
              raise_lds_limit(gemm_a8w8_tile128<MODE, C_BF16, 4>, small_lds_bytes(MODE, 4)) &&
-             raise_lds_limit(gemm_a8w8_tile128<MODE, C_FP32, 4>, small_lds_bytes(MODE, 4));
+             raise_lds_limit(gemm_a8w8_tile128<MODE, C_FP32, 4>, small_lds_bytes(MODE, 4)) &&
+             raise_lds_limit(gemm_a8w8_tile128<MODE, C_BF16, narrow_stages(MODE), 64>, small_lds_bytes(MODE, narrow_stages(MODE), 64)) &&
+             raise_lds_limit(gemm_a8w8_tile128<MODE, C_FP32, narrow_stages(MODE), 64>, small_lds_bytes(MODE, narrow_stages(MODE), 64));
     return ok;
 }
 
@@ -245,6 +250,17 @@ bool small_ok(const a8w8_gemm_args* g)
     return items128 <= 2ll * num_cus();
 }
 
+// 128 x 64 tiles instead of 128 x 128: when the wide tiles would occupy at most half of the compute units and the K
+// loop is long enough for the deeper staging to matter (a problem of a few K steps is bound by launch and store latency,
+// which narrower tiles do not change).
+#ifndef A8W8_NARROW_MIN_KSTEPS
+#define A8W8_NARROW_MIN_KSTEPS 16
+#endif
+bool narrow_tiles_pay(long long items128, int n, int k)
+{
+    return 2 * items128 <= num_cus() && n > 64 && k / BK >= A8W8_NARROW_MIN_KSTEPS;
+}
+
 template <int MODE, int CDT, int STAGES>
 int launch_small_stages(const GemmParams& q, int batch, hipStream_t stream)
 {
@@ -262,7 +278,16 @@ int launch_small(const GemmParams& p, int batch, hipStream_t stream)
         GemmParams q = p;
         q.tiles_m = (p.m + SM_BM - 1) / SM_BM;
         q.tiles_n = (p.n + SM_BN - 1) / SM_BN;
-        if ((long long)q.tiles_m * q.tiles_n * batch <= num_cus())
+        const long long items = (long long)q.tiles_m * q.tiles_n * batch;
+        if (narrow_tiles_pay(items, p.n, p.k)) {
+            // short and wide: 128 x 64 tiles give every compute unit a workgroup, deep staging keeps its share of the
+            // weights in flight
+            q.tiles_n = (p.n + 63) / 64;
+            dim3 grid((unsigned)(q.tiles_m * q.tiles_n), 1, (unsigned)batch);
+            constexpr int ST = narrow_stages(MODE);
+            return launch(gemm_a8w8_tile128<MODE, CDT, ST, 64>, grid, dim3(SM_THREADS), small_lds_bytes(MODE, ST, 64), stream, q);
+        }
+        if (items <= num_cus())
             return launch_small_stages<MODE, CDT, 4>(q, batch, stream);
         return launch_small_stages<MODE, CDT, 2>(q, batch, stream);
     } else {

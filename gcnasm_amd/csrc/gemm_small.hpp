@@ -16,17 +16,17 @@
 
 namespace a8w8 {
 
-constexpr int SM_BM = 128, SM_BN = 128;
+constexpr int SM_BM = 128, SM_BN = 128;               // SM_BN: the widest tile; the kernel also takes 64 columns
 constexpr int SM_THREADS = 256;
-constexpr int SM_STAGE_BYTES = (SM_BM + SM_BN) * BK;   // 32768
+constexpr int small_stage_bytes(int bn) { return (SM_BM + bn) * BK; }   // 32768 for 128 columns, 24576 for 64
 // Scale bytes per stage.  Block mode: 128 A-row scales, the B scale at +512 and +768.  Row-major MX: the step's
 // four E8M0 bytes of 128 A rows, then of 128 B rows.  Tiled MX: 1 KiB per wave, whose first half is the 512-byte
 // unit (64 rows x one pair of K steps) of the wave's row block.
 constexpr int small_scale_bytes(int mode) { return mode == MODE_MXT || mode == MODE_F4T ? 4096 : (mode == MODE_BLOCK || mode == MODE_MX) ? 1024 : 0; }
-constexpr int SM_TM = 4, SM_TN = 4;                    // MFMA tiles per wave
-constexpr int small_lds_bytes(int mode, int stages)
+constexpr int SM_TM = 4;                               // MFMA tiles per wave along M (along N: a quarter of the tile's columns / 8)
+constexpr int small_lds_bytes(int mode, int stages, int bn = SM_BN)
 {
-    return stages * (SM_STAGE_BYTES + small_scale_bytes(mode));
+    return stages * (small_stage_bytes(bn) + small_scale_bytes(mode));
 }
 
 // p.tiles_m / p.tiles_n count 128 x 128 tiles here; grid = (tiles, 1, batch).  The launch bound asks for a
@@ -36,10 +36,19 @@ constexpr int small_lds_bytes(int mode, int stages)
 // LDS) -- for grids of at most one workgroup per compute unit, where nothing else hides the load latency.
 // SM_STAGES = 2: loads issued when a stage has been read, two barriers per step, two workgroups per compute unit
 // that hide each other's waits -- for larger grids.
-template <int MODE, int CDT, int SM_STAGES>
+// BN_ = 64: tiles of 128 x 64 (a wave owns 64 x 32) for short, wide problems -- M of a few hundred rows over weights
+// of many megabytes -- where 128 x 128 tiles would leave half of the compute units without a workgroup.  Such a
+// problem is bound by how many bytes of the weights each compute unit keeps in flight, hence SM_STAGES = 6 there
+// (five K steps of loads ahead, 144-154 KiB of LDS; 5 with tiled MX scales, whose 4 KiB per stage would not fit six).
+template <int MODE, int CDT, int SM_STAGES, int BN_ = SM_BN>
 __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 {
-    static_assert(SM_STAGES == 2 || SM_STAGES == 4, "two or four LDS stages");
+    static_assert(SM_STAGES == 2 || SM_STAGES == 4 || SM_STAGES == 5 || SM_STAGES == 6, "two, four, five or six LDS stages");
+    static_assert(BN_ == 128 || BN_ == 64, "tile width");
+    constexpr int SM_BN = BN_;
+    constexpr int SM_STAGE_BYTES = small_stage_bytes(SM_BN);
+    constexpr int SM_TN = SM_BN / 32;                  // MFMA tiles per wave along N
+    constexpr int B_LOADS = SM_BN / 32;                // 1 KiB chunks of B per wave and stage
     static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT ||
                       MODE == MODE_BF16 || MODE == MODE_F4T,
                   "fp32 scales, MX scales, bf16 operands (byte rows of 2k columns, no scales) or packed E2M1 operands (byte "
@@ -68,20 +77,19 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(a_base, (uint32_t)(p.m - 1) * p.lda + p.k);
     const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(b_base, b_extent_bytes(p));
 
-    // ---- global -> LDS.  A stage holds 16 A chunks then 16 B chunks of 1 KiB (8 rows x 128 B); wave w
-    // fills chunks w, w+4, w+8, w+12 of each matrix.  Lane i of a load lands on row i/8, slot i%8 of its
+    // ---- global -> LDS.  A stage holds 16 A chunks then 16 (or 8) B chunks of 1 KiB (8 rows x 128 B); wave w
+    // fills chunks w, w+4, .. of each matrix.  Lane i of a load lands on row i/8, slot i%8 of its
     // chunk and therefore fetches K-piece slot ^ (row & 7) = (i%8) ^ (i/8).
     const int ld_row = wave * 8 + (lane >> 3);
     const int ld_piece16 = ((lane & 7) ^ (lane >> 3)) * 16;
-    int voff_a[4], voff_b[4];
+    int voff_a[4], voff_b[B_LOADS];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        voff_a[j] = min(m0 + ld_row + 32 * j, p.m - 1) * p.lda + ld_piece16;
-        voff_b[j] = b_lane_offset(p, min(n0 + ld_row + 32 * j, p.n - 1), ld_piece16);
-    }
+    for (int j = 0; j < 4; ++j) voff_a[j] = min(m0 + ld_row + 32 * j, p.m - 1) * p.lda + ld_piece16;
+#pragma unroll
+    for (int j = 0; j < B_LOADS; ++j) voff_b[j] = b_lane_offset(p, min(n0 + ld_row + 32 * j, p.n - 1), ld_piece16);
     // block mode: waves 0 and 1 fetch the step's 128 A-row scales (64 each), waves 2 and 3 the B scale
     // of the tile's 128 x 128 block (every lane the same dword: the stage's copy at +512 is the one read)
-    constexpr int LOADS_PER_STAGE = 8 + (STEP_SCALES ? 1 : 0);
+    constexpr int LOADS_PER_STAGE = 4 + B_LOADS + (STEP_SCALES ? 1 : 0);
     __amdgpu_buffer_rsrc_t rsrc_sf = rsrc_a;
     int voff_sf = 0, sf_step_bytes = 0;
     if constexpr (MODE == MODE_BLOCK) {
@@ -118,7 +126,8 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
         rsrc_sf = make_rsrc(base, (uint32_t)mx_tiled_bytes(rows, MODE == MODE_F4T ? 2 * p.k : p.k));      // k in elements
         voff_sf = lane * 16;
         mxt_nblk = (rows + 63) >> 6;
-        mxt_blk = min(((is_b ? n0 : m0) >> 6) + (wave & 1), mxt_nblk - 1);     // a block past the last row: its rows are never stored
+        // (a block past the last row: its rows are never stored; a 64-wide tile has one B block, wave 3 brings the next along unused)
+        mxt_blk = min(((is_b ? n0 : m0) >> 6) + (wave & 1), mxt_nblk - 1);
     }
     auto issue_stage = [&](int stage, int kstep) __attribute__((always_inline)) {
         kstep = min(kstep, nk - 1);         // past the end: reload the last step into a stage nobody reads (fixed wait counts)
@@ -127,7 +136,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
         for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_a, s + j * 4096, voff_a[j], koff);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) load_to_lds_16(rsrc_b, s + SM_BM * BK + j * 4096, voff_b[j], kstep << p.b_kshift);
+        for (int j = 0; j < B_LOADS; ++j) load_to_lds_16(rsrc_b, s + SM_BM * BK + j * 4096, voff_b[j], kstep << p.b_kshift);
         if constexpr (TILED_SCALES) {
             A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 1024;
             // the pair of 128-element K steps this step belongs to (FP8: two byte steps) or is (FP4: 256 elements)
@@ -146,7 +155,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     for (int h = 0; h < 2; ++h) {
         const int slot = (g + 4 * h) ^ (lane & 7);
         rd_a[h] = (wave_m * 64 + r16) * BK + (slot << 4);
-        rd_b[h] = SM_BM * BK + (wave_n * 64 + r16) * BK + (slot << 4);
+        rd_b[h] = SM_BM * BK + (wave_n * (SM_BN / 2) + r16) * BK + (slot << 4);
     }
     auto read_frag = [&](int stage, const int (&base)[2], int t) __attribute__((always_inline)) -> v8i {
         const char* s = smem + stage * SM_STAGE_BYTES + t * (16 * BK);
@@ -157,17 +166,22 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 
     // tiled MX: byte of (row 16 t + r16 of a 64-row block, 32-block g of the K step, step s of the pair) inside the
     // block's unit, without s (see mx_tiled_index); the same for A tiles and B tiles
-    int mxt_off[4];
+    // (a 64-wide tile lies inside one 64-row block of B: wave column 1 owns the block's MFMA tiles 2 and 3)
+    int mxt_off[4], mxt_off_b[SM_TN];
+    const int mxt_unit_b = SM_BN == 128 ? (2 + wave_n) * 1024 : 2 * 1024;     // where the wave's B block lies in the stage's scale bytes
     if constexpr (TILED_SCALES) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        auto unit_offset = [&](int t) __attribute__((always_inline)) {
             const int x = (2 * t + (r16 >> 3)) & 3, y = r16 & 3, par = (r16 >> 2) & 1;
-            mxt_off[t] = ((4 * x + y) * 4 + g) * 8 + (t >> 1) * 4 + par * 2;
-        }
+            return ((4 * x + y) * 4 + g) * 8 + (t >> 1) * 4 + par * 2;
+        };
+#pragma unroll
+        for (int t = 0; t < 4; ++t) mxt_off[t] = unit_offset(t);
+#pragma unroll
+        for (int t = 0; t < SM_TN; ++t) mxt_off_b[t] = unit_offset(SM_BN == 128 ? t : 2 * wave_n + t);
     }
 
     const int cm_base = m0 + wave_m * 64 + r16;          // + 16 * i
-    const int cn_base = n0 + wave_n * 64 + 4 * g;        // + 16 * j + e
+    const int cn_base = n0 + wave_n * (SM_BN / 2) + 4 * g;        // + 16 * j + e
 
     v4f acc[SM_TM][SM_TN];
 #pragma unroll
@@ -177,14 +191,20 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 
     issue_stage(0, 0);
     issue_stage(1, 1);
-    if constexpr (SM_STAGES == 4) issue_stage(2, 2);
+    if constexpr (SM_STAGES > 2) {
+#pragma unroll
+        for (int st = 2; st < SM_STAGES - 1; ++st) issue_stage(st, st);
+    }
+    // stages in flight behind the one being read: one of two, else all but the one being refilled
+    constexpr int YOUNGER = SM_STAGES == 2 ? 1 : SM_STAGES - 2;
+    static_assert(YOUNGER * LOADS_PER_STAGE < 64, "the wait count is a 6-bit field");
 
+    int cur = 0, refill = SM_STAGES - 1;      // the stage of step ks, the stage of step ks - 1 (refilled with step ks + SM_STAGES - 1)
     for (int ks = 0; ks < nk; ++ks) {
-        const int cur = ks & (SM_STAGES - 1);
-        // this wave's loads of stage `cur` have landed once only the younger stages (two of four, one of two) are in flight
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SM_STAGES / 2) * LOADS_PER_STAGE) : "memory");
-        A8W8_RAW_BARRIER();                 // ... everyone's have; and (four stages) everyone is done reading the stage of step ks-1
-        if constexpr (SM_STAGES == 4) issue_stage((ks + 3) & 3, ks + 3);
+        // this wave's loads of stage `cur` have landed once only the younger stages are in flight
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(YOUNGER * LOADS_PER_STAGE) : "memory");
+        A8W8_RAW_BARRIER();                 // ... everyone's have; and (more than two stages) everyone is done reading the stage of step ks-1
+        if constexpr (SM_STAGES > 2) issue_stage(refill, ks + SM_STAGES - 1);
 
         v8i fa[SM_TM], fb[2];
 #pragma unroll
@@ -223,7 +243,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
                 for (int t = 0; t < SM_TM; ++t) mx_sa[t] = (int)__builtin_amdgcn_ubfe(sc[wave_m * 64 + 16 * t + r16], 8 * g, 8);
 #pragma unroll
-                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe(sc[128 + wave_n * 64 + 16 * t + r16], 8 * g, 8);
+                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe(sc[128 + wave_n * (SM_BN / 2) + 16 * t + r16], 8 * g, 8);
             }
             if constexpr (MODE == MODE_F4T) {
                 // both halves' bytes sit side by side: one 16-bit read, the half is chosen by op_sel
@@ -231,14 +251,14 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
                 for (int t = 0; t < SM_TM; ++t) mx_sa[t] = *(const unsigned short*)(sc + wave_m * 1024 + mxt_off[t]);
 #pragma unroll
-                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = *(const unsigned short*)(sc + (2 + wave_n) * 1024 + mxt_off[t]);
+                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = *(const unsigned short*)(sc + mxt_unit_b + mxt_off_b[t]);
             }
             if constexpr (MODE == MODE_MXT) {
                 const uint8_t* sc = (const uint8_t*)(smem + SM_STAGES * SM_STAGE_BYTES + cur * SM_SCALE_BYTES) + (ks & 1);
 #pragma unroll
                 for (int t = 0; t < SM_TM; ++t) mx_sa[t] = sc[wave_m * 1024 + mxt_off[t]];
 #pragma unroll
-                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = sc[(2 + wave_n) * 1024 + mxt_off[t]];
+                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = sc[mxt_unit_b + mxt_off_b[t]];
             }
 #pragma unroll
             for (int j = 0; j < SM_TN; ++j) {
@@ -292,6 +312,8 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
             A8W8_RAW_BARRIER();
             issue_stage(cur, ks + 2);
         }
+        refill = cur;
+        cur = cur + 1 == SM_STAGES ? 0 : cur + 1;
     }
 
     // ---- epilogue: dequantise in fp32, convert, store

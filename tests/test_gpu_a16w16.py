@@ -18,7 +18,9 @@ def _rand(m, k, seed):
     return torch.randn((m, k), generator=gen, device="cuda").to(torch.bfloat16)
 
 
-@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 384, 1024), (130, 270, 192), (64, 64, 4096), (300, 520, 64 * 7)])
+# (the last two: short and wide with a long K loop, which the 128-tile kernel runs on 128 x 64 tiles)
+@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 384, 1024), (130, 270, 192), (64, 64, 4096), (300, 520, 64 * 7),
+                                   (200, 1088, 1024), (256, 320, 1088)])
 def test_pipelined_kernel(orc, shape):
     m, n, k = shape
     a, b = _rand(m, k, 1 + m), _rand(n, k, 2 + n)

@@ -48,7 +48,9 @@ def test_general_kernel_is_bit_exact(orc, shape):
     assert (got == ref).all()
 
 
-@pytest.mark.parametrize("shape", [(256, 256, 512), (512, 256, 2048), (130, 270, 1024), (300, 520, 768)])
+# (the last two: short and wide with a long K loop, which the 128-tile kernel runs on 128 x 64 tiles)
+@pytest.mark.parametrize("shape", [(256, 256, 512), (512, 256, 2048), (130, 270, 1024), (300, 520, 768),
+                                   (200, 1088, 4096), (256, 320, 4352)])
 def test_pipelined_kernel(orc, shape):
     m, n, k = shape
     qa, ea = orc.quantize_mxfp4(_x(m, k, 21 + m))

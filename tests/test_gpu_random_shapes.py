@@ -56,6 +56,26 @@ def test_random_case(case, shuffled):
     # small problems run on 128 x 128 tiles; many batch entries of a small shape put the same ragged tiles on the 256 x 256 kernels
     batch = int(r.choice([1, 1, 2, 3, 70, 140])) if m <= 300 and n <= 300 else int(r.choice([1, 1, 2, 3]))
     c_dtype = [g.BF16, g.FP32][int(r.integers(0, 2))]
+    _exact_case(r, f"case {case}", mode, batch, m, n, k, c_dtype, shuffled)
+
+
+@pytest.mark.parametrize("shuffled", [False, True], ids=["row_major_b", "shuffled_b"])
+@pytest.mark.parametrize("mode", [g.TENSOR, g.ROWCOL, g.BLOCK, g.MX, g.MX_TILED])
+@pytest.mark.parametrize("m,n,k,batch", [(130, 320, 2048, 1), (256, 1152, 2176, 1), (200, 128, 2304, 3), (257, 2048, 2048, 1)])
+def test_short_wide_problems_on_narrow_tiles(m, n, k, batch, mode, shuffled):
+    """A few hundred rows, a long K loop and so few 128 x 128 tiles that half of the compute units would idle: the
+    128-tile kernel takes 128 x 64 tiles and five or six LDS stages (step counts that are and are not multiples of
+    the stage count; a ragged last tile column; three M tiles)."""
+    r = np.random.default_rng(9900 + m + n + k + 7 * mode)
+    if mode == g.BLOCK:
+        n = max(128, n // 128 * 128)            # block scales need N in whole blocks
+    args = g.raw_gemm_args(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, m, n, k, mode, batch=batch, b_preshuffled=int(shuffled))
+    assert g.kernel_name(args) == "gemm_a8w8_tile128"
+    for c_dtype in (g.BF16, g.FP32):
+        _exact_case(r, "narrow tiles", mode, batch, m, n, k, c_dtype, shuffled)
+
+
+def _exact_case(r, label, mode, batch, m, n, k, c_dtype, shuffled):
     a = r.integers(-4, 5, (batch, m, k)).astype(np.float32)
     b = r.integers(-4, 5, (batch, n, k)).astype(np.float32)
     qa, qb = oracle.encode(a), oracle.encode(b)
@@ -89,7 +109,7 @@ def test_random_case(case, shuffled):
         tiles = [g.mx_tile_scales_ab(dsa[i], dsb[i]) for i in range(batch)]
         dsa = torch.stack([t[0] for t in tiles])
         dsb = torch.stack([t[1] for t in tiles])
-    what = f"case {case}{' (shuffled B)' if shuffled else ''}: mode {mode} {batch}x{m}x{n}x{k} c={c_dtype} lda={da.stride(-2)} ldb={db.stride(-2)} ldc={c_view.stride(-2)}"
+    what = f"{label}{' (shuffled B)' if shuffled else ''}: mode {mode} {batch}x{m}x{n}x{k} c={c_dtype} lda={da.stride(-2)} ldb={db.stride(-2)} ldc={c_view.stride(-2)}"
     print(what, flush=True)
     if batch == 1:
         g.gemm(da[0], db[0], dsa[0], dsb[0], mode, c=c_view[0], n=n if shuffled else None)
