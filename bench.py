@@ -164,9 +164,20 @@ def time_best_of(torch, fn, steps, warmup, rounds=3):
     return best
 
 
-def run_workload(name, torch, g, steps, warmup, seed, headline=True):
+def run_workload(name, torch, g, steps, warmup, seed, headline=True, operands="as_configured"):
     mode, m, n, k, abytes = WORKLOADS[name]
     inp = make_inputs(name, torch, g, seed)
+    if operands == "zeros":
+        # the same launch on operands that toggle nothing: what the schedule alone allows (a measurement aid)
+        inp["a"].zero_()
+        inp["b"].zero_()
+    elif operands == "random_bytes":
+        # full-entropy operand bytes (the two NaN codes of E4M3 mapped to finite values)
+        for t in (inp["a"], inp["b"]):
+            r = torch.randint(0, 256, t.shape, device="cuda", dtype=torch.int16).to(torch.uint8)
+            r[(r & 0x7F) == 0x7F] = 0x3C
+            t.copy_(r)
+            del r
     flops = 2.0 * m * n * k
     c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     res = {"workload": name, "m": m, "n": n, "k": k}
@@ -486,6 +497,8 @@ def main():
     ap.add_argument("--seed", type=int, default=0xA8A80004)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="time only the selected workload")
+    ap.add_argument("--operands", default="as_configured", choices=["as_configured", "zeros", "random_bytes"],
+                    help="measurement aid: replace the selected workload's quantised operands (the result is then not the configuration's)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -497,7 +510,7 @@ def main():
     g.lib()     # raises if the HIP library has not been built; there is no fallback path
     torch.cuda.set_device(0)
 
-    res, inp, c = run_workload(args.workload, torch, g, args.steps, args.warmup, args.seed)
+    res, inp, c = run_workload(args.workload, torch, g, args.steps, args.warmup, args.seed, operands=args.operands)
     mode, m, n, k, abytes = WORKLOADS[args.workload]
     if mode == "flat":
         value, unit = res["gbs"], "GB/s"
@@ -518,6 +531,10 @@ def main():
                    "algorithmic_bytes": abytes, "flop": 2 * m * n * k},
         "roofline": roof,
     }
+    if args.operands != "as_configured" or g.lib().a8w8_version() < 0 or os.environ.get("MI355_A8W8_LIBRARY"):
+        # a measurement run: other operand contents, or a library built with measurement switches
+        line["config"]["measurement_run"] = {"operands": args.operands, "library": g.library_path(),
+                                             "library_version": g.lib().a8w8_version()}
     for key in ("step", "ms_gemm_kernel", "tflops_gemm_kernel", "ms_row_major_scales_one_launch",
                 "tflops_row_major_scales_one_launch", "first_region_ms_per_step", "first_region_tflops"):
         if key in res:

@@ -10,7 +10,9 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_SO = os.path.join(_HERE, "libmi355a8w8.so")
+# MI355_A8W8_LIBRARY: another build of the same sources (a measurement build made with `make EXTRA=-D... OUT=...`),
+# for A/B timings of one program against two libraries; unset, the library next to this file
+_SO = os.environ.get("MI355_A8W8_LIBRARY") or os.path.join(_HERE, "libmi355a8w8.so")
 
 TENSOR, ROWCOL, BLOCK, MX, MX_TILED = 0, 1, 2, 3, 4
 BF16, FP32 = 0, 1

@@ -24,6 +24,31 @@
 
 #include "gemm_persist.hpp"
 
+// Measurement switches (all off in the library that ships): each removes one ingredient of the K loop so that its
+// cost can be read off a timing of the same launch.  The results of an ablated build are wrong by construction.
+//   A8W8_ABLATE_OPERAND_LOADS   the loop issues no A/B loads (the two stages keep what the prologue brought)
+//   A8W8_ABLATE_SCALE_LOADS     tiled MX: no scale bytes are fetched after the first batch
+//   A8W8_ABLATE_HOT_SCALES      tiled MX: every batch re-reads the tile's first batch (lines that are already in L2)
+//   A8W8_ABLATE_SCALE_READS     tiled MX: the scale registers are not refreshed from LDS
+//   A8W8_ABLATE_UNSCALED_MFMA   tiled MX: the plain form of the MFMA in place of the scaled one
+//   A8W8_ABLATE_STORES          whole tiles are neither converted nor written (the accumulators are still read out)
+//   A8W8_ABLATE_STORE_INSTRUCTIONS   whole tiles are read out and converted, only the store instructions are left out (bf16)
+// and three that keep the results right:
+//   A8W8_WIDE_WRITE_THROUGH=0   bf16 tiles are stored write-back instead of written through
+//   A8W8_WIDE_BURST_EPILOGUE    every tile is written after its last K step in one burst (the path of the edge tiles)
+//   A8W8_WIDE_STAGGER=n         workgroups start up to 7 n 64 clocks apart
+#if defined(A8W8_ABLATE_OPERAND_LOADS) || defined(A8W8_ABLATE_SCALE_LOADS) || defined(A8W8_ABLATE_HOT_SCALES) || \
+    defined(A8W8_ABLATE_SCALE_READS) || defined(A8W8_ABLATE_UNSCALED_MFMA) || defined(A8W8_ABLATE_STORES) || \
+    defined(A8W8_ABLATE_STORE_INSTRUCTIONS)
+#define A8W8_ABLATED 1
+#else
+#define A8W8_ABLATED 0
+#endif
+
+#ifndef A8W8_WIDE_WRITE_THROUGH
+#define A8W8_WIDE_WRITE_THROUGH 1
+#endif
+
 namespace a8w8 {
 
 constexpr int WIDE_THREADS = 256;
@@ -329,11 +354,19 @@ gemm_a8w8_wide(PersistParams pp)
             constexpr int ES = CDT == C_BF16 ? 2 : 4;
             constexpr int row = PERM_A ? 32 * (i >> 1) + 4 * (i & 1) : 16 * i;
             const int voff = ep_lane_off + 32 * jp * ES, soff = (int)((uint32_t)row * (uint32_t)ep_row_bytes);
+#ifdef A8W8_ABLATE_STORES
+            asm volatile("" ::"v"(v[0]), "v"(v[7]), "s"(voff), "s"(soff));
+            return;
+#endif
             if constexpr (CDT == C_BF16) {
                 v4i w;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
-                store_c_16<true>(ep_rs, w, voff, soff);
+#ifdef A8W8_ABLATE_STORE_INSTRUCTIONS
+                asm volatile("s_nop 1" ::"v"(w), "s"(voff), "s"(soff));      // everything but the store itself
+#else
+                store_c_16<A8W8_WIDE_WRITE_THROUGH != 0>(ep_rs, w, voff, soff);
+#endif
             } else {
                 (void)voff;
                 store_c_lines(ep_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}),
@@ -387,6 +420,10 @@ gemm_a8w8_wide(PersistParams pp)
     // ---------------------------------------------------------------- prologue
     const int my_items = (pp.items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
     if (my_items == 0) return;
+#ifdef A8W8_WIDE_STAGGER
+    // measurement: workgroups start up to 7 * A8W8_WIDE_STAGGER * 64 clocks apart, so that their tiles do not all end at once
+    for (int i = (int)((blockIdx.x * 0x9E37u >> 6) & 7u); i > 0; --i) __builtin_amdgcn_s_sleep(A8W8_WIDE_STAGGER);
+#endif
     point_loads_at(ld_item);
     point_compute_at(cur_item);
     point_scales_at(sf_cur, cur_item);
@@ -470,7 +507,11 @@ gemm_a8w8_wide(PersistParams pp)
                 const v4i ah = hf ? v4i{fa[i][4], fa[i][5], fa[i][6], fa[i][7]} : v4i{fa[i][0], fa[i][1], fa[i][2], fa[i][3]};
                 mfma_acc_bf16<lo, z>(bh, ah);
             } else if constexpr (IS_MXT) {
+#ifdef A8W8_ABLATE_UNSCALED_MFMA
+                mfma_acc<lo, z>(fb[j], fa[i]);
+#else
                 mfma_acc_mx<lo, z, 2 * (j & 1) + sp, 2 * (i & 1) + sp>(fb[j], fa[i], sc_b[j >> 2][(j >> 1) & 1], sc_a[i >> 2][(i >> 1) & 1]);
+#endif
             } else {
                 mfma_acc<lo, z>(fb[j], fa[i]);
             }
@@ -481,11 +522,17 @@ gemm_a8w8_wide(PersistParams pp)
                 constexpr int off = (f >> 1) * (32 * BK) + par * (ref < 2 ? A_PAR_BYTES : B_PAR_BYTES);
                 half[r] = *(const v4i*)(smem + (rs * HALF_STAGE + off) + base[par ^ h]);
             }
+#ifndef A8W8_ABLATE_OPERAND_LOADS
             if constexpr (sl % (4 * MPF) == 2 * MPF) issue_one(ls, lq, sl / (4 * MPF));
+#endif
             if constexpr (IS_MXT && SCR && sl % (4 * MPF) == 0) {
                 // the next pair's scales, four 8-byte reads spread over the quadrant
                 constexpr int u = sl / (4 * MPF);
+#ifdef A8W8_ABLATE_SCALE_READS
+                const v2i v = u < 2 ? sc_a[u] : sc_b[u - 2];
+#else
                 const v2i v = *(const v2i*)(smem + sc_rd_off + (u < 2 ? rd_sfa : rd_sfb) + (u & 1) * 1024);
+#endif
                 if constexpr (u < 2) sc_a_next[u] = v;
                 else sc_b_next[u - 2] = v;
             }
@@ -517,7 +564,11 @@ gemm_a8w8_wide(PersistParams pp)
     // finished: N = the 16 loads of the last four quadrants plus the stores issued among them, so that
     // what has finished is exactly the two quarters the next two quadrants read.
     auto handover = [&](auto STORES) __attribute__((always_inline)) {
+#if defined(A8W8_ABLATE_STORES) || defined(A8W8_ABLATE_STORE_INSTRUCTIONS)
+        constexpr int want = 16;      // no stores are issued: the newest 16 operations are the loads
+#else
         constexpr int want = 16 + decltype(STORES)::value * STORES_PER_PIECE;
+#endif
         constexpr int n = want < 63 ? want : 63;             // a 6-bit counter; fewer is only stricter
         __builtin_amdgcn_s_waitcnt(((n & 15) | ((n >> 4) << 14)) | 0x0070);
         A8W8_RAW_BARRIER();
@@ -604,8 +655,14 @@ gemm_a8w8_wide(PersistParams pp)
                 // first of the next tile) into the other buffer; its first pair is read steps from here
                 if (ks % BATCH_STEPS == 0) {
                     const int b1 = ks / BATCH_STEPS + 1;
+#if defined(A8W8_ABLATE_SCALE_LOADS)
+                    (void)b1;
+#elif defined(A8W8_ABLATE_HOT_SCALES)
+                    issue_mx_batch(sf_cur, 0, (cur_bbase + b1) & 1);
+#else
                     if (b1 < batches_per_tile) issue_mx_batch(sf_cur, b1, (cur_bbase + b1) & 1);
                     else issue_mx_batch(sf_next, 0, (cur_bbase + batches_per_tile) & 1);
+#endif
                 }
             }
             // where the scales of the pair that starts at tile step `first` live (past the end: the next
@@ -633,7 +690,11 @@ gemm_a8w8_wide(PersistParams pp)
                 const uintptr_t c_addr = (uintptr_t)p.c + (uintptr_t)((long long)cur_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4));
                 ep_vec_ok = (p.ldc & (CDT == C_BF16 ? 7 : 3)) == 0 && (c_addr & 15) == 0;
                 // pieces are written without checks: only for whole tiles with aligned rows
+#ifdef A8W8_WIDE_BURST_EPILOGUE
+                const bool fast = false;      // measurement: every tile is written after its last step, in one burst
+#else
                 const bool fast = ep_vec_ok && m0 + BM <= p.m && n0 + BN <= p.n;
+#endif
                 {
                     constexpr int ES = CDT == C_BF16 ? 2 : 4;
                     ep_rs = make_rsrc((const char*)c_addr + ((long long)m0 * p.ldc + n0) * ES, (uint32_t)((BM - 1) * p.ldc + BN) * ES);
