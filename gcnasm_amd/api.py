@@ -101,6 +101,7 @@ def lib():
         L.a8w8_version.restype = ctypes.c_int
         L.a8w8_init.argtypes = [ctypes.c_int]
         L.a8w8_hbm_read_probe.argtypes = [vp, ctypes.c_size_t, vp, vp]
+        L.a8w8_route_override.argtypes = [ctypes.c_int]
         _lib = L
     return _lib
 

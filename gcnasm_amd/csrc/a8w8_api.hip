@@ -446,39 +446,54 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 
 // On shuffled weights both the flat GEMM and the MFMA kernels can run a skinny problem; the entry points take the
 // one a small cost model calls faster.  Times in microseconds, W = weight bytes, row_bytes = bytes of one weight row:
-//   flat:  one pass over the weights at ~6.3 TB/s; every further group of 16 activation rows adds ~2 us of
-//          activation traffic and MFMA work (the scale bytes of MXFP8 add about a tenth).
-//   dense: the 128-tile kernel has only n/128 workgroups to pull the weights with, ~28 GB/s each (128 rows a
-//          workgroup), and ~5 TB/s at best over the chip.
-// Weights of at most 32 MiB always go flat.  Measured on MI355X, M = 16 / 32 / 48 / 64, flat against dense:
-//   16384 x 7168   FP8 21 / 21 / 23 / 24 against 37-40, MXFP8 20 / 22 / 24 / 27 against 38-41,
-//                  MXFP4 12 / 13 / 14 / 20 against 21-22, bf16 37 / 38 / 41 / 45 against 66-72
-//   8192 x 8192    FP8 13 / 14 / 16 / 18 against 40-41 (64 workgroups on the dense side)
-//   28672 x 4096   FP8 21 / 23 / 26 / 28 against 26-27, MXFP8 22 / 25 / 28 / 29 against 26-28,
-//                  MXFP4 13 / 16 / 17 / 25 against 15-16, bf16 43 / 43 / 48 / 52 against 47-48
-// The model takes the faster side in these except where the two are within ~8% of each other.
+//   flat:  one pass over the weights at ~6.4 TB/s; every further group of 16 activation rows adds the activation rows
+//          that each workgroup reads again for its weight tiles, W / NT bytes at ~21 TB/s (1.4 us on 16384 x 7168), and
+//          the scale bytes of MXFP8 about a tenth; a second pass (more than 64 rows over at least four weight tiles
+//          per compute unit) reads the weights from L2 and costs 55% more.
+//   dense: the 128-tile kernel pulls the weights with one workgroup per 128 weight rows at ~28 GB/s each, or, where
+//          128 x 128 tiles would occupy at most half of the compute units, per 64 rows at ~22 GB/s each (its 128 x 64
+//          tiles), ~5 TB/s at best over the chip; 20% more at 128 activation rows than at a few.
+// Weights of at most 32 MiB always go flat.  Measured on MI355X, shuffled FP8 weights, M = 16 / 32 / 48 / 64 / 80 / 96 /
+// 128, flat against dense:
+//   16384 x 7168   20 / 21 / 23 / 24 / 35 / 36 / 41  against  30 / 27 / 27 / 28 / 30 / 31 / 33   (MXFP8 about 10% more on both sides)
+//   8192 x 8192    13 / 14 / 16 / 18 / 20 / 21 / 26  against  26 / 26 / 26 / 27 / 28 / 29 / 31
+//   28672 x 4096   20 / 23 / 25 / 28 / 39 / 41 / 47  against  26 / 26 / 27 / 28 / 29 / 30 / 31
+//   4096 x 14336   13 / 19 / 23 / 26 / 31 / 32 / 38  against  41 throughout
+// (tests/test_gpu_routing.py times both sides of such cells through a8w8_route_override and checks the choice).
 // Row-major weights (a8w8_gemm without b_preshuffled; the flat kernel stages the weight rows through LDS, whole lines
 // per load): as fast as shuffled ones unless the rows are a large power of two apart, where the 16 rows of a tile fall
 // on the same memory channels -- 16384 x 7168 FP8 M = 16 / 32 / 64: 20 / 21 / 25 us, 8192 x 8192: 17 / 17 / 20 us
 // (13 / 14 / 18 shuffled).
+int g_route = A8W8_ROUTE_MODEL;      // a8w8_route_override
+
 bool prefer_flat(int m, int n, long long row_bytes, bool scaled_in_loop, double layout_factor = 1.0)
 {
+    if (g_route != A8W8_ROUTE_MODEL) return g_route == A8W8_ROUTE_FLAT;
     const double w = (double)n * (double)row_bytes;
     if (w <= (double)(32ll << 20)) return true;
     const int groups = (m + 15) / 16, passes = (groups + 3) / 4;
     const int mt = (groups + passes - 1) / passes;
     const int cus = num_cus();
     const int rounds = ((n + 127) / 128 + cus - 1) / cus;
-    double flat;
-    if (groups > 4 && n / 16 < 4 * cus && (groups <= 6 || !scaled_in_loop)) {
-        flat = 3.5 + w / 6.3e6 + 2.0 * (groups - 1);      // one pass with six or eight row groups (see launch_flat)
+    // one pass over the weights, plus, for every further group of 16 activation rows, the activation rows each
+    // workgroup reads again for its NT weight tiles (n * row_bytes / NT bytes from L2) and their MFMAs; nearly twice
+    // that where the workgroups do not fit the chip at once
+    const long long tiles = n / 16;
+    const int nt = tiles >= 4ll * cus ? 4 : tiles >= 2ll * cus ? 2 : 1;
+    const double per_group = w / nt / 21.0e6 * (tiles / nt > cus ? 1.9 : 1.0);
+    double flat = 1.5 + w / 6.4e6;
+    if (groups > 4 && tiles < 4ll * cus && (groups <= 6 || !scaled_in_loop)) {
+        flat += per_group * (groups - 1);      // one pass with six or eight row groups (see launch_flat)
     } else {
-        flat = 3.5 + w / 6.3e6 + 2.0 * (mt - 1);
+        flat += per_group * (mt - 1);
         if (passes == 2) flat *= 1.55;      // the second pass reads the weights from L2
     }
     flat *= layout_factor;      // row-major weights: rows staged through LDS, rows a power of two apart share channels
-    double dense = 4.0 + std::max(rounds * 128.0 * (double)row_bytes / 28.0e3, w / 5.0e6);
-    if (m > 64) dense *= 1.0 + 0.25 * (m - 64) / 64.0;
+    // (the 128-tile kernel's own choice of tile width, narrow_tiles_pay, for one row of 128-row tiles)
+    const bool narrow = narrow_tiles_pay((n + 127) / 128, n, (int)std::min<long long>(row_bytes, 1 << 30));
+    const double per_workgroup = narrow ? 64.0 * (double)row_bytes / 22.0e3 : rounds * 128.0 * (double)row_bytes / 28.0e3;
+    double dense = 4.0 + std::max(per_workgroup, w / 5.0e6);
+    dense *= 1.0 + 0.2 * m / 128.0;
     return flat <= dense;
 }
 
@@ -486,7 +501,8 @@ bool prefer_flat_fp8(const a8w8_gemm_args* g)
 {
     const bool scaled_in_loop = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;      // no kernel with eight row groups
     const double layout_factor = g->b_preshuffled ? 1.0 : g->stride_b % 4096 == 0 ? 1.3 : 1.05;
-    return prefer_flat(g->m, g->n, g->k, scaled_in_loop, layout_factor);
+    // (the flat kernel's MX scale bytes, one byte load per weight tile and K pair, cost it about a tenth)
+    return prefer_flat(g->m, g->n, g->k, scaled_in_loop, layout_factor * (scaled_in_loop ? 1.1 : 1.0));
 }
 
 template <bool BROW>
@@ -1158,6 +1174,14 @@ int a8w8_hbm_read_probe(const void* src, size_t bytes, void* sink, void* hip_str
     const unsigned grid = (unsigned)(want < most ? want : most);
     return launch(hbm_read_probe_kernel, dim3(grid), dim3(HBM_PROBE_THREADS), 0, (hipStream_t)hip_stream, (const v4i*)src, n16,
                   (int*)sink);
+}
+
+int a8w8_route_override(int choice)
+{
+    if (choice != A8W8_ROUTE_MODEL && choice != A8W8_ROUTE_FLAT && choice != A8W8_ROUTE_DENSE) return A8W8_ERR_BAD_MODE;
+    const int before = g_route;
+    g_route = choice;
+    return before;
 }
 
 int a8w8_init(int device)

@@ -158,5 +158,14 @@ A8W8_DEV unsigned short bf16_bits(float f)
     __bf16 h = (__bf16)f;
     return __builtin_bit_cast(unsigned short, h);
 }
+// Two at once, `lo` in the low half of the word: one v_cvt_pk_bf16_f32.  (Built from two bf16_bits the compiler
+// converts each value with an instruction of its own and joins them with a shift and an or: six instructions for
+// two values, which in an epilogue that runs beside the MFMAs is what the MFMAs end up waiting for.)
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+A8W8_DEV int bf16x2_bits(float lo, float hi)
+{
+    return __builtin_bit_cast(int, __builtin_convertvector((v2f{lo, hi}), v2bf));
+}
 
 }  // namespace a8w8

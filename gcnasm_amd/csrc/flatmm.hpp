@@ -471,7 +471,7 @@ __global__ void __launch_bounds__(FLAT_THREADS) flatmm_a8w8(GemmParams p)
             if constexpr (CDT == C_BF16) {
                 unsigned short* dst = (unsigned short*)p.c + ci;
                 if ((ldc & 3) == 0 && (((uintptr_t)p.c + 2 * c_batch_off) & 7) == 0) {
-                    *(v4u16*)dst = v4u16{bf16_bits(s.x), bf16_bits(s.y), bf16_bits(s.z), bf16_bits(s.w)};
+                    *(v2i*)dst = v2i{bf16x2_bits(s.x, s.y), bf16x2_bits(s.z, s.w)};
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dst[e] = bf16_bits(s[e]);

@@ -350,7 +350,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         auto packed_bf16 = [&](const float (&v)[8]) __attribute__((always_inline)) {
             v4i w;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+            for (int e = 0; e < 4; ++e) w[e] = bf16x2_bits(v[2 * e], v[2 * e + 1]);
             return w;
         };
         if (whole) {
@@ -386,7 +386,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                         v4i w;
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+                            w[e] = bf16x2_bits(v[2 * e], v[2 * e + 1]);
                         A8W8_STORE_C((v4i*)dst, w);
                     } else {
 #pragma unroll

@@ -344,8 +344,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
             if constexpr (MODE == MODE_ROWCOL) v *= sb * sa[i];
             if (whole) {        // inside the matrix, aligned rows: no per-lane checks
                 if constexpr (CDT == C_BF16)
-                    A8W8_STORE_C((v4u16*)((unsigned short*)c_base + (long long)cm * p.ldc + cn),
-                                 (v4u16{bf16_bits(v.x), bf16_bits(v.y), bf16_bits(v.z), bf16_bits(v.w)}));
+                    A8W8_STORE_C((v2i*)((unsigned short*)c_base + (long long)cm * p.ldc + cn), (v2i{bf16x2_bits(v.x, v.y), bf16x2_bits(v.z, v.w)}));
                 else
                     A8W8_STORE_C((v4f*)((float*)c_base + (long long)cm * p.ldc + cn), v);
                 continue;
@@ -354,7 +353,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
             if constexpr (CDT == C_BF16) {
                 unsigned short* dst = (unsigned short*)c_base + (long long)cm * p.ldc + cn;
                 if (vec_ok && cn + 3 < p.n) {
-                    A8W8_STORE_C((v4u16*)dst, (v4u16{bf16_bits(v.x), bf16_bits(v.y), bf16_bits(v.z), bf16_bits(v.w)}));
+                    A8W8_STORE_C((v2i*)dst, (v2i{bf16x2_bits(v.x, v.y), bf16x2_bits(v.z, v.w)}));
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)

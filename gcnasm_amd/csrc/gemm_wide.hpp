@@ -361,7 +361,7 @@ gemm_a8w8_wide(PersistParams pp)
             if constexpr (CDT == C_BF16) {
                 v4i w;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+                for (int e = 0; e < 4; ++e) w[e] = bf16x2_bits(v[2 * e], v[2 * e + 1]);
 #ifdef A8W8_ABLATE_STORE_INSTRUCTIONS
                 asm volatile("s_nop 1" ::"v"(w), "s"(voff), "s"(soff));      // everything but the store itself
 #else
@@ -381,7 +381,7 @@ gemm_a8w8_wide(PersistParams pp)
             if (vec) {
                 v4i w;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = (int)bf16_bits(v[2 * e]) | ((int)bf16_bits(v[2 * e + 1]) << 16);
+                for (int e = 0; e < 4; ++e) w[e] = bf16x2_bits(v[2 * e], v[2 * e + 1]);
                 A8W8_STORE_C((v4i*)dst, w);
             } else {
 #pragma unroll

@@ -254,6 +254,15 @@ A8W8_API const char* a8w8_kernel_name(const a8w8_gemm_args* args);
  * bandwidth_memread/bandwidth_kernel.cu:68-92.  bytes % 16 == 0, src_dev 16-byte aligned. */
 A8W8_API int a8w8_hbm_read_probe(const void* src_dev, size_t bytes, void* sink_dev, void* hip_stream);
 
+/* Measurement aid, no counterpart in the reference (its flat GEMM and its tile GEMM are separate programs): for a
+ * skinny problem (m <= 128) both the flat kernel and the MFMA tile kernels can run, and the entry points choose
+ * with a small cost model.  choice = A8W8_ROUTE_FLAT / A8W8_ROUTE_DENSE makes every later call in this process
+ * take that side wherever both can run the problem, A8W8_ROUTE_MODEL (the default) restores the model.  For
+ * timing the two sides against each other; a process-wide setting, not meant to be changed while other threads
+ * are inside the library.  Returns the previous choice, or A8W8_ERR_BAD_MODE for an unknown one. */
+enum { A8W8_ROUTE_MODEL = 0, A8W8_ROUTE_FLAT = 1, A8W8_ROUTE_DENSE = 2 };
+A8W8_API int a8w8_route_override(int choice);
+
 /* Optional explicit set-up of one device (device < 0: the current one): queries its architecture and
  * compute-unit count and raises the dynamic-LDS limit of every kernel variant.  The same work happens,
  * once per device and thread-safely, inside the first entry point called with that device current; call

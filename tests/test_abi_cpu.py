@@ -123,9 +123,12 @@ def test_gemm_on_shuffled_weights_preconditions():
     assert g.kernel_name(_ok_args(m=64, mode=g.MX_TILED, **big)) == "flatmm_a8w8"
     wide = dict(n=28672, k=4096, b_preshuffled=1)                # 224 workgroups on the 128-tile kernel, short rows
     assert g.kernel_name(_ok_args(m=48, mode=g.ROWCOL, **wide)) == "flatmm_a8w8"
-    assert g.kernel_name(_ok_args(m=64, mode=g.ROWCOL, **wide)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(m=96, mode=g.ROWCOL, **wide)) == "gemm_a8w8_tile128"       # (at 64 rows the two are level)
     assert g.kernel_name(_ok_args(m=48, mode=g.MX_TILED, **wide)) == "flatmm_a8w8"
     assert g.kernel_name(_ok_args(m=64, mode=g.MX_TILED, **wide)) == "gemm_a8w8_tile128"
+    # past 64 rows the flat kernel makes two passes over weights of this size: the 128-tile kernel's 128 x 64 tiles win
+    assert g.kernel_name(_ok_args(m=96, mode=g.ROWCOL, **big)) == "gemm_a8w8_tile128"
+    assert g.kernel_name(_ok_args(m=128, mode=g.MX_TILED, **big)) == "gemm_a8w8_tile128"
     assert g.kernel_name(_ok_args(m=64, n=4096, k=4096, mode=g.ROWCOL, b_preshuffled=1)) == "flatmm_a8w8"
     assert g.kernel_name(_ok_args(m=64, n=16384, k=7104, mode=g.ROWCOL, b_preshuffled=1)) == "flatmm_a8w8"   # K % 128 != 0: flat only
     for mutate, want in [(lambda x: setattr(x, "n", 4088), -3), (lambda x: setattr(x, "k", 448), -3),
