@@ -20,6 +20,7 @@
 //  * Loads complete in issue order: "all but the newest 16" at a barrier is "the two quarters the
 //    next two quadrants read have landed".
 #pragma once
+#include <type_traits>
 #include <utility>
 
 #include "gemm_persist.hpp"
@@ -35,7 +36,8 @@
 //   A8W8_ABLATE_STORE_INSTRUCTIONS   whole tiles are read out and converted, only the store instructions are left out (bf16)
 // and three that keep the results right:
 //   A8W8_WIDE_WRITE_THROUGH=0   bf16 tiles are stored write-back instead of written through
-//   A8W8_WIDE_BURST_EPILOGUE    every tile is written after its last K step in one burst (the path of the edge tiles)
+//   A8W8_WIDE_BURST=0           the tile is written out in pieces among the MFMAs of its last K step and of the next
+//                               tile's first quadrant, instead of in one burst between the two steps
 //   A8W8_WIDE_STAGGER=n         workgroups start up to 7 n 64 clocks apart
 #if defined(A8W8_ABLATE_OPERAND_LOADS) || defined(A8W8_ABLATE_SCALE_LOADS) || defined(A8W8_ABLATE_HOT_SCALES) || \
     defined(A8W8_ABLATE_SCALE_READS) || defined(A8W8_ABLATE_UNSCALED_MFMA) || defined(A8W8_ABLATE_STORES) || \
@@ -47,6 +49,9 @@
 
 #ifndef A8W8_WIDE_WRITE_THROUGH
 #define A8W8_WIDE_WRITE_THROUGH 1
+#endif
+#ifndef A8W8_WIDE_BURST
+#define A8W8_WIDE_BURST 1
 #endif
 
 namespace a8w8 {
@@ -576,6 +581,8 @@ gemm_a8w8_wide(PersistParams pp)
     using S0 = std::integral_constant<int, 0>;
     using S8 = std::integral_constant<int, 8>;
     using S24 = std::integral_constant<int, 24>;
+    using SALL = std::integral_constant<int, 32>;      // the whole tile's pieces (one wave's share)
+    constexpr bool BURST = A8W8_WIDE_BURST != 0;
 
     // A K step.  FIRST: the tile's first step (even): accumulators start from zero, and the previous
     // tile's last quadrant is written out behind the first 16 MFMAs.  LAST: the tile's last step
@@ -592,11 +599,11 @@ gemm_a8w8_wide(PersistParams pp)
         using Z = std::integral_constant<int, FIRST ? 1 : 0>;
         if constexpr (P == 0) {
             // aL x bL | read bH of this step | load aL            (| write out aH x bH of the previous tile)
-            quad(I0{}, I0{}, I3{}, SP{}, I0{}, SP{}, I0{}, SP{}, I0{}, Z{}, std::integral_constant<int, FIRST ? 4 : 0>{}, I0{});
+            quad(I0{}, I0{}, I3{}, SP{}, I0{}, SP{}, I0{}, SP{}, I0{}, Z{}, std::integral_constant<int, FIRST && !BURST ? 4 : 0>{}, I0{});
             // aL x bH | read aH of this step | load bL
             quad(I0{}, I4{}, I1{}, SP{}, I2{}, SP{}, I0{}, SP{}, I0{}, Z{}, I0{}, I0{});
             if constexpr (FIRST) {
-                if (have_prev) handover(S24{});
+                if (have_prev) handover(std::conditional_t<BURST, SALL, S24>{});
                 else handover(S0{});
             } else {
                 handover(S0{});
@@ -614,7 +621,7 @@ gemm_a8w8_wide(PersistParams pp)
                 }
             }
             if constexpr (FIRST) {
-                if (have_prev) handover(S8{});
+                if (have_prev) handover(std::conditional_t<BURST, SALL, S8>{});
                 else handover(S0{});
             } else {
                 handover(S0{});
@@ -690,11 +697,7 @@ gemm_a8w8_wide(PersistParams pp)
                 const uintptr_t c_addr = (uintptr_t)p.c + (uintptr_t)((long long)cur_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4));
                 ep_vec_ok = (p.ldc & (CDT == C_BF16 ? 7 : 3)) == 0 && (c_addr & 15) == 0;
                 // pieces are written without checks: only for whole tiles with aligned rows
-#ifdef A8W8_WIDE_BURST_EPILOGUE
-                const bool fast = false;      // measurement: every tile is written after its last step, in one burst
-#else
                 const bool fast = ep_vec_ok && m0 + BM <= p.m && n0 + BN <= p.n;
-#endif
                 {
                     constexpr int ES = CDT == C_BF16 ? 2 : 4;
                     ep_rs = make_rsrc((const char*)c_addr + ((long long)m0 * p.ldc + n0) * ES, (uint32_t)((BM - 1) * p.ldc + BN) * ES);
@@ -706,7 +709,17 @@ gemm_a8w8_wide(PersistParams pp)
                         c_line_offsets<16>(r16, (int)((uint32_t)(wave_m * 128 + row_of(r16 & 7)) * (uint32_t)ep_row_bytes), (int)((uint32_t)(wave_m * 128 + row_of((r16 & 7) + 8)) * (uint32_t)ep_row_bytes),
                                            (wave_n * 128 + 8 * g) * 4, ep_f32_low, ep_f32_high);
                 }
-                if (fast) {
+                if (fast && BURST) {
+                    // The whole tile in one burst between its last step and the next tile's first: a store among the
+                    // MFMAs makes its wave wait for a place in the memory pipeline, which the loads of the next steps
+                    // share, and the K steps around a tile boundary then take three times as long as the others;
+                    // written back to back the 32 stores of a wave cost less than they stretched those steps by.
+                    // The next tile's first step lets them stay in flight (have_prev).
+                    step(T{}, F{}, F{});
+                    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // last MFMA -> first accumulator read
+                    static_for<WIDE_T / 2>([&](auto JP) { static_for<WIDE_T>([&](auto I) { store_piece(I, JP, false); }); });
+                    have_prev = true;
+                } else if (fast) {
                     step(T{}, F{}, T{});
                     have_prev = true;
                 } else {
@@ -728,7 +741,7 @@ gemm_a8w8_wide(PersistParams pp)
     }
     // the last tile's last quadrant (the compiler does not see the MFMAs: keep the required distance
     // between the last of them and the first read of an accumulator)
-    if (have_prev) {
+    if (have_prev && !BURST) {
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         static_for<8>([&](auto GQ) { flush_piece(std::integral_constant<int, 3>{}, GQ, std::integral_constant<int, 0>{}); });
     }
