@@ -110,7 +110,9 @@ A8W8_DEV void load_to_lds_16(__amdgpu_buffer_rsrc_t rsrc, A8W8_LDS void* lds_bas
 template <bool WRITE_THROUGH>
 A8W8_DEV void store_c_16(__amdgpu_buffer_rsrc_t rsrc, v4i data, int lane_offset, int scalar_offset)
 {
-#ifdef A8W8_STORE_AUX
+#if defined(A8W8_ABLATE_STORE_INSTRUCTIONS)
+    asm volatile("" ::"v"(lane_offset), "s"(scalar_offset), "s"(rsrc));      // measurement: everything but the store itself
+#elif defined(A8W8_STORE_AUX)
     __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, lane_offset, scalar_offset, A8W8_STORE_AUX);      // measurement: cache policy bits
 #else
     __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, lane_offset, scalar_offset, WRITE_THROUGH ? 16 : 0);

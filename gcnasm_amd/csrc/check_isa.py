@@ -10,7 +10,7 @@ The four-wave GEMM kernels:
 Those kernels keep their accumulators in registers a[0:255] that only their own assembly statements
 name.  That is sound as long as the compiler places nothing of its own there and spills nothing:
 this script reads the device assembly of the library and fails the build otherwise.
-Usage: check_isa.py <device .s file>
+Usage: check_isa.py <device .s file> [--no-stores-ok]     (the option: for measurement builds that leave the stores out)
 """
 import re
 import sys
@@ -23,7 +23,7 @@ def instructions(func):
             yield ins
 
 
-def main(path):
+def main(path, no_stores_ok=False):
     text = open(path).read()
     funcs = re.split(r"\n(?=_Z\w+:)", text)
     checked = stores = 0
@@ -67,11 +67,11 @@ def main(path):
             sys.exit(f"{name}: expected MFMAs and accumulator reads, found {mfma} and {reads}")
     if checked == 0:
         sys.exit("no four-wave kernel found in " + path)
-    if stores == 0:
+    if stores == 0 and not no_stores_ok:
         sys.exit("no 16-byte buffer store found in " + path)
     print(f"four-wave kernels: {checked} checked, accumulator registers untouched by the compiler, no scratch")
     print(f"16-byte buffer stores: {stores} checked, each followed by its idle cycles")
 
 
 if __name__ == "__main__":
-    main(sys.argv[1])
+    main(sys.argv[1], "--no-stores-ok" in sys.argv[2:])

@@ -33,11 +33,13 @@
 //   A8W8_ABLATE_SCALE_READS     tiled MX: the scale registers are not refreshed from LDS
 //   A8W8_ABLATE_UNSCALED_MFMA   tiled MX: the plain form of the MFMA in place of the scaled one
 //   A8W8_ABLATE_STORES          whole tiles are neither converted nor written (the accumulators are still read out)
-//   A8W8_ABLATE_STORE_INSTRUCTIONS   whole tiles are read out and converted, only the store instructions are left out (bf16)
+//   A8W8_ABLATE_STORE_INSTRUCTIONS   whole tiles are read out and converted, only the 16-byte store instructions are left out
+//                               (store_c_16 in a8w8_device.hpp: every kernel's whole-tile stores)
 // and three that keep the results right:
 //   A8W8_WIDE_WRITE_THROUGH=0   bf16 tiles are stored write-back instead of written through
 //   A8W8_WIDE_BURST=0           the tile is written out in pieces among the MFMAs of its last K step and of the next
 //                               tile's first quadrant, instead of in one burst between the two steps
+//   A8W8_WIDE_LINE_PAIRS=0      bf16 tiles go out as 64-byte pieces of sixteen rows per store instead of whole lines of eight
 //   A8W8_WIDE_STAGGER=n         workgroups start up to 7 n 64 clocks apart
 #if defined(A8W8_ABLATE_OPERAND_LOADS) || defined(A8W8_ABLATE_SCALE_LOADS) || defined(A8W8_ABLATE_HOT_SCALES) || \
     defined(A8W8_ABLATE_SCALE_READS) || defined(A8W8_ABLATE_UNSCALED_MFMA) || defined(A8W8_ABLATE_STORES) || \
@@ -52,6 +54,9 @@
 #endif
 #ifndef A8W8_WIDE_BURST
 #define A8W8_WIDE_BURST 1
+#endif
+#ifndef A8W8_WIDE_LINE_PAIRS
+#define A8W8_WIDE_LINE_PAIRS 1
 #endif
 
 namespace a8w8 {
@@ -326,15 +331,13 @@ gemm_a8w8_wide(PersistParams pp)
     // whole tiles go out through a buffer descriptor over the tile's own rows (store_c_16)
     __amdgpu_buffer_rsrc_t ep_rs;
     int ep_lane_off = 0, ep_row_bytes = 0;
-    int ep_f32_low = 0, ep_f32_high = 0;            // fp32: the lane's places in the two stores of a piece (store_c_lines)
+    int ep_line_low = 0, ep_line_high = 0;          // the lane's places in the two stores of store_c_lines (fp32: one piece; bf16: two pieces side by side)
     // One piece = the lane's eight consecutive n of MFMA tile row i and tile pair jp: scale, convert,
     // one 16-byte store (bf16) or two (fp32).
-    auto store_piece = [&](auto I, auto JP, bool checked) __attribute__((always_inline)) {
+    auto piece_values = [&](auto I, auto JP, float (&v)[8]) __attribute__((always_inline)) {
         constexpr int i = decltype(I)::value, jp = decltype(JP)::value;
         const int cm = ep_m0 + wave_m * 128 + (PERM_A ? 8 * (r16 >> 2) + (r16 & 3) + 32 * (i >> 1) + 4 * (i & 1) : r16 + 16 * i);
         const int cn = ep_n0 + wave_n * 128 + 8 * g + 32 * jp;
-        char* c_base = (char*)p.c + (long long)ep_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
-        float v[8];
         static_for<8>([&](auto E) {
             constexpr int e = decltype(E)::value;
             v[e] = acc_read<(i * 8 + 2 * jp + (e >> 2)) * 4 + (e & 3)>();
@@ -354,6 +357,31 @@ gemm_a8w8_wide(PersistParams pp)
                 v[4 + e] *= hi[e] * sa;
             }
         }
+    };
+    // bf16, whole tiles: the pieces of tile pairs 2 jpp and 2 jpp + 1 of one MFMA tile row lie 64 bytes apart in every row;
+    // the lanes of rows r and r + 8 exchange them (store_c_lines), and each of the two stores then writes eight whole
+    // 128-byte lines instead of 64-byte halves of sixteen (a compute unit writes whole lines nearly twice as fast)
+    auto store_line_pair = [&](auto I, auto JPP) __attribute__((always_inline)) {
+        constexpr int i = decltype(I)::value, jpp = decltype(JPP)::value;
+        float v0[8], v1[8];
+        piece_values(I, std::integral_constant<int, 2 * jpp>{}, v0);
+        piece_values(I, std::integral_constant<int, 2 * jpp + 1>{}, v1);
+        v4i w0, w1;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            w0[e] = bf16x2_bits(v0[2 * e], v0[2 * e + 1]);
+            w1[e] = bf16x2_bits(v1[2 * e], v1[2 * e + 1]);
+        }
+        constexpr int row = PERM_A ? 32 * (i >> 1) + 4 * (i & 1) : 16 * i;
+        store_c_lines(ep_rs, w0, w1, r16 >= 8, ep_line_low + 128 * jpp, ep_line_high + 128 * jpp, (int)((uint32_t)row * (uint32_t)ep_row_bytes));
+    };
+    auto store_piece = [&](auto I, auto JP, bool checked) __attribute__((always_inline)) {
+        constexpr int i = decltype(I)::value, jp = decltype(JP)::value;
+        const int cm = ep_m0 + wave_m * 128 + (PERM_A ? 8 * (r16 >> 2) + (r16 & 3) + 32 * (i >> 1) + 4 * (i & 1) : r16 + 16 * i);
+        const int cn = ep_n0 + wave_n * 128 + 8 * g + 32 * jp;
+        char* c_base = (char*)p.c + (long long)ep_batch * p.c_batch * (CDT == C_BF16 ? 2 : 4);
+        float v[8];
+        piece_values(I, JP, v);
         if (!checked) {
             // a whole tile: through the tile's buffer descriptor
             constexpr int ES = CDT == C_BF16 ? 2 : 4;
@@ -367,15 +395,11 @@ gemm_a8w8_wide(PersistParams pp)
                 v4i w;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[e] = bf16x2_bits(v[2 * e], v[2 * e + 1]);
-#ifdef A8W8_ABLATE_STORE_INSTRUCTIONS
-                asm volatile("s_nop 1" ::"v"(w), "s"(voff), "s"(soff));      // everything but the store itself
-#else
                 store_c_16<A8W8_WIDE_WRITE_THROUGH != 0>(ep_rs, w, voff, soff);
-#endif
             } else {
                 (void)voff;
                 store_c_lines(ep_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}),
-                              r16 >= 8, ep_f32_low + 32 * jp * 4, ep_f32_high + 32 * jp * 4, soff);
+                              r16 >= 8, ep_line_low + 32 * jp * 4, ep_line_high + 32 * jp * 4, soff);
             }
             return;
         }
@@ -705,9 +729,9 @@ gemm_a8w8_wide(PersistParams pp)
                     auto row_of = [&](int r) __attribute__((always_inline)) { return PERM_A ? 8 * (r >> 2) + (r & 3) : r; };
                     // (unsigned arithmetic: with stride_c in the millions these byte offsets pass 2^31; the hardware takes them as unsigned)
                     ep_lane_off = (int)((uint32_t)(wave_m * 128 + row_of(r16)) * (uint32_t)ep_row_bytes + (uint32_t)((wave_n * 128 + 8 * g) * ES));
-                    if constexpr (CDT == C_FP32)
-                        c_line_offsets<16>(r16, (int)((uint32_t)(wave_m * 128 + row_of(r16 & 7)) * (uint32_t)ep_row_bytes), (int)((uint32_t)(wave_m * 128 + row_of((r16 & 7) + 8)) * (uint32_t)ep_row_bytes),
-                                           (wave_n * 128 + 8 * g) * 4, ep_f32_low, ep_f32_high);
+                    c_line_offsets<CDT == C_FP32 ? 16 : 64>(r16, (int)((uint32_t)(wave_m * 128 + row_of(r16 & 7)) * (uint32_t)ep_row_bytes),
+                                                            (int)((uint32_t)(wave_m * 128 + row_of((r16 & 7) + 8)) * (uint32_t)ep_row_bytes),
+                                                            (wave_n * 128 + 8 * g) * ES, ep_line_low, ep_line_high);
                 }
                 if (fast && BURST) {
                     // The whole tile in one burst between its last step and the next tile's first: a store among the
@@ -717,7 +741,10 @@ gemm_a8w8_wide(PersistParams pp)
                     // The next tile's first step lets them stay in flight (have_prev).
                     step(T{}, F{}, F{});
                     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // last MFMA -> first accumulator read
-                    static_for<WIDE_T / 2>([&](auto JP) { static_for<WIDE_T>([&](auto I) { store_piece(I, JP, false); }); });
+                    if constexpr (CDT == C_BF16 && A8W8_WIDE_LINE_PAIRS)
+                        static_for<WIDE_T / 4>([&](auto JPP) { static_for<WIDE_T>([&](auto I) { store_line_pair(I, JPP); }); });
+                    else
+                        static_for<WIDE_T / 2>([&](auto JP) { static_for<WIDE_T>([&](auto I) { store_piece(I, JP, false); }); });
                     have_prev = true;
                 } else if (fast) {
                     step(T{}, F{}, T{});
