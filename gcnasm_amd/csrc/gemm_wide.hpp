@@ -40,6 +40,7 @@
 //   A8W8_WIDE_BURST=0           the tile is written out in pieces among the MFMAs of its last K step and of the next
 //                               tile's first quadrant, instead of in one burst between the two steps
 //   A8W8_WIDE_LINE_PAIRS=0      bf16 tiles go out as 64-byte pieces of sixteen rows per store instead of whole lines of eight
+//   A8W8_WIDE_READS_EARLY=0     a quadrant's LDS reads follow every second MFMA to its end instead of its first eight
 //   A8W8_WIDE_STAGGER=n         workgroups start up to 7 n 64 clocks apart
 #if defined(A8W8_ABLATE_OPERAND_LOADS) || defined(A8W8_ABLATE_SCALE_LOADS) || defined(A8W8_ABLATE_HOT_SCALES) || \
     defined(A8W8_ABLATE_SCALE_READS) || defined(A8W8_ABLATE_UNSCALED_MFMA) || defined(A8W8_ABLATE_STORES) || \
@@ -57,6 +58,9 @@
 #endif
 #ifndef A8W8_WIDE_LINE_PAIRS
 #define A8W8_WIDE_LINE_PAIRS 1
+#endif
+#ifndef A8W8_WIDE_READS_EARLY
+#define A8W8_WIDE_READS_EARLY 1
 #endif
 
 namespace a8w8 {
@@ -544,8 +548,12 @@ gemm_a8w8_wide(PersistParams pp)
             } else {
                 mfma_acc<lo, z>(fb[j], fa[i]);
             }
-            if constexpr (sl % (2 * MPF) == 2 * MPF - 1) {
-                constexpr int r = sl / (2 * MPF), f = (ref & 1) * 4 + (r >> 1), h = r & 1;     // half h of fragment f
+            // The eight LDS reads of the quadrant go out behind its first eight MFMAs (A8W8_WIDE_READS_EARLY) rather than
+            // one per two MFMAs to its end: the hand-over that follows every second quadrant waits for all of them, and a
+            // read issued behind the last MFMA would leave the matrix cores idle for the whole of its latency.
+            constexpr bool read_here = A8W8_WIDE_READS_EARLY ? (sl < 8 * MPF && sl % MPF == MPF - 1) : (sl % (2 * MPF) == 2 * MPF - 1);
+            if constexpr (read_here) {
+                constexpr int r = A8W8_WIDE_READS_EARLY ? sl / MPF : sl / (2 * MPF), f = (ref & 1) * 4 + (r >> 1), h = r & 1;     // half h of fragment f
                 constexpr int par = f & 1;
                 const int* base = ref < 2 ? rd_a : rd_b;
                 constexpr int off = (f >> 1) * (32 * BK) + par * (ref < 2 ? A_PAR_BYTES : B_PAR_BYTES);
