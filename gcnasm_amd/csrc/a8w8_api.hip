@@ -58,13 +58,14 @@ bool raise_lds_limits_of_mode()
     if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_MXT || MODE == MODE_BF16 || MODE == MODE_F4T)
         ok = ok && raise_lds_limit(gemm_a8w8_wide<MODE, C_BF16>, wide_lds_bytes(MODE)) &&
              raise_lds_limit(gemm_a8w8_wide<MODE, C_FP32>, wide_lds_bytes(MODE));
-    if constexpr (MODE != MODE_F4)
+    {
         ok = ok && raise_lds_limit(gemm_a8w8_tile128<MODE, C_BF16, 2>, small_lds_bytes(MODE, 2)) &&
              raise_lds_limit(gemm_a8w8_tile128<MODE, C_FP32, 2>, small_lds_bytes(MODE, 2)) &&
              raise_lds_limit(gemm_a8w8_tile128<MODE, C_BF16, 4>, small_lds_bytes(MODE, 4)) &&
              raise_lds_limit(gemm_a8w8_tile128<MODE, C_FP32, 4>, small_lds_bytes(MODE, 4)) &&
              raise_lds_limit(gemm_a8w8_tile128<MODE, C_BF16, narrow_stages(MODE), 64>, small_lds_bytes(MODE, narrow_stages(MODE), 64)) &&
              raise_lds_limit(gemm_a8w8_tile128<MODE, C_FP32, narrow_stages(MODE), 64>, small_lds_bytes(MODE, narrow_stages(MODE), 64));
+    }
     return ok;
 }
 
@@ -79,7 +80,7 @@ void set_up_device(int dev)
     const bool ok = raise_lds_limits_of_mode<MODE_TENSOR>() && raise_lds_limits_of_mode<MODE_ROWCOL>() &&
                     raise_lds_limits_of_mode<MODE_BLOCK>() && raise_lds_limits_of_mode<MODE_MX>() &&
                     raise_lds_limits_of_mode<MODE_MXT>() && raise_lds_limits_of_mode<MODE_BF16>() &&
-                    raise_lds_limits_of_mode<MODE_F4T>();
+                    raise_lds_limits_of_mode<MODE_F4T>() && raise_lds_limits_of_mode<MODE_F4>();
     d.status = ok ? A8W8_OK : A8W8_ERR_LAUNCH;
 }
 
@@ -274,7 +275,7 @@ template <int MODE, int CDT>
 int launch_small(const GemmParams& p, int batch, hipStream_t stream)
 {
     if constexpr (MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT ||
-                  MODE == MODE_BF16 || MODE == MODE_F4T) {
+                  MODE == MODE_BF16 || MODE == MODE_F4T || MODE == MODE_F4) {
         GemmParams q = p;
         q.tiles_m = (p.m + SM_BM - 1) / SM_BM;
         q.tiles_n = (p.n + SM_BN - 1) / SM_BN;
@@ -692,6 +693,17 @@ static int a4w4_gemm_impl(const a8w8_gemm_args* g, void* hip_stream, bool allow_
     if (g->b_preshuffled && (!tiled || g->k % 256 != 0 || validate_shuffled_b(&bytes) != A8W8_OK ||
                              (!small_ok(&bytes) && !persist_ok(&bytes))))
         return A8W8_ERR_BAD_GROUP;
+    // row-major scales: the 128-tile kernel at any size (it stages the step's eight scale bytes per row as two dwords:
+    // scale rows have to start on dwords)
+    if (!tiled && !g->b_preshuffled && g->k % 256 == 0) {
+        a8w8_gemm_args rows = bytes;
+        rows.scale_mode = A8W8_SCALE_MX_E8M0_1x32;      // what tiled_ok checks the scale strides and pointers against
+        if (tiled_ok(&rows) && (long long)((g->m + SM_BM - 1) / SM_BM) * ((g->n + 63) / 64) < (1ll << 31)) {
+            const GemmParams p = make_params(&bytes);
+            return g->c_dtype == A8W8_C_BF16 ? launch_small<MODE_F4, C_BF16>(p, g->batch, s)
+                                             : launch_small<MODE_F4, C_FP32>(p, g->batch, s);
+        }
+    }
     if (tiled && g->k % 256 == 0 && tiled_ok(&bytes)) {
         const GemmParams p = make_params(&bytes);
         if (small_ok(&bytes))       // few tiles, or an odd number of 128-byte K steps

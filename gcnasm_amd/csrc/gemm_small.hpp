@@ -22,7 +22,12 @@ constexpr int small_stage_bytes(int bn) { return (SM_BM + bn) * BK; }   // 32768
 // Scale bytes per stage.  Block mode: 128 A-row scales, the B scale at +512 and +768.  Row-major MX: the step's
 // four E8M0 bytes of 128 A rows, then of 128 B rows.  Tiled MX: 1 KiB per wave, whose first half is the 512-byte
 // unit (64 rows x one pair of K steps) of the wave's row block.
-constexpr int small_scale_bytes(int mode) { return mode == MODE_MXT || mode == MODE_F4T ? 4096 : (mode == MODE_BLOCK || mode == MODE_MX) ? 1024 : 0; }
+// Row-major MX scales of packed E2M1 operands (MODE_F4): a 128-byte K step is 256 elements, eight E8M0 bytes per row:
+// the rows' first dwords (128 A rows, then 128 B rows), then their second dwords.
+constexpr int small_scale_bytes(int mode)
+{
+    return mode == MODE_MXT || mode == MODE_F4T ? 4096 : mode == MODE_F4 ? 2048 : (mode == MODE_BLOCK || mode == MODE_MX) ? 1024 : 0;
+}
 constexpr int SM_TM = 4;                               // MFMA tiles per wave along M (along N: a quarter of the tile's columns / 8)
 constexpr int small_lds_bytes(int mode, int stages, int bn = SM_BN)
 {
@@ -50,12 +55,13 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     constexpr int SM_TN = SM_BN / 32;                  // MFMA tiles per wave along N
     constexpr int B_LOADS = SM_BN / 32;                // 1 KiB chunks of B per wave and stage
     static_assert(MODE == MODE_TENSOR || MODE == MODE_ROWCOL || MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_MXT ||
-                      MODE == MODE_BF16 || MODE == MODE_F4T,
+                      MODE == MODE_BF16 || MODE == MODE_F4T || MODE == MODE_F4,
                   "fp32 scales, MX scales, bf16 operands (byte rows of 2k columns, no scales) or packed E2M1 operands (byte "
                   "rows of k/2 columns) with tiled MX scales");
     // tiled scales: of FP8 operands (a K step is 4 blocks of 32: one step of a pair) or of FP4 operands (8 blocks: a pair)
     constexpr bool TILED_SCALES = MODE == MODE_MXT || MODE == MODE_F4T;
-    constexpr bool STEP_SCALES = MODE == MODE_BLOCK || MODE == MODE_MX || TILED_SCALES;      // scales that change with the K step
+    constexpr bool STEP_SCALES = MODE == MODE_BLOCK || MODE == MODE_MX || MODE == MODE_F4 || TILED_SCALES;      // scales that change with the K step
+    constexpr bool IS_F4 = MODE == MODE_F4T || MODE == MODE_F4;      // packed E2M1 operands
     constexpr int SM_SCALE_BYTES = small_scale_bytes(MODE);
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     const int tid = threadIdx.x;
@@ -89,7 +95,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     for (int j = 0; j < B_LOADS; ++j) voff_b[j] = b_lane_offset(p, min(n0 + ld_row + 32 * j, p.n - 1), ld_piece16);
     // block mode: waves 0 and 1 fetch the step's 128 A-row scales (64 each), waves 2 and 3 the B scale
     // of the tile's 128 x 128 block (every lane the same dword: the stage's copy at +512 is the one read)
-    constexpr int LOADS_PER_STAGE = 4 + B_LOADS + (STEP_SCALES ? 1 : 0);
+    constexpr int LOADS_PER_STAGE = 4 + B_LOADS + (MODE == MODE_F4 ? 2 : STEP_SCALES ? 1 : 0);
     __amdgpu_buffer_rsrc_t rsrc_sf = rsrc_a;
     int voff_sf = 0, sf_step_bytes = 0;
     if constexpr (MODE == MODE_BLOCK) {
@@ -105,15 +111,16 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     }
     // MX: waves 0 and 1 fetch the step's dword (four E8M0 bytes, one per 32 of K) of 64 A rows each, waves 2
     // and 3 those of 64 B rows each
-    if constexpr (MODE == MODE_MX) {
+    // (packed E2M1 operands: p.k counts bytes, a row has p.k / 16 scale bytes, eight per K step, fetched as two dwords)
+    if constexpr (MODE == MODE_MX || MODE == MODE_F4) {
         const bool is_b = wave >= 2;
         const int rows = is_b ? p.n : p.m;
         const int stride = is_b ? p.stride_sfb : p.stride_sfa;
         const uint8_t* base = is_b ? (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch
                                    : (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
-        rsrc_sf = make_rsrc(base, (uint32_t)(rows - 1) * stride + (uint32_t)(p.k >> 5));
+        rsrc_sf = make_rsrc(base, (uint32_t)(rows - 1) * stride + (uint32_t)(MODE == MODE_F4 ? p.k >> 4 : p.k >> 5));
         voff_sf = min((is_b ? n0 : m0) + (wave & 1) * 64 + lane, rows - 1) * stride;
-        sf_step_bytes = 4;
+        sf_step_bytes = MODE == MODE_F4 ? 8 : 4;
     }
     // tiled MX: wave w fetches the 512-byte unit of its 64-row block (waves 0, 1: the tile's A blocks, 2, 3: its B
     // blocks) for the step's pair of K steps with one 16-byte load; lanes 32-63 bring the next unit along, unused
@@ -145,6 +152,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
         } else if constexpr (STEP_SCALES) {
             A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 256;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sf, sc, 4, voff_sf, kstep * sf_step_bytes, 0, 0);
+            if constexpr (MODE == MODE_F4) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sf, sc + 1024, 4, voff_sf, kstep * sf_step_bytes + 4, 0, 0);
         }
     };
 
@@ -245,6 +253,18 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
                 for (int t = 0; t < SM_TN; ++t) mx_sb[t] = (int)__builtin_amdgcn_ubfe(sc[128 + wave_n * (SM_BN / 2) + 16 * t + r16], 8 * g, 8);
             }
+            if constexpr (MODE == MODE_F4) {
+                // lane (r16, g) scales 32-block g of each 128-element half of its row: byte g of the row's first and of
+                // its second dword, put side by side as in the tiled layout (the half is chosen by op_sel)
+                const unsigned* sc = (const unsigned*)(smem + SM_STAGES * SM_STAGE_BYTES + cur * SM_SCALE_BYTES);
+                auto two_bytes = [&](int row) __attribute__((always_inline)) {
+                    return (int)(__builtin_amdgcn_ubfe(sc[row], 8 * g, 8) | (__builtin_amdgcn_ubfe(sc[256 + row], 8 * g, 8) << 8));
+                };
+#pragma unroll
+                for (int t = 0; t < SM_TM; ++t) mx_sa[t] = two_bytes(wave_m * 64 + 16 * t + r16);
+#pragma unroll
+                for (int t = 0; t < SM_TN; ++t) mx_sb[t] = two_bytes(128 + wave_n * (SM_BN / 2) + 16 * t + r16);
+            }
             if constexpr (MODE == MODE_F4T) {
                 // both halves' bytes sit side by side: one 16-bit read, the half is chosen by op_sel
                 const char* sc = smem + SM_STAGES * SM_STAGE_BYTES + cur * SM_SCALE_BYTES;
@@ -263,7 +283,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
             for (int j = 0; j < SM_TN; ++j) {
                 if (j + 1 < SM_TN) fb[(j + 1) & 1] = read_frag(cur, rd_b, j + 1);
-                if constexpr (MODE == MODE_F4T) {
+                if constexpr (IS_F4) {
                     // two FP4 MFMAs per fragment pair: elements [0, 128) of the step sit in the fragments' first 16
                     // bytes, [128, 256) in the second; op_sel picks the half's scale byte
 #pragma unroll

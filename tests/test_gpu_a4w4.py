@@ -80,6 +80,43 @@ def test_scale_bytes_reach_the_right_lane_and_half(orc):
     assert (got == exact).all()
 
 
+@pytest.mark.parametrize("shape", [(256, 256, 512), (130, 270, 1024), (300, 520, 768), (200, 1088, 4096), (256, 320, 4352),
+                                   (1024, 2304, 256), (640, 4224, 1280)])
+def test_row_major_scales_on_the_pipelined_kernel(orc, shape):
+    """Row-major E8M0 scales (the quantiser's plain output) with k a multiple of 256 run on the 128-tile MFMA kernel, at
+    any size: same bound against the float64 value as the tiled-scale path, same bits where that path runs the same
+    kernel (up to two 128 x 128 tiles per compute unit)."""
+    m, n, k = shape
+    qa, ea = orc.quantize_mxfp4(_x(m, k, 31 + m))
+    qb, eb = orc.quantize_mxfp4(_x(n, k, 32 + n))
+    ref = orc.gemm_ref_mxfp4(qa, qb, ea, eb)
+    exact, mag = _exact(orc, qa, qb, ea, eb)
+    c32 = g.gemm_a4w4(dev(qa), dev(qb), dev(ea), dev(eb), g.MX, c_dtype=g.FP32)
+    assert (np.abs(c32.cpu().numpy() - exact) <= MFMA_ACC_ERR * mag + 1e-30).all()
+    if ((m + 127) // 128) * ((n + 127) // 128) <= 512:
+        assert torch.equal(c32, g.gemm_a4w4(dev(qa), dev(qb), g.mx_tile_scales(dev(ea)), g.mx_tile_scales(dev(eb)), c_dtype=g.FP32))
+    c = g.gemm_a4w4(dev(qa), dev(qb), dev(ea), dev(eb), g.MX).float().cpu().numpy()
+    miss = ~(np.abs(c - ref) <= 1e-2 * np.abs(ref) + 1e-2)
+    assert miss.mean() <= 1e-3
+    assert (np.abs(c - exact)[miss] <= MFMA_ACC_ERR * mag[miss] + 2.0 ** -8 * np.abs(exact)[miss]).all()
+
+
+@pytest.mark.parametrize("shape", [(256, 512, 1024), (100, 200, 256), (128, 1100, 4096), (384, 640, 2304)])
+def test_row_major_scale_bytes_reach_the_right_lane_and_block(orc, shape):
+    """Distinct powers of two per (row, 32-block) on exactly representable operands, row-major scales: any mix-up of
+    row, block or byte changes the exact result."""
+    m, n, k = shape
+    rng = np.random.Generator(np.random.Philox(19 + m))
+    qa = rng.integers(0, 256, (m, k // 2), dtype=np.uint8)
+    qb = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    ea = (125 + (np.arange(m)[:, None] * 3 + np.arange(k // 32)[None, :]) % 4).astype(np.uint8)
+    eb = (126 + (np.arange(n)[:, None] * 5 + np.arange(k // 32)[None, :] * 2) % 3).astype(np.uint8)
+    exact, _ = _exact(orc, qa, qb, ea, eb)
+    got = g.gemm_a4w4(dev(qa), dev(qb), dev(ea), dev(eb), g.MX, c_dtype=g.FP32).cpu().numpy()
+    bad = np.argwhere(got != exact.astype(np.float32))
+    assert bad.size == 0, f"{m}x{n}x{k}: {len(bad)} elements differ, first {bad[:4].tolist()}"
+
+
 def test_full_size_8192(orc):
     m = n = k = 8192
     gen = torch.Generator(device="cuda"); gen.manual_seed(7)
