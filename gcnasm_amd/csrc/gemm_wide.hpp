@@ -370,6 +370,10 @@ gemm_a8w8_wide(PersistParams pp)
         float v0[8], v1[8];
         piece_values(I, std::integral_constant<int, 2 * jpp>{}, v0);
         piece_values(I, std::integral_constant<int, 2 * jpp + 1>{}, v1);
+#ifdef A8W8_ABLATE_STORES
+        asm volatile("" ::"v"(v0[0]), "v"(v0[7]), "v"(v1[0]), "v"(v1[7]));
+        return;
+#endif
         v4i w0, w1;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
