@@ -125,8 +125,10 @@ A8W8_API int a16w16_flatmm(const a8w8_gemm_args* args, void* hip_stream);
  * 32 elements) through the same f8f6f4 instruction in its FP4 format (the reference names the format,
  * wmma_opus_rdna4/opus/opus.hpp:1854-1855, and has no program for it).  A [batch, m, k/2 bytes],
  * B [batch, n, k/2 bytes]; m, n, k and every stride count ELEMENTS (strides even); scale_mode is
- * MX_E8M0_1x32 (row-major scales, general kernel) or MX_E8M0_TILED (MFMA kernels when k % 256 == 0 and rows
- * are 16-byte aligned). */
+ * MX_E8M0_1x32 (row-major scales, as a4w4_quantize_mx writes them by default) or MX_E8M0_TILED.  The MFMA kernels
+ * take either when k % 256 == 0 and rows are 16-byte aligned (row-major scales: scale pointers and strides
+ * multiples of 4; on the 128 x 128-tile kernel at any size, about half the rate of tiled scales on large problems);
+ * everything else runs on the one-thread-per-element kernel. */
 A8W8_API int a4w4_gemm(const a8w8_gemm_args* args, void* hip_stream);
 /* MXFP4 skinny-M GEMM over pre-shuffled weights (no counterpart in the reference, which has neither an FP4
  * program nor a flat one for it; it is a8w8_flatmm for the FP4 form of the same instruction).  A [batch, m, k/2
