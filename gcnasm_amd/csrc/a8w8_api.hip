@@ -311,6 +311,7 @@ int launch_persist(const GemmParams& p, int batch, hipStream_t stream)
     pp.g = p;
     pp.batch = batch;
     pp.items = batch * p.tiles_m * p.tiles_n;
+    pp.map = make_tile_map(p.tiles_m, p.tiles_n);
     const int cus = num_cus();
     dim3 grid((unsigned)(pp.items < cus ? pp.items : cus), 1, 1);
     return launch(gemm_a8w8_persist<MODE, CDT>, grid, dim3(GEMM_THREADS), persist_lds_bytes(MODE), stream, pp);
@@ -327,6 +328,7 @@ int launch_wide(const GemmParams& p, int batch, hipStream_t stream)
         pp.g = p;
         pp.batch = batch;
         pp.items = batch * p.tiles_m * p.tiles_n;
+        pp.map = make_tile_map(p.tiles_m, p.tiles_n);
         const int cus = num_cus();
         dim3 grid((unsigned)(pp.items < cus ? pp.items : cus), 1, 1);
         return launch(gemm_a8w8_wide<MODE, CDT>, grid, dim3(WIDE_THREADS), wide_lds_bytes(MODE), stream, pp);

@@ -84,6 +84,7 @@ struct PersistParams {
     GemmParams g;
     int batch;        // work items = batch * tiles_m * tiles_n, walked with stride gridDim.x
     int items;
+    TileMap map;      // item -> (batch entry, tile) without run-time divisors
 };
 
 template <int MODE, int CDT>
@@ -102,7 +103,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     constexpr int GROUP_MASK = (1 << GROUP_SHIFT) - 1;
     const int r16 = lane & 15, g = lane >> 4;
     const int nk = p.k / BK;                       // >= 2 (checked by the host)
-    const int tiles = p.tiles_m * p.tiles_n;
 
     // ---------------------------------------------------------------- load side state
     // position of the stage whose loads are being issued: (item, k step), two steps ahead
@@ -121,9 +121,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     const int ld_piece16 = ((lane & 7) ^ (((lane >> 3) ^ ((wave & 3) << 1)) & 7)) * 16;
     auto point_loads_at = [&](int item) __attribute__((always_inline)) {
         item = min(item, pp.items - 1);            // past the end: keep loading valid data nobody reads
-        const int batch = item / tiles;
-        int tm, tn;
-        tile_of_block(item - batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+        int batch, tm, tn;
+        tile_of_item(pp.map, item, batch, tm, tn);
         const int m0 = tm * BM, n0 = tn * BN;
         rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
         rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, b_extent_bytes(p));
@@ -225,9 +224,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
     int cur_item = blockIdx.x, cur_ks = 0;         // the step being multiplied
     int cur_batch = 0, m0 = 0, n0 = 0;
     auto point_compute_at = [&](int item) __attribute__((always_inline)) {
-        cur_batch = item / tiles;
         int tm, tn;
-        tile_of_block(item - cur_batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+        tile_of_item(pp.map, item, cur_batch, tm, tn);
         m0 = tm * BM;
         n0 = tn * BN;
     };
@@ -488,9 +486,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         const int nx_ks = last_of_tile ? 0 : cur_ks + 1;
         if (last_of_tile) {
             const int item = min(cur_item + (int)gridDim.x, pp.items - 1);
-            nx_batch = item / tiles;
             int tm, tn;
-            tile_of_block(item - nx_batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+            tile_of_item(pp.map, item, nx_batch, tm, tn);
             nx_m0 = tm * BM;
             nx_n0 = tn * BN;
             nx_gbase = cur_gbase + groups_per_tile;

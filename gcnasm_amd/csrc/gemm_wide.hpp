@@ -159,7 +159,6 @@ gemm_a8w8_wide(PersistParams pp)
     const int wave_m = wave >> 1, wave_n = wave & 1;
     const int r16 = lane & 15, g = lane >> 4;
     const int nk = p.k / BK;                       // >= 2 (checked by the host)
-    const int tiles = p.tiles_m * p.tiles_n;
 
     // LDS: [A of stage 0][A of stage 1][B of stage 0][B of stage 1], 32 KiB each.  A lane's read
     // addresses are its row and K-piece offset inside an operand (below 32 KiB) plus the stage and the
@@ -183,9 +182,8 @@ gemm_a8w8_wide(PersistParams pp)
     int ld_voff_a[2] = {0, 0}, ld_voff_b[2] = {0, 0};   // rows 8w.. and 128 + 8w.. of the tile
     auto point_loads_at = [&](int item) __attribute__((always_inline)) {
         item = min(item, pp.items - 1);            // past the end: keep loading valid data nobody reads
-        const int batch = item / tiles;
-        int tm, tn;
-        tile_of_block(item - batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+        int batch, tm, tn;
+        tile_of_item(pp.map, item, batch, tm, tn);
         rsrc_a = make_rsrc(p.a + (long long)batch * p.a_batch, (uint32_t)(p.m - 1) * p.lda + p.k);
         rsrc_b = make_rsrc(p.b + (long long)batch * p.b_batch, b_extent_bytes(p));
 #pragma unroll
@@ -230,9 +228,8 @@ gemm_a8w8_wide(PersistParams pp)
     auto point_scales_at = [&](ScaleTile& t, int item) __attribute__((always_inline)) {
         if constexpr (IS_MXT) {
             item = min(item, pp.items - 1);
-            const int batch = item / tiles;
-            int tm, tn;
-            tile_of_block(item - batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+            int batch, tm, tn;
+            tile_of_item(pp.map, item, batch, tm, tn);
             t.base[0] = (const uint8_t*)p.sfa + (long long)batch * p.sfa_batch;
             t.base[1] = (const uint8_t*)p.sfb + (long long)batch * p.sfb_batch;
             t.blk[0] = tm * (BM / 64);
@@ -318,9 +315,8 @@ gemm_a8w8_wide(PersistParams pp)
     int cur_batch = 0, m0 = 0, n0 = 0;
     auto point_compute_at = [&](int item) __attribute__((always_inline)) {
         item = min(item, pp.items - 1);
-        cur_batch = item / tiles;
         int tm, tn;
-        tile_of_block(item - cur_batch * tiles, p.tiles_m, p.tiles_n, tm, tn);
+        tile_of_item(pp.map, item, cur_batch, tm, tn);
         m0 = tm * BM;
         n0 = tn * BN;
     };
