@@ -127,29 +127,69 @@ A8W8_DEV int from_lane_8_apart(int v)
 }
 
 // The two 16-byte halves `lo`, `hi` of the eight consecutive fp32 columns a lane holds of one row of a whole C tile
-// (`hi` DISTANCE = 16 bytes after `lo`).  Stored as they are, each store of a wave would cover every other 16 bytes of
-// 16 rows.  Instead the lanes of rows r and r + 8 (of the 16 a wave's store covers) exchange halves, so that one store
-// writes rows 0 .. 7 and the other rows 8 .. 15, each row as one contiguous 128-byte line (lane r < 8: its own `lo`;
-// lane r + 8: the `hi` of lane r, DISTANCE bytes on): whole lines, which can take the write-through path.  (The same
-// for two bf16 pieces side by side, DISTANCE 64, measured no faster than their 64-byte pieces.)
-// lane_offset_low / _high: the lane's place in the first / second store (c_line_offsets, per tile); upper: the
-// lane's row index within the 16 is 8 or more.
-A8W8_DEV void store_c_lines(__amdgpu_buffer_rsrc_t rsrc, v4i lo, v4i hi, bool upper, int lane_offset_low, int lane_offset_high,
-                            int scalar_offset)
+// (`hi` DISTANCE = 16 bytes after `lo`), or two bf16 pieces of the row side by side (DISTANCE 64).  Stored as they are,
+// each store of a wave would cover every other 16 bytes (bf16: 64-byte halves) of 16 rows.  Instead
+//  1. the lanes of rows r and r + 8 (of the 16 a wave's store covers) exchange halves (DPP row_ror:8), so that one store
+//     holds rows 0 .. 7 and the other rows 8 .. 15, each row as one contiguous 128-byte line: whole lines, which can take
+//     the write-through path;
+//  2. (BY_LANE) the 16-byte units of each store are moved between the lanes (ds_bpermute, four per store) so that
+//     CONSECUTIVE LANES hold consecutive 16 bytes of a line: lane L writes piece L % 8 of row L / 8.  The memory pipeline
+//     takes a store's lanes in order, and a store whose neighbouring lanes lie in different rows occupies it 2.7 times as
+//     long as one whose lanes run along the lines (26.8 against 10.5 ns per 1 KiB store and compute unit, measured with
+//     nothing else running).  The eight-wave kernel gains 1.5-2% from it; the four-wave kernel, whose workgroups all
+//     reach their stores within the same few microseconds and are then bound by what the whole chip can store at once
+//     (about 30 ns per store and compute unit either way), does not, and leaves step 2 out.
+// upper: the lane's row index within the 16 is 8 or more; source_low / _high: c_line_source of the lane for the two stores;
+// lane_offset_low / _high: the lane's place in the first / second store (c_line_offsets, per tile).
+template <bool BY_LANE>
+A8W8_DEV void store_c_lines(__amdgpu_buffer_rsrc_t rsrc, v4i lo, v4i hi, bool upper, int source_low, int source_high,
+                            int lane_offset_low, int lane_offset_high, int scalar_offset)
 {
     const v4i r = {from_lane_8_apart(hi.x), from_lane_8_apart(hi.y), from_lane_8_apart(hi.z), from_lane_8_apart(hi.w)};
-    const v4i first = upper ? r : lo, second = upper ? lo : r;
+    v4i first = upper ? r : lo, second = upper ? lo : r;
+    if constexpr (BY_LANE) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            first[e] = __builtin_amdgcn_ds_bpermute(source_low, first[e]);
+            second[e] = __builtin_amdgcn_ds_bpermute(source_high, second[e]);
+        }
+    }
     store_c_16<true>(rsrc, first, lane_offset_low, scalar_offset);
     store_c_16<true>(rsrc, second, lane_offset_high, scalar_offset);
 }
-// The two lane offsets of store_c_lines: row_low / row_high = byte offsets of the rows that lanes (r16 & 7) and
-// (r16 & 7) + 8 own, col = the lane's byte offset inside a row (a multiple of 2 * DISTANCE).
-template <int DISTANCE>
-A8W8_DEV void c_line_offsets(int r16, int row_low, int row_high, int col, int& lane_offset_low, int& lane_offset_high)
+// After step 1 lane 16 g + r16 holds, of row r16 % 8 of each store, a 16-byte piece of the row's line: in the first
+// store piece 4 u + g (bf16 pairs, DISTANCE 64: the line is two 64-byte halves of four pieces) or 2 g + u (fp32, DISTANCE
+// 16) with u = r16 / 8, in the second store the same with 1 - u.  The byte address (lane x 4) of the lane that holds what
+// lane `lane` is to write, piece lane % 8 of row lane / 8, in the first (second = false) or second store.
+template <int DISTANCE, bool BY_LANE>
+A8W8_DEV int c_line_source(int lane, bool second)
 {
-    const bool upper = r16 >= 8;
-    lane_offset_low = (int)((uint32_t)row_low + (uint32_t)(col + (upper ? DISTANCE : 0)));
-    lane_offset_high = (int)((uint32_t)row_high + (uint32_t)(col + (upper ? 0 : DISTANCE)));
+    if constexpr (!BY_LANE) return 4 * lane;
+    const int row = lane >> 3, piece = lane & 7;
+    const int g = DISTANCE == 64 ? (piece & 3) : (piece >> 1), u = DISTANCE == 64 ? (piece >> 2) : (piece & 1);
+    return 4 * (16 * g + 8 * (second ? 1 - u : u) + row);
+}
+// the row (0 .. 7) of the 16 that `lane` writes in the first store (the second: 8 more)
+template <bool BY_LANE>
+A8W8_DEV int c_line_row(int lane)
+{
+    return BY_LANE ? lane >> 3 : lane & 7;
+}
+// The two lane offsets of store_c_lines: row_low / row_high = byte offsets of rows c_line_row(lane) and c_line_row(lane) + 8
+// of the 16, col = byte offset of the line inside a row.  By lane: piece lane % 8 of the line.  Otherwise (r16, g = lane % 16,
+// lane / 16): the lane's own piece g, the halves DISTANCE apart.
+template <int DISTANCE, bool BY_LANE>
+A8W8_DEV void c_line_offsets(int lane, int row_low, int row_high, int col, int& lane_offset_low, int& lane_offset_high)
+{
+    if constexpr (BY_LANE) {
+        lane_offset_low = (int)((uint32_t)row_low + (uint32_t)(col + 16 * (lane & 7)));
+        lane_offset_high = (int)((uint32_t)row_high + (uint32_t)(col + 16 * (lane & 7)));
+    } else {
+        const bool upper = (lane & 15) >= 8;
+        const int piece = (lane >> 4) * (DISTANCE == 64 ? 16 : 32);
+        lane_offset_low = (int)((uint32_t)row_low + (uint32_t)(col + piece + (upper ? DISTANCE : 0)));
+        lane_offset_high = (int)((uint32_t)row_high + (uint32_t)(col + piece + (upper ? 0 : DISTANCE)));
+    }
 }
 
 // Barrier without the wait for every outstanding load that __syncthreads() implies: the pipelined kernels

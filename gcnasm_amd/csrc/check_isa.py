@@ -1,9 +1,9 @@
 #!/usr/bin/env python3
 """Build-time checks of the compiler's output.
 
-Every kernel: a 16-byte (or 12-byte) buffer store (the C tiles' stores) is followed, before anything that writes a vector
-register, by the two idle cycles that keep the next write to its data registers at a distance (store_c_16 in
-a8w8_device.hpp).
+Every kernel: a 16-byte (or 12-byte) buffer store (the C tiles' stores) reads its data registers for a few cycles after it
+issues, so nothing may write them in the two issue slots behind it: the first write to one of them has to come after the
+two idle cycles that store_c_16 (a8w8_device.hpp) puts behind the store, or after at least two other instructions.
 
 The four-wave GEMM kernels:
 
@@ -23,6 +23,17 @@ def instructions(func):
             yield ins
 
 
+def registers(operand):
+    """The vector registers an operand names: 'v7' or 'v[4:7]' (anything else: none)."""
+    m = re.fullmatch(r"v(\d+)", operand.strip())
+    if m:
+        return {int(m.group(1))}
+    m = re.fullmatch(r"v\[(\d+):(\d+)\]", operand.strip())
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    return set()
+
+
 def main(path, no_stores_ok=False):
     text = open(path).read()
     funcs = re.split(r"\n(?=_Z\w+:)", text)
@@ -35,13 +46,22 @@ def main(path, no_stores_ok=False):
             # part is held to the same rule)
             if ins.startswith("buffer_store_dwordx4") or ins.startswith("buffer_store_dwordx3"):
                 stores += 1
-                # nothing that could write a vector register may come between the store and its idle cycles
-                j = i + 1
-                while j < len(seq) and seq[j] != "s_nop 1" and (seq[j].startswith("s_") or seq[j].startswith("v_readlane_b32") or
-                                                                 seq[j].startswith("v_readfirstlane_b32")):
-                    j += 1
-                if j >= len(seq) or seq[j] != "s_nop 1":
-                    sys.exit(f"{name}: 16-byte buffer store without the idle cycles behind it: {ins} / {seq[j] if j < len(seq) else ''}")
+                data = registers(ins.split(None, 1)[1].split(",")[0])
+                # walk on until the idle cycles (or two other instructions) have passed; nothing before that may write the data
+                slots = 0
+                for nxt in seq[i + 1:i + 4]:
+                    if nxt == "s_nop 1" or slots >= 2:
+                        break
+                    if nxt.startswith("s_nop"):
+                        slots += 1 + int(nxt.split()[1])
+                        continue
+                    if nxt.endswith(":") or nxt.startswith("s_cbranch") or nxt.startswith("s_branch") or nxt.startswith("s_endpgm"):
+                        sys.exit(f"{name}: control flow directly behind a 16-byte buffer store: {ins} / {nxt}")
+                    parts = nxt.split(None, 1)
+                    written = registers(parts[1].split(",")[0]) if len(parts) > 1 and not parts[0].startswith(("buffer_store", "global_store", "ds_write", "s_")) else set()
+                    if written & data:
+                        sys.exit(f"{name}: the data registers of a 16-byte buffer store are written directly behind it: {ins} / {nxt}")
+                    slots += 1
         if "gemm_a8w8_wide" not in name:
             continue
         checked += 1
@@ -70,7 +90,7 @@ def main(path, no_stores_ok=False):
     if stores == 0 and not no_stores_ok:
         sys.exit("no 16-byte buffer store found in " + path)
     print(f"four-wave kernels: {checked} checked, accumulator registers untouched by the compiler, no scratch")
-    print(f"16-byte buffer stores: {stores} checked, each followed by its idle cycles")
+    print(f"16-byte buffer stores: {stores} checked, none with a write to its data registers in the two slots behind it")
 
 
 if __name__ == "__main__":

@@ -71,6 +71,9 @@ constexpr int PERSIST_LDS_BYTES_ROWCOL = GEMM_LDS_BYTES + 2 * ROWCOL_SCALE_BYTES
 #ifndef A8W8_PERSIST_LINE_PAIRS
 #define A8W8_PERSIST_LINE_PAIRS 1
 #endif
+#ifndef A8W8_PERSIST_LINES_BY_LANE
+#define A8W8_PERSIST_LINES_BY_LANE 1      // 0: whole-line stores without the re-ordering of the lanes (measurement)
+#endif
 #ifndef A8W8_PERSIST_SB
 #define A8W8_PERSIST_SB 0
 #endif
@@ -339,9 +342,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         const bool upper = r16 >= 8;
         int line_off_low, line_off_high;
         // (fp32: the two halves of a piece, 16 bytes apart; bf16: two pieces side by side, 64 bytes apart)
-        c_line_offsets<CDT == C_FP32 ? 16 : 64>(r16, (int)((uint32_t)(wave_m * WAVE_M + (r16 & 7)) * ldc_bytes),
-                                                (int)((uint32_t)(wave_m * WAVE_M + (r16 & 7) + 8) * ldc_bytes), (wave_n * WAVE_N + 8 * g) * C_ES,
-                                                line_off_low, line_off_high);
+        constexpr bool BL = A8W8_PERSIST_LINES_BY_LANE != 0;
+        c_line_offsets<CDT == C_FP32 ? 16 : 64, BL>(lane, (int)((uint32_t)(wave_m * WAVE_M + c_line_row<BL>(lane)) * ldc_bytes),
+                                                    (int)((uint32_t)(wave_m * WAVE_M + c_line_row<BL>(lane) + 8) * ldc_bytes), wave_n * WAVE_N * C_ES,
+                                                    line_off_low, line_off_high);
+        const int line_src_low = c_line_source<CDT == C_FP32 ? 16 : 64, BL>(lane, false), line_src_high = c_line_source<CDT == C_FP32 ? 16 : 64, BL>(lane, true);
         auto scaled_piece = [&](int i, int jp, float (&v)[8]) __attribute__((always_inline)) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -367,7 +372,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                     float v0[8], v1[8];
                     scaled_piece(i, 2 * jpp, v0);
                     scaled_piece(i, 2 * jpp + 1, v1);
-                    store_c_lines(tile_rs, packed_bf16(v0), packed_bf16(v1), upper, line_off_low + 128 * jpp, line_off_high + 128 * jpp, i * tile_row16);
+                    store_c_lines<BL>(tile_rs, packed_bf16(v0), packed_bf16(v1), upper, line_src_low, line_src_high, line_off_low + 128 * jpp, line_off_high + 128 * jpp, i * tile_row16);
                 }
             return;
         }
@@ -382,8 +387,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
                     if constexpr (CDT == C_BF16) {
                         store_c_16<true>(tile_rs, packed_bf16(v), tile_lane_off + 32 * jp * C_ES, i * tile_row16);
                     } else {
-                        store_c_lines(tile_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}),
-                                      __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), upper, line_off_low + 32 * jp * C_ES,
+                        store_c_lines<BL>(tile_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}),
+                                      __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}), upper, line_src_low, line_src_high, line_off_low + 32 * jp * C_ES,
                                       line_off_high + 32 * jp * C_ES, i * tile_row16);
                     }
                 }

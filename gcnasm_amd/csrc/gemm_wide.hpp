@@ -40,6 +40,8 @@
 //   A8W8_WIDE_BURST=0           the tile is written out in pieces among the MFMAs of its last K step and of the next
 //                               tile's first quadrant, instead of in one burst between the two steps
 //   A8W8_WIDE_LINE_PAIRS=0      bf16 tiles go out as 64-byte pieces of sixteen rows per store instead of whole lines of eight
+//   A8W8_WIDE_LINES_BY_LANE=1   the whole-line stores' 16-byte units are moved between the lanes so that consecutive lanes write
+//                               consecutive bytes (store_c_lines in a8w8_device.hpp; what the eight-wave kernel does)
 //   A8W8_WIDE_READS_EARLY=0     a quadrant's LDS reads follow every second MFMA to its end instead of its first eight
 //   A8W8_WIDE_STAGGER=n         workgroups start up to 7 n 64 clocks apart
 #if defined(A8W8_ABLATE_OPERAND_LOADS) || defined(A8W8_ABLATE_SCALE_LOADS) || defined(A8W8_ABLATE_HOT_SCALES) || \
@@ -58,6 +60,9 @@
 #endif
 #ifndef A8W8_WIDE_LINE_PAIRS
 #define A8W8_WIDE_LINE_PAIRS 1
+#endif
+#ifndef A8W8_WIDE_LINES_BY_LANE
+#define A8W8_WIDE_LINES_BY_LANE 0
 #endif
 #ifndef A8W8_WIDE_READS_EARLY
 #define A8W8_WIDE_READS_EARLY 1
@@ -331,6 +336,9 @@ gemm_a8w8_wide(PersistParams pp)
     // whole tiles go out through a buffer descriptor over the tile's own rows (store_c_16)
     __amdgpu_buffer_rsrc_t ep_rs;
     int ep_lane_off = 0, ep_row_bytes = 0;
+    // whose 16 bytes the lane writes in the two stores of store_c_lines (itself unless the lanes are re-ordered)
+    const int ep_line_src_low = c_line_source<CDT == C_FP32 ? 16 : 64, A8W8_WIDE_LINES_BY_LANE != 0>(lane, false);
+    const int ep_line_src_high = c_line_source<CDT == C_FP32 ? 16 : 64, A8W8_WIDE_LINES_BY_LANE != 0>(lane, true);
     int ep_line_low = 0, ep_line_high = 0;          // the lane's places in the two stores of store_c_lines (fp32: one piece; bf16: two pieces side by side)
     // One piece = the lane's eight consecutive n of MFMA tile row i and tile pair jp: scale, convert,
     // one 16-byte store (bf16) or two (fp32).
@@ -377,7 +385,7 @@ gemm_a8w8_wide(PersistParams pp)
             w1[e] = bf16x2_bits(v1[2 * e], v1[2 * e + 1]);
         }
         constexpr int row = PERM_A ? 32 * (i >> 1) + 4 * (i & 1) : 16 * i;
-        store_c_lines(ep_rs, w0, w1, r16 >= 8, ep_line_low + 128 * jpp, ep_line_high + 128 * jpp, (int)((uint32_t)row * (uint32_t)ep_row_bytes));
+        store_c_lines<A8W8_WIDE_LINES_BY_LANE != 0>(ep_rs, w0, w1, r16 >= 8, ep_line_src_low, ep_line_src_high, ep_line_low + 128 * jpp, ep_line_high + 128 * jpp, (int)((uint32_t)row * (uint32_t)ep_row_bytes));
     };
     auto store_piece = [&](auto I, auto JP, bool checked) __attribute__((always_inline)) {
         constexpr int i = decltype(I)::value, jp = decltype(JP)::value;
@@ -402,8 +410,8 @@ gemm_a8w8_wide(PersistParams pp)
                 store_c_16<A8W8_WIDE_WRITE_THROUGH != 0>(ep_rs, w, voff, soff);
             } else {
                 (void)voff;
-                store_c_lines(ep_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}),
-                              r16 >= 8, ep_line_low + 32 * jp * 4, ep_line_high + 32 * jp * 4, soff);
+                store_c_lines<A8W8_WIDE_LINES_BY_LANE != 0>(ep_rs, __builtin_bit_cast(v4i, v4f{v[0], v[1], v[2], v[3]}), __builtin_bit_cast(v4i, v4f{v[4], v[5], v[6], v[7]}),
+                              r16 >= 8, ep_line_src_low, ep_line_src_high, ep_line_low + 32 * jp * 4, ep_line_high + 32 * jp * 4, soff);
             }
             return;
         }
@@ -737,9 +745,10 @@ gemm_a8w8_wide(PersistParams pp)
                     auto row_of = [&](int r) __attribute__((always_inline)) { return PERM_A ? 8 * (r >> 2) + (r & 3) : r; };
                     // (unsigned arithmetic: with stride_c in the millions these byte offsets pass 2^31; the hardware takes them as unsigned)
                     ep_lane_off = (int)((uint32_t)(wave_m * 128 + row_of(r16)) * (uint32_t)ep_row_bytes + (uint32_t)((wave_n * 128 + 8 * g) * ES));
-                    c_line_offsets<CDT == C_FP32 ? 16 : 64>(r16, (int)((uint32_t)(wave_m * 128 + row_of(r16 & 7)) * (uint32_t)ep_row_bytes),
-                                                            (int)((uint32_t)(wave_m * 128 + row_of((r16 & 7) + 8)) * (uint32_t)ep_row_bytes),
-                                                            (wave_n * 128 + 8 * g) * ES, ep_line_low, ep_line_high);
+                    constexpr bool BL = A8W8_WIDE_LINES_BY_LANE != 0;
+                    c_line_offsets<CDT == C_FP32 ? 16 : 64, BL>(lane, (int)((uint32_t)(wave_m * 128 + row_of(c_line_row<BL>(lane))) * (uint32_t)ep_row_bytes),
+                                                                (int)((uint32_t)(wave_m * 128 + row_of(c_line_row<BL>(lane) + 8)) * (uint32_t)ep_row_bytes),
+                                                                wave_n * 128 * ES, ep_line_low, ep_line_high);
                 }
                 if (fast && BURST) {
                     // The whole tile in one burst between its last step and the next tile's first: a store among the
