@@ -28,6 +28,9 @@ constexpr int small_scale_bytes(int mode)
 {
     return mode == MODE_MXT || mode == MODE_F4T ? 4096 : mode == MODE_F4 ? 2048 : (mode == MODE_BLOCK || mode == MODE_MX) ? 1024 : 0;
 }
+#ifndef A8W8_SMALL_LINES_BY_LANE
+#define A8W8_SMALL_LINES_BY_LANE 1      // 0: whole tiles are stored from the MFMA layout as they are (measurement)
+#endif
 constexpr int SM_TM = 4;                               // MFMA tiles per wave along M (along N: a quarter of the tile's columns / 8)
 constexpr int small_lds_bytes(int mode, int stages, int bn = SM_BN)
 {
@@ -348,6 +351,53 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     const bool vec_ok = (CDT == C_BF16) ? ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 7) == 0)
                                         : ((p.ldc & 3) == 0 && (((uintptr_t)c_base) & 15) == 0);
     const bool whole = vec_ok && m0 + SM_BM <= p.m && n0 + SM_BN <= p.n;
+#if A8W8_SMALL_LINES_BY_LANE
+    // A tile inside the matrix leaves through LDS, 16 rows of the wave's 64 at a time: the MFMA layout's stores have
+    // neighbouring lanes in different rows (16 rows x 16 bytes per 16 lanes), which occupies the memory pipeline 2.7 times as long as
+    // stores whose consecutive lanes write consecutive 16 bytes of a row.  A problem of few tiles ends with every workgroup's stores
+    // and nothing to hide them behind.  The wave writes the 16 x (16 SM_TN) values into its own 4.25 KiB of LDS (rows padded
+    // by 16 bytes against bank conflicts), reads them back along the rows and stores 16 bytes per lane; a wave's LDS
+    // operations complete in order, so neither step needs a barrier.  Every direct-to-LDS load has landed by then (the
+    // loop's last loads re-fill stages nobody reads).
+    if (whole && (CDT == C_FP32 ? (p.ldc & 3) == 0 : (p.ldc & 7) == 0) && (((uintptr_t)c_base) & 15) == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        constexpr int ES = CDT == C_BF16 ? 2 : 4;
+        constexpr int ROW_BYTES = SM_TN * 16 * ES;                 // the wave's columns of one row
+        constexpr int ROW_PITCH = ROW_BYTES + 16;
+        constexpr int LANES_PER_ROW = ROW_BYTES / 16, ROWS_PER_STORE = 64 / LANES_PER_ROW, STORES = 16 / ROWS_PER_STORE;
+        char* mine = smem + wave * (16 * (SM_BN / 2 * 4 + 16));
+        const int wr = r16 * ROW_PITCH + 4 * g * ES;              // + 16 j ES: the lane's four values of MFMA tile j
+        const int rd = (lane / LANES_PER_ROW) * ROW_PITCH + (lane % LANES_PER_ROW) * 16;      // + ROWS_PER_STORE rows per store
+        char* c_wave = c_base + ((long long)(m0 + wave_m * 64) * p.ldc + n0 + wave_n * (SM_BN / 2)) * ES;
+        const long long row_bytes = (long long)p.ldc * ES;
+        float sb_all[SM_TN][4];
+        if constexpr (MODE == MODE_ROWCOL) {
+#pragma unroll
+            for (int j = 0; j < SM_TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sb_all[j][e] = sfb_f[cn_base + 16 * j + e];
+        }
+#pragma unroll
+        for (int i = 0; i < SM_TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < SM_TN; ++j) {
+                v4f v = acc[i][j];
+                if constexpr (MODE == MODE_TENSOR) v *= ts;
+                if constexpr (MODE == MODE_ROWCOL) v *= v4f{sb_all[j][0], sb_all[j][1], sb_all[j][2], sb_all[j][3]} * sa[i];
+                if constexpr (CDT == C_BF16) *(v2i*)(mine + wr + 16 * j * ES) = v2i{bf16x2_bits(v.x, v.y), bf16x2_bits(v.z, v.w)};
+                else *(v4f*)(mine + wr + 16 * j * ES) = v;
+            }
+#pragma unroll
+            for (int st = 0; st < STORES; ++st) {
+                const v4i w = *(const v4i*)(mine + rd + st * ROWS_PER_STORE * ROW_PITCH);
+                const int row = 16 * i + st * ROWS_PER_STORE + lane / LANES_PER_ROW;
+                A8W8_STORE_C((v4i*)(c_wave + row * row_bytes + (lane % LANES_PER_ROW) * 16), w);
+            }
+        }
+        return;
+    }
+#endif
 #pragma unroll
     for (int j = 0; j < SM_TN; ++j) {
         const int cn = cn_base + 16 * j;
