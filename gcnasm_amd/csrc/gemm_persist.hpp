@@ -343,10 +343,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) gemm_a8w8_persist(PersistPara
         int line_off_low, line_off_high;
         // (fp32: the two halves of a piece, 16 bytes apart; bf16: two pieces side by side, 64 bytes apart)
         constexpr bool BL = A8W8_PERSIST_LINES_BY_LANE != 0;
-        c_line_offsets<CDT == C_FP32 ? 16 : 64, BL>(lane, (int)((uint32_t)(wave_m * WAVE_M + c_line_row<BL>(lane)) * ldc_bytes),
-                                                    (int)((uint32_t)(wave_m * WAVE_M + c_line_row<BL>(lane) + 8) * ldc_bytes), wave_n * WAVE_N * C_ES,
+        // (worked out from an opaque copy of the lane number: values that depend on the lane alone would otherwise be computed
+        // once, before the K loop, and held in registers the block-scale loop does not have: two of them spilled)
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        c_line_offsets<CDT == C_FP32 ? 16 : 64, BL>(ln, (int)((uint32_t)(wave_m * WAVE_M + c_line_row<BL>(ln)) * ldc_bytes),
+                                                    (int)((uint32_t)(wave_m * WAVE_M + c_line_row<BL>(ln) + 8) * ldc_bytes), wave_n * WAVE_N * C_ES,
                                                     line_off_low, line_off_high);
-        const int line_src_low = c_line_source<CDT == C_FP32 ? 16 : 64, BL>(lane, false), line_src_high = c_line_source<CDT == C_FP32 ? 16 : 64, BL>(lane, true);
+        const int line_src_low = c_line_source<CDT == C_FP32 ? 16 : 64, BL>(ln, false), line_src_high = c_line_source<CDT == C_FP32 ? 16 : 64, BL>(ln, true);
         auto scaled_piece = [&](int i, int jp, float (&v)[8]) __attribute__((always_inline)) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {

@@ -215,7 +215,7 @@ def test_pipelined_kernels_use_no_scratch():
     # compiler put nothing of its own there (gcnasm_amd/csrc/check_isa.py) and records the verdict
     assert "accumulator registers untouched by the compiler" in text
     # ... and that every 16-byte buffer store of a C tile is followed by the idle cycles its data registers need
-    assert re.search(r"16-byte buffer stores: \d+ checked, each followed by its idle cycles", text)
+    assert re.search(r"16-byte buffer stores: \d+ checked, none with a write to its data registers in the two slots behind it", text)
     # MXFP8 flat GEMM: four weight tiles x four row groups exists (and is among the kernels checked above)
     assert "flatmm_a8w8ILi4ELi4ELi0ELi4ELb0EE" in text
 
