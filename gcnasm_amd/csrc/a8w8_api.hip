@@ -242,13 +242,17 @@ int num_cus()
 // 256-tile kernels (block / row-col / tiled MX): 2.2x / 1.7x / 1.6x at 64 workgroups, 1.9x / 1.6x / 1.5x at 256,
 // +45% / +21% / +15% at 400, +37% / +17% / +9% at 512; beyond that the second round of workgroups costs more than
 // the idle compute units did (-9% for row/col at 576).
+// (the bound as a switch, for measurement: with 8 instead of 2, 4096 x 7168 x 2048 and 4096^3 take 12-30% longer in every scale mode)
+#ifndef A8W8_SMALL_TILES_PER_CU
+#define A8W8_SMALL_TILES_PER_CU 2
+#endif
 bool small_ok(const a8w8_gemm_args* g)
 {
     const bool mxt = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;
     // tiled MX scales with an odd number of K steps have no 256-tile kernel: any size runs here
     if (mxt && (g->k / BK) % 2 != 0) return true;
     const long long items128 = (long long)g->batch * ((g->m + SM_BM - 1) / SM_BM) * ((g->n + SM_BN - 1) / SM_BN);
-    return items128 <= 2ll * num_cus();
+    return items128 <= (long long)A8W8_SMALL_TILES_PER_CU * num_cus();
 }
 
 // 128 x 64 tiles instead of 128 x 128: when the wide tiles would occupy at most half of the compute units and the K
