@@ -7,7 +7,8 @@
 * Routing corners: row strides of 2^23 bytes and more, a single K step over many tiles, one weight matrix shared
   by a batch, explicit device set-up.
 * The whole-tile C stores (buffer stores through a per-tile descriptor) of both pipelined kernels, bit for bit, in
-  both output types, into a C whose rows are padded.
+  both output types, into a C whose rows are padded; the same for the 128-tile kernel, whose whole tiles leave
+  through LDS.
 """
 import ctypes
 
@@ -243,3 +244,27 @@ def test_c_rows_millions_of_elements_apart(orc, k, c_dtype):
     assert torch.equal(c.float(), want.to(torch_dtype).float())
     del store
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("shape", [(256, 384, 256), (384, 256, 2304), (256, 192, 384)], ids=["wide_tiles", "narrow_tiles", "ragged_last_column"])
+@pytest.mark.parametrize("c_dtype", [g.BF16, g.FP32])
+def test_small_kernel_whole_tile_stores_bit_for_bit(orc, shape, c_dtype):
+    """The 128-tile kernel sends tiles that lie inside the matrix through LDS and stores them along the rows.  Exact
+    integers with power-of-two row/col scales: any value that lands in the wrong row or column shows.  C has padded
+    rows, which must keep their padding; the third shape ends with a tile column that is not whole (stored from the
+    registers, element by element where it crosses the edge); the second takes 128 x 64 tiles."""
+    m, n, k = shape
+    ldc = n + 40
+    a, b = datagen.small_ints(m, n, k, seed=7400 + n, lo=-2, hi=2)
+    rng = np.random.Generator(np.random.Philox(7401))
+    sa = np.exp2(rng.integers(-2, 3, m)).astype(np.float32)
+    sb = np.exp2(rng.integers(-2, 3, n)).astype(np.float32)
+    want = (torch.from_numpy(orc.decode(a)).cuda() @ torch.from_numpy(orc.decode(b)).cuda().T) * dev(sa)[:, None] * dev(sb)[None, :]
+    torch_dtype = torch.bfloat16 if c_dtype == g.BF16 else torch.float32
+    store = torch.full((m, ldc), -7.0, dtype=torch_dtype, device="cuda")
+    c = store[:, :n]
+    g.gemm(dev(a), dev(b), dev(sa), dev(sb), g.ROWCOL, c=c, c_dtype=c_dtype)
+    args = g.raw_gemm_args(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, m, n, k, g.ROWCOL, c_dtype=c_dtype, stride_c=ldc)
+    assert g.kernel_name(args) == "gemm_a8w8_tile128"
+    assert torch.equal(c.float(), want.to(torch_dtype).float())
+    assert bool((store[:, n:] == -7.0).all())
