@@ -466,7 +466,7 @@ int launch_flat(const GemmParams& p, int batch, hipStream_t stream)
 //   8192 x 8192    13 / 14 / 16 / 18 / 20 / 21 / 26  against  26 / 26 / 26 / 27 / 28 / 29 / 31
 //   28672 x 4096   20 / 23 / 25 / 28 / 39 / 41 / 47  against  26 / 26 / 27 / 28 / 29 / 30 / 31
 //   4096 x 14336   13 / 19 / 23 / 26 / 31 / 32 / 38  against  41 throughout
-// (tests/test_gpu_routing.py times both sides of such cells through a8w8_route_override and checks the choice).
+// (tests/test_zz_gpu_routing.py times both sides of such cells through a8w8_route_override and checks the choice).
 // Row-major weights (a8w8_gemm without b_preshuffled; the flat kernel stages the weight rows through LDS, whole lines
 // per load): as fast as shuffled ones unless the rows are a large power of two apart, where the 16 rows of a tile fall
 // on the same memory channels -- 16384 x 7168 FP8 M = 16 / 32 / 64: 20 / 21 / 25 us, 8192 x 8192: 17 / 17 / 20 us
