@@ -66,7 +66,13 @@ WORKLOADS = {
     # short and wide (a prefill chunk of 256 tokens over a 64 MiB weight): between the flat GEMM's M <= 128 and the
     # 256-row tiles; A 2 MiB + B 64 MiB + C 4 MiB + scales
     "gemm_rowcol_256x8192x8192": ("rowcol", 256, 8192, 8192, 73434112),
+    # the two pipelined kernels on one scale mode: 64 K steps run on the four-wave kernel, 65 (an odd count) on the
+    # eight-wave kernel with two waves per SIMD; compared per K step
+    "tensor_8192": ("tensor", 8192, 8192, 8192, 268435464),
+    "tensor_8192x8192x8320": ("tensor", 8192, 8192, 8320, 270532616),
 }
+# selectable with --workload, not part of the default run's secondary workloads
+SELECT_ONLY = {"tensor_8192", "tensor_8192x8192x8320"}
 # workloads whose weights would stay in the 256 MB Infinity Cache between launches: timed over rotating copies of B
 ROTATE_B = {"gemm_rowcol_256x8192x8192": 5}
 
@@ -549,7 +555,7 @@ def main():
     if not args.no_extra:
         others = []
         for name in WORKLOADS:
-            if name == args.workload:
+            if name == args.workload or name in SELECT_ONLY:
                 continue
             r, i2, c2 = run_workload(name, torch, g, args.steps, args.warmup, args.seed + 1, headline=False)
             r["timing"] = "best of 3 regions of K launches after 100 ms of warm-up"
