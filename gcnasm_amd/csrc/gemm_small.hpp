@@ -28,6 +28,9 @@ constexpr int small_scale_bytes(int mode)
 {
     return mode == MODE_MXT || mode == MODE_F4T ? 4096 : mode == MODE_F4 ? 2048 : (mode == MODE_BLOCK || mode == MODE_MX) ? 1024 : 0;
 }
+#ifndef A8W8_SMALL_PIPELINED
+#define A8W8_SMALL_PIPELINED 1          // 0: loads in a block behind the barrier, fragments read in their own step (measurement)
+#endif
 #ifndef A8W8_SMALL_LINES_BY_LANE
 #define A8W8_SMALL_LINES_BY_LANE 1      // 0: whole tiles are stored from the MFMA layout as they are (measurement)
 #endif
@@ -200,6 +203,154 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 #pragma unroll
         for (int j = 0; j < SM_TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
+    // Deep staging: the step's three instruction streams overlap inside the one wave of a SIMD.  The fragments (and
+    // scales) of step ks + 1 are read from LDS while the MFMAs of step ks run (two register sets, the loop unrolled by
+    // two), and the stage of step ks -- free as soon as everyone holds its fragments -- is refilled with step
+    // ks + SM_STAGES by loads issued one at a time between those MFMAs.  Issued in a block behind the barrier, the loads
+    // (which the compute unit's address path takes at 1 KiB per 7 ns), the LDS reads and the MFMAs follow one another:
+    // 0.46 us per K step on 128 x 64 tiles where each of the three is 0.11-0.17 us.
+    constexpr bool PIPELINED = A8W8_SMALL_PIPELINED && SM_STAGES > 2;
+    if constexpr (PIPELINED) {
+        constexpr int HALVES = (IS_F4 || MODE == MODE_BF16) ? 2 : 1;      // MFMAs per pair of fragments
+        constexpr int NFRAG = SM_TM + SM_TN, NSLOT = SM_TM * SM_TN * HALVES, NLOAD = LOADS_PER_STAGE;
+        constexpr int LOAD_EVERY = NSLOT / NLOAD, READ_EVERY = NSLOT / NFRAG;
+        constexpr int BLK_LAG = MODE == MODE_BLOCK ? 4 : 0;
+        static_assert(LOAD_EVERY >= 1 && READ_EVERY >= 1 && (SM_STAGES - 1) * NLOAD < 64, "the wait count is a 6-bit field");
+        v8i fr[2][NFRAG];       // A tiles, then B tiles
+        int sc_a[2][SM_TM], sc_b[2][SM_TN];      // the step's scales: E8M0 bytes (MX modes), or the A-side factors as float bits (block)
+        auto read_one = [&](int stage, int t) __attribute__((always_inline)) -> v8i {
+            return t < SM_TM ? read_frag(stage, rd_a, t) : read_frag(stage, rd_b, t - SM_TM);
+        };
+        auto read_scales = [&](int stage, int ks, int (&sa)[SM_TM], int (&sb)[SM_TN]) __attribute__((always_inline)) {
+            const char* sc = smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES;
+            if constexpr (MODE == MODE_BLOCK) {
+                const float* f = (const float*)sc;
+                const float b = f[128];
+#pragma unroll
+                for (int t = 0; t < SM_TM; ++t) sa[t] = __builtin_bit_cast(int, f[wave_m * 64 + 16 * t + r16] * b);
+            }
+            if constexpr (MODE == MODE_MX) {
+                // lane (r16, g) scales K [32g, 32g+32) of its row: byte g of the row's dword
+                const unsigned* w = (const unsigned*)sc;
+#pragma unroll
+                for (int t = 0; t < SM_TM; ++t) sa[t] = (int)__builtin_amdgcn_ubfe(w[wave_m * 64 + 16 * t + r16], 8 * g, 8);
+#pragma unroll
+                for (int t = 0; t < SM_TN; ++t) sb[t] = (int)__builtin_amdgcn_ubfe(w[128 + wave_n * (SM_BN / 2) + 16 * t + r16], 8 * g, 8);
+            }
+            if constexpr (MODE == MODE_F4) {
+                // lane (r16, g) scales 32-block g of each 128-element half of its row: byte g of the row's first and of
+                // its second dword, put side by side as in the tiled layout (the half is chosen by op_sel)
+                const unsigned* w = (const unsigned*)sc;
+                auto two_bytes = [&](int row) __attribute__((always_inline)) {
+                    return (int)(__builtin_amdgcn_ubfe(w[row], 8 * g, 8) | (__builtin_amdgcn_ubfe(w[256 + row], 8 * g, 8) << 8));
+                };
+#pragma unroll
+                for (int t = 0; t < SM_TM; ++t) sa[t] = two_bytes(wave_m * 64 + 16 * t + r16);
+#pragma unroll
+                for (int t = 0; t < SM_TN; ++t) sb[t] = two_bytes(128 + wave_n * (SM_BN / 2) + 16 * t + r16);
+            }
+            if constexpr (MODE == MODE_F4T) {
+                // both halves' bytes sit side by side: one 16-bit read, the half is chosen by op_sel
+#pragma unroll
+                for (int t = 0; t < SM_TM; ++t) sa[t] = *(const unsigned short*)(sc + wave_m * 1024 + mxt_off[t]);
+#pragma unroll
+                for (int t = 0; t < SM_TN; ++t) sb[t] = *(const unsigned short*)(sc + mxt_unit_b + mxt_off_b[t]);
+            }
+            if constexpr (MODE == MODE_MXT) {
+                const uint8_t* u = (const uint8_t*)sc + (ks & 1);
+#pragma unroll
+                for (int t = 0; t < SM_TM; ++t) sa[t] = u[wave_m * 1024 + mxt_off[t]];
+#pragma unroll
+                for (int t = 0; t < SM_TN; ++t) sb[t] = u[mxt_unit_b + mxt_off_b[t]];
+            }
+        };
+        // load n of a stage: four chunks of A, the chunks of B, then the step's scales
+        auto load_one = [&](int stage, int kstep, int n) __attribute__((always_inline)) {
+            A8W8_LDS char* s = (A8W8_LDS char*)smem + stage * SM_STAGE_BYTES + wave * 1024;
+            if (n < 4) load_to_lds_16(rsrc_a, s + n * 4096, voff_a[n], kstep * BK);
+            else if (n < 4 + B_LOADS) load_to_lds_16(rsrc_b, s + SM_BM * BK + (n - 4) * 4096, voff_b[n - 4], kstep << p.b_kshift);
+            else if constexpr (TILED_SCALES) {
+                A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 1024;
+                const int pair = MODE == MODE_F4T ? kstep : kstep >> 1;
+                load_to_lds_16(rsrc_sf, sc, voff_sf, ((((pair >> 1) * mxt_nblk + mxt_blk) * 2 + (pair & 1)) * 512));
+            } else if constexpr (STEP_SCALES) {
+                A8W8_LDS char* sc = (A8W8_LDS char*)smem + SM_STAGES * SM_STAGE_BYTES + stage * SM_SCALE_BYTES + wave * 256;
+                if (n == 4 + B_LOADS) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sf, sc, 4, voff_sf, kstep * sf_step_bytes, 0, 0);
+                else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sf, sc + 1024, 4, voff_sf, kstep * sf_step_bytes + 4, 0, 0);
+            }
+        };
+#pragma unroll
+        for (int st = 0; st < SM_STAGES; ++st) issue_stage(st, st);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SM_STAGES - 1) * NLOAD) : "memory");
+        A8W8_RAW_BARRIER();
+#pragma unroll
+        for (int t = 0; t < NFRAG; ++t) fr[0][t] = read_one(0, t);
+        read_scales(0, 0, sc_a[0], sc_b[0]);
+        // one K step: `have`, `sa`, `sb` hold its fragments and scales, the `next_` ones receive those of the step after it
+        auto step = [&](int ks, int stage, v8i (&have)[NFRAG], int (&sa)[SM_TM], int (&sb)[SM_TN], v8i (&next)[NFRAG],
+                        int (&next_sa)[SM_TM], int (&next_sb)[SM_TN]) __attribute__((always_inline)) {
+            const int next_stage = stage + 1 == SM_STAGES ? 0 : stage + 1;
+            // this wave's loads of the next step's stage have landed once only the SM_STAGES - 2 younger stages are in
+            // flight, and its reads of this step's fragments are complete: behind the barrier both hold for every wave
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SM_STAGES - 2) * NLOAD) : "memory");
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            A8W8_RAW_BARRIER();
+            const int kload = min(ks + SM_STAGES, nk - 1);      // past the end: the last step again, into a stage nobody reads
+            v4f part[BLK_LAG + 1];
+#pragma unroll
+            for (int t = 0; t < NSLOT + BLK_LAG; ++t) {
+                if (t < NSLOT) {
+                    // fragments pairs column by column; two-MFMA pairs: first halves of the column's four tiles, then second
+                    // halves (back-to-back MFMAs on one accumulator stall)
+                    const int i = t % SM_TM, h = (t / SM_TM) % HALVES, j = t / (SM_TM * HALVES);
+                    const v8i& fb = have[SM_TM + j];
+                    const v8i& fa = have[i];
+                    if constexpr (MODE == MODE_BLOCK) {
+                        part[t % (BLK_LAG + 1)] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                    } else if constexpr (IS_F4) {
+                        // elements [0, 128) of the step sit in the fragments' first 16 bytes, [128, 256) in the second;
+                        // op_sel picks the half's scale byte
+                        if (h == 0)
+                            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                                (v8i{fb[0], fb[1], fb[2], fb[3], 0, 0, 0, 0}), (v8i{fa[0], fa[1], fa[2], fa[3], 0, 0, 0, 0}), acc[i][j], 4, 4, 0,
+                                sb[j], 0, sa[i]);
+                        else
+                            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                                (v8i{fb[4], fb[5], fb[6], fb[7], 0, 0, 0, 0}), (v8i{fa[4], fa[5], fa[6], fa[7], 0, 0, 0, 0}), acc[i][j], 4, 4, 1,
+                                sb[j], 1, sa[i]);
+                    } else if constexpr (MODE == MODE_MX || MODE == MODE_MXT) {
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[i][j], 0, 0, 0, sb[j], 0, sa[i]);
+                    } else if constexpr (MODE == MODE_BF16) {
+                        // a 128-byte row is 64 bf16: the fragment's two 16-byte halves feed one 16x16x32 MFMA each
+                        const v4i bh = {fb[4 * h], fb[4 * h + 1], fb[4 * h + 2], fb[4 * h + 3]};
+                        const v4i ah = {fa[4 * h], fa[4 * h + 1], fa[4 * h + 2], fa[4 * h + 3]};
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, bh), __builtin_bit_cast(v8bf, ah), acc[i][j], 0, 0, 0);
+                    } else {
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[i][j], 0, 0, 0, 0, 0, 0);
+                    }
+                    if (t % LOAD_EVERY == 0 && t / LOAD_EVERY < NLOAD) load_one(stage, kload, t / LOAD_EVERY);
+                    if (t % READ_EVERY == 0 && t / READ_EVERY < NFRAG) next[t / READ_EVERY] = read_one(next_stage, t / READ_EVERY);
+                    if (t == 0) read_scales(next_stage, ks + 1, next_sa, next_sb);
+                }
+                if constexpr (MODE == MODE_BLOCK) {
+                    // acc += part * (sfa * sfb); the multiply-adds trail the MFMAs by BLK_LAG tiles so that they never
+                    // wait on a matrix-core result that is still in flight
+                    if (t >= BLK_LAG) {
+                        const int u = t - BLK_LAG;
+                        acc[u % SM_TM][u / SM_TM] += part[u % (BLK_LAG + 1)] * __builtin_bit_cast(float, sa[u % SM_TM]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            return next_stage;
+        };
+        int ks = 0, stage = 0;
+        for (; ks + 1 < nk; ks += 2) {
+            stage = step(ks, stage, fr[0], sc_a[0], sc_b[0], fr[1], sc_a[1], sc_b[1]);
+            stage = step(ks + 1, stage, fr[1], sc_a[1], sc_b[1], fr[0], sc_a[0], sc_b[0]);
+        }
+        if (ks < nk) step(ks, stage, fr[0], sc_a[0], sc_b[0], fr[1], sc_a[1], sc_b[1]);
+    } else {
     issue_stage(0, 0);
     issue_stage(1, 1);
     if constexpr (SM_STAGES > 2) {
@@ -337,6 +488,7 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
         }
         refill = cur;
         cur = cur + 1 == SM_STAGES ? 0 : cur + 1;
+    }
     }
 
     // ---- epilogue: dequantise in fp32, convert, store
