@@ -246,6 +246,9 @@ int num_cus()
 #ifndef A8W8_SMALL_TILES_PER_CU
 #define A8W8_SMALL_TILES_PER_CU 2
 #endif
+#ifndef A8W8_SMALL_DEEP_UP_TO
+#define A8W8_SMALL_DEEP_UP_TO 1         // four LDS stages up to this many 128-tiles per compute unit, two stages beyond
+#endif
 bool small_ok(const a8w8_gemm_args* g)
 {
     const bool mxt = g->scale_mode == A8W8_SCALE_MX_E8M0_TILED;
@@ -292,7 +295,7 @@ int launch_small(const GemmParams& p, int batch, hipStream_t stream)
             constexpr int ST = narrow_stages(MODE);
             return launch(gemm_a8w8_tile128<MODE, CDT, ST, 64>, grid, dim3(SM_THREADS), small_lds_bytes(MODE, ST, 64), stream, q);
         }
-        if (items <= num_cus())
+        if (items <= (long long)A8W8_SMALL_DEEP_UP_TO * num_cus())
             return launch_small_stages<MODE, CDT, 4>(q, batch, stream);
         return launch_small_stages<MODE, CDT, 2>(q, batch, stream);
     } else {
