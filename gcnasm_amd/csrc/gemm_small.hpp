@@ -31,6 +31,9 @@ constexpr int small_scale_bytes(int mode)
 #ifndef A8W8_SMALL_PIPELINED
 #define A8W8_SMALL_PIPELINED 1          // 0: loads in a block behind the barrier, fragments read in their own step (measurement)
 #endif
+#ifndef A8W8_SMALL_PIPELINED_TWO
+#define A8W8_SMALL_PIPELINED_TWO 1      // the same switch for the two-stage variant
+#endif
 #ifndef A8W8_SMALL_LINES_BY_LANE
 #define A8W8_SMALL_LINES_BY_LANE 1      // 0: whole tiles are stored from the MFMA layout as they are (measurement)
 #endif
@@ -209,15 +212,19 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
     // ks + SM_STAGES by loads issued one at a time between those MFMAs.  Issued in a block behind the barrier, the loads
     // (which the compute unit's address path takes at 1 KiB per 7 ns), the LDS reads and the MFMAs follow one another:
     // 0.46 us per K step on 128 x 64 tiles where each of the three is 0.11-0.17 us.
-    constexpr bool PIPELINED = A8W8_SMALL_PIPELINED && SM_STAGES > 2;
+    // Two stages (two workgroups per compute unit): there is no third stage to read ahead from, so a step reads all of its
+    // fragments first, and behind a second barrier -- the stage is then free -- runs its MFMAs with the refill loads (step
+    // ks + 2) between them; the other workgroup's MFMAs run beside this one's LDS reads.
+    constexpr bool TWO = SM_STAGES == 2;
+    constexpr bool PIPELINED = TWO ? A8W8_SMALL_PIPELINED_TWO != 0 : A8W8_SMALL_PIPELINED != 0;
     if constexpr (PIPELINED) {
         constexpr int HALVES = (IS_F4 || MODE == MODE_BF16) ? 2 : 1;      // MFMAs per pair of fragments
         constexpr int NFRAG = SM_TM + SM_TN, NSLOT = SM_TM * SM_TN * HALVES, NLOAD = LOADS_PER_STAGE;
         constexpr int LOAD_EVERY = NSLOT / NLOAD, READ_EVERY = NSLOT / NFRAG;
         constexpr int BLK_LAG = MODE == MODE_BLOCK ? 4 : 0;
         static_assert(LOAD_EVERY >= 1 && READ_EVERY >= 1 && (SM_STAGES - 1) * NLOAD < 64, "the wait count is a 6-bit field");
-        v8i fr[2][NFRAG];       // A tiles, then B tiles
-        int sc_a[2][SM_TM], sc_b[2][SM_TN];      // the step's scales: E8M0 bytes (MX modes), or the A-side factors as float bits (block)
+        v8i fr[TWO ? 1 : 2][NFRAG];       // A tiles, then B tiles
+        int sc_a[TWO ? 1 : 2][SM_TM], sc_b[TWO ? 1 : 2][SM_TN];      // the step's scales: E8M0 bytes (MX modes), or the A-side factors as float bits (block)
         auto read_one = [&](int stage, int t) __attribute__((always_inline)) -> v8i {
             return t < SM_TM ? read_frag(stage, rd_a, t) : read_frag(stage, rd_b, t - SM_TM);
         };
@@ -281,18 +288,29 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
         };
 #pragma unroll
         for (int st = 0; st < SM_STAGES; ++st) issue_stage(st, st);
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SM_STAGES - 1) * NLOAD) : "memory");
-        A8W8_RAW_BARRIER();
+        if constexpr (!TWO) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SM_STAGES - 1) * NLOAD) : "memory");
+            A8W8_RAW_BARRIER();
 #pragma unroll
-        for (int t = 0; t < NFRAG; ++t) fr[0][t] = read_one(0, t);
-        read_scales(0, 0, sc_a[0], sc_b[0]);
+            for (int t = 0; t < NFRAG; ++t) fr[0][t] = read_one(0, t);
+            read_scales(0, 0, sc_a[0], sc_b[0]);
+        }
         // one K step: `have`, `sa`, `sb` hold its fragments and scales, the `next_` ones receive those of the step after it
         auto step = [&](int ks, int stage, v8i (&have)[NFRAG], int (&sa)[SM_TM], int (&sb)[SM_TN], v8i (&next)[NFRAG],
                         int (&next_sa)[SM_TM], int (&next_sb)[SM_TN]) __attribute__((always_inline)) {
             const int next_stage = stage + 1 == SM_STAGES ? 0 : stage + 1;
+            if constexpr (TWO) {
+                // this wave's loads of the step's stage have landed once only the other stage's are in flight; behind the
+                // barrier everyone's have
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLOAD) : "memory");
+                A8W8_RAW_BARRIER();
+#pragma unroll
+                for (int t = 0; t < NFRAG; ++t) have[t] = read_one(stage, t);
+                read_scales(stage, ks, sa, sb);
+            }
             // this wave's loads of the next step's stage have landed once only the SM_STAGES - 2 younger stages are in
             // flight, and its reads of this step's fragments are complete: behind the barrier both hold for every wave
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SM_STAGES - 2) * NLOAD) : "memory");
+            if constexpr (!TWO) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SM_STAGES - 2) * NLOAD) : "memory");
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             A8W8_RAW_BARRIER();
             const int kload = min(ks + SM_STAGES, nk - 1);      // past the end: the last step again, into a stage nobody reads
@@ -329,8 +347,10 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
                         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc[i][j], 0, 0, 0, 0, 0, 0);
                     }
                     if (t % LOAD_EVERY == 0 && t / LOAD_EVERY < NLOAD) load_one(stage, kload, t / LOAD_EVERY);
-                    if (t % READ_EVERY == 0 && t / READ_EVERY < NFRAG) next[t / READ_EVERY] = read_one(next_stage, t / READ_EVERY);
-                    if (t == 0) read_scales(next_stage, ks + 1, next_sa, next_sb);
+                    if constexpr (!TWO) {
+                        if (t % READ_EVERY == 0 && t / READ_EVERY < NFRAG) next[t / READ_EVERY] = read_one(next_stage, t / READ_EVERY);
+                        if (t == 0) read_scales(next_stage, ks + 1, next_sa, next_sb);
+                    }
                 }
                 if constexpr (MODE == MODE_BLOCK) {
                     // acc += part * (sfa * sfb); the multiply-adds trail the MFMAs by BLK_LAG tiles so that they never
@@ -345,11 +365,15 @@ __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
             return next_stage;
         };
         int ks = 0, stage = 0;
-        for (; ks + 1 < nk; ks += 2) {
-            stage = step(ks, stage, fr[0], sc_a[0], sc_b[0], fr[1], sc_a[1], sc_b[1]);
-            stage = step(ks + 1, stage, fr[1], sc_a[1], sc_b[1], fr[0], sc_a[0], sc_b[0]);
+        if constexpr (TWO) {
+            for (; ks < nk; ++ks) stage = step(ks, stage, fr[0], sc_a[0], sc_b[0], fr[0], sc_a[0], sc_b[0]);
+        } else {
+            for (; ks + 1 < nk; ks += 2) {
+                stage = step(ks, stage, fr[0], sc_a[0], sc_b[0], fr[1], sc_a[1], sc_b[1]);
+                stage = step(ks + 1, stage, fr[1], sc_a[1], sc_b[1], fr[0], sc_a[0], sc_b[0]);
+            }
+            if (ks < nk) step(ks, stage, fr[0], sc_a[0], sc_b[0], fr[1], sc_a[1], sc_b[1]);
         }
-        if (ks < nk) step(ks, stage, fr[0], sc_a[0], sc_b[0], fr[1], sc_a[1], sc_b[1]);
     } else {
     issue_stage(0, 0);
     issue_stage(1, 1);
