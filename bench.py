@@ -362,6 +362,7 @@ REFERENCE_PUBLISHED = {"block_fp32_1024": 118.96, "block_fp32_2048": 616.77, "bl
 def run_reference_program_sizes(torch, g, steps, warmup, seed):
     """The reference's own programs at the sizes it publishes numbers for, with its inputs and its metric
     (2*M*N*K / average launch time): the ratio to the published TFlops is reported beside each."""
+    import ctypes
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
 
@@ -378,7 +379,12 @@ def run_reference_program_sizes(torch, g, steps, warmup, seed):
         sfa, sfb = uniform((k // 128, m), 0.8, 1.2), uniform((n // 128, k // 128), 0.8, 1.2)
         c = torch.empty((m, n), dtype=torch.float32, device="cuda")
         big_steps = steps if size < 16384 else max(5, steps // 5)      # 3.5 ms a launch: fewer of them
-        ms, wall = time_best_of(torch, lambda i: g.gemm_blockscale(a, b, sfa, sfb, c=c), big_steps, min(warmup, big_steps))
+        # the argument block is filled once, as the reference's C++ program does: a launch through the tensor wrapper costs
+        # the host 10 us, which is as long as the 1024-cube kernel runs
+        args = g.raw_gemm_args(a.data_ptr(), b.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, g.BLOCK, c_dtype=g.FP32)
+        ref, lib, stream = ctypes.byref(args), g.lib(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        assert lib.a8w8_gemm_blockscale(ref, stream) == 0
+        ms, wall = time_best_of(torch, lambda i: lib.a8w8_gemm_blockscale(ref, stream), big_steps, min(warmup, big_steps))
         name = f"block_fp32_{size}"
         tf = 2.0 * m * n * k / ms / 1e9
         out.append({"workload": name, "m": m, "n": n, "k": k, "kernel": g.kernel_name(g.raw_gemm_args(
@@ -392,13 +398,17 @@ def run_reference_program_sizes(torch, g, steps, warmup, seed):
     b, sfb = g.quantize(torch.randn((n, k), generator=gen, device="cuda"), g.ROWCOL)
     bs = g.preshuffle_b_device(b)
     c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
-    ms, wall = time_best_of(torch, lambda i: g.flatmm(a, bs, sfa, sfb, n, c=c), steps, warmup)
+    args = g.raw_gemm_args(a.data_ptr(), bs.data_ptr(), c.data_ptr(), sfa.data_ptr(), sfb.data_ptr(), m, n, k, g.ROWCOL, c_dtype=g.BF16,
+                           b_preshuffled=1)
+    ref, lib, stream = ctypes.byref(args), g.lib(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert lib.a8w8_flatmm(ref, stream) == 0
+    ms, wall = time_best_of(torch, lambda i: lib.a8w8_flatmm(ref, stream), steps, warmup)
     tf = 2.0 * m * n * k / ms / 1e9
     out.append({"workload": "flatmm_16x4096x4096", "m": m, "n": n, "k": k, "kernel": "flatmm_a8w8", "ms_per_launch": ms,
                 "wall_ms_per_launch": wall, "tflops": tf, "reference_published_tflops": REFERENCE_PUBLISHED["flatmm_16x4096x4096"],
                 "vs_reference_published": tf / REFERENCE_PUBLISHED["flatmm_16x4096x4096"],
-                "note": "a launch from Python through ctypes costs about 9 us, which bounds this entry; the C++ program "
-                        "tests/harness/flatmm_a8w8.exe -m 16 -n 4096 -k 4096 measures the kernel's own rate"})
+                "note": "a launch from Python through ctypes still costs the host several us, which bounds this entry; the C++ "
+                        "program tests/harness/flatmm_a8w8.exe -m 16 -n 4096 -k 4096 measures the kernel's own rate"})
     return out
 
 
