@@ -75,6 +75,20 @@ def test_short_wide_problems_on_narrow_tiles(m, n, k, batch, mode, shuffled):
         _exact_case(r, "narrow tiles", mode, batch, m, n, k, c_dtype, shuffled)
 
 
+@pytest.mark.parametrize("mode", [g.TENSOR, g.ROWCOL, g.BLOCK, g.MX, g.MX_TILED])
+@pytest.mark.parametrize("ksteps", [1, 2, 3, 4, 5, 7, 8, 9])
+@pytest.mark.parametrize("m,n", [(384, 256), (2176, 2048)], ids=["four_stages", "two_stages"])
+def test_overlapped_steps_of_the_128_tile_kernel(m, n, ksteps, mode):
+    """The 128-tile kernel reads a step's fragments one step ahead (four stages: up to one tile per compute unit) or in
+    front of a second barrier (two stages: up to two), and refills the stage between the MFMAs: every step count from
+    one to past twice the stage count, odd and even (the four-stage loop is unrolled by two), exact in every scale mode."""
+    k = 128 * ksteps
+    r = np.random.default_rng(4200 + m + 13 * ksteps + 7 * mode)
+    args = g.raw_gemm_args(1 << 12, 1 << 12, 1 << 12, 1 << 12, 1 << 12, m, n, k, mode)
+    assert g.kernel_name(args) == "gemm_a8w8_tile128"
+    _exact_case(r, f"{ksteps} K steps", mode, 1, m, n, k, g.FP32 if ksteps % 2 else g.BF16, False)
+
+
 def _exact_case(r, label, mode, batch, m, n, k, c_dtype, shuffled):
     a = r.integers(-4, 5, (batch, m, k)).astype(np.float32)
     b = r.integers(-4, 5, (batch, n, k)).astype(np.float32)
