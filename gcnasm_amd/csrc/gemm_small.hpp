@@ -51,9 +51,10 @@ constexpr int small_lds_bytes(int mode, int stages, int bn = SM_BN)
 // SM_STAGES = 2: loads issued when a stage has been read, two barriers per step, two workgroups per compute unit
 // that hide each other's waits -- for larger grids.
 // BN_ = 64: tiles of 128 x 64 (a wave owns 64 x 32) for short, wide problems -- M of a few hundred rows over weights
-// of many megabytes -- where 128 x 128 tiles would leave half of the compute units without a workgroup.  Such a
-// problem is bound by how many bytes of the weights each compute unit keeps in flight, hence SM_STAGES = 6 there
-// (five K steps of loads ahead, 144-154 KiB of LDS; 5 with tiled MX scales, whose 4 KiB per stage would not fit six).
+// of many megabytes -- where 128 x 128 tiles would leave half of the compute units without a workgroup.  A workgroup
+// alone on its compute unit streams its share of the weights through a long K loop: SM_STAGES = 6 there (five K
+// steps of loads ahead, 144-154 KiB of LDS; 5 with tiled MX scales, whose 4 KiB per stage would not fit six; measured,
+// five and six stages run alike, and so does a separate ring of ten stages for the weights).
 template <int MODE, int CDT, int SM_STAGES, int BN_ = SM_BN>
 __global__ void __launch_bounds__(SM_THREADS, 2) gemm_a8w8_tile128(GemmParams p)
 {
