@@ -70,9 +70,12 @@ WORKLOADS = {
     # eight-wave kernel with two waves per SIMD; compared per K step
     "tensor_8192": ("tensor", 8192, 8192, 8192, 268435464),
     "tensor_8192x8192x8320": ("tensor", 8192, 8192, 8320, 270532616),
+    # the 128-tile kernel's variants: one tile per compute unit (four LDS stages), two per compute unit (two stages)
+    "rowcol_2048": ("rowcol", 2048, 2048, 2048, 16793600),
+    "rowcol_2048x4096x2048": ("rowcol", 2048, 4096, 2048, 29384704),
 }
 # selectable with --workload, not part of the default run's secondary workloads
-SELECT_ONLY = {"tensor_8192", "tensor_8192x8192x8320"}
+SELECT_ONLY = {"tensor_8192", "tensor_8192x8192x8320", "rowcol_2048", "rowcol_2048x4096x2048"}
 # workloads whose weights would stay in the 256 MB Infinity Cache between launches: timed over rotating copies of B
 ROTATE_B = {"gemm_rowcol_256x8192x8192": 5}
 
